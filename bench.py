@@ -1,0 +1,157 @@
+#!/usr/bin/env python3
+"""ROIAlign forward+backward throughput on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2] [--impl auto]
+
+One step = one forward pass plus one backward pass (gradient overwritten) of the
+operator over one batch of synthetic, seeded input that is already resident in
+HBM, issued through the launcher library's C ABI on one HIP stream.  Prints ONE
+JSON line: whole-job ROIs/s, the roofline figures of the dominant pass measured
+with HIP events around each pass, and the CPU baseline (the reference's own
+kernels compiled for the host where that build is present, else the CPU
+restatement), timed on this machine's cores on a bounded sample.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, 'tests'))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def cpu_baseline(w, budget_s=25.0):
+    """Reference kernels on the host cores: forward+backward ROIs/s on a
+    bounded sample (the first ROIs of the same workload, full channel count)."""
+    import numpy as np
+    from oracle import roialign as oracle
+    kind = 'reference' if oracle.ref_available('omp') else 'port'
+    impl = 'ref_omp' if kind == 'reference' else 'oracle'
+    x = w['data'].astype(np.float32)
+    pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
+    R = w['rois'].shape[0]
+    n = min(R, 64)
+    best = None
+    spent = 0.0
+    while True:
+        rois = w['rois'][:n]
+        dy = w['dy'][:n] if w['dy'] is not None else None
+        t0 = time.perf_counter()
+        oracle.forward(x, rois, pooled, scale, S, impl=impl)
+        if dy is not None:
+            oracle.backward(dy, rois, x.shape, scale, S, impl=impl)
+        dt = time.perf_counter() - t0
+        spent += dt
+        best = (n, dt)
+        # grow the sample until one pass costs a few seconds or covers everything
+        if n >= R or dt > budget_s / 4 or spent > budget_s:
+            break
+        n = min(R, n * 4)
+    n, dt = best
+    return {'value': n / dt, 'unit': 'ROIs/s', 'cores': oracle.num_threads(), 'kind': kind,
+            'sample': 'first {} of {} ROIs of {} ({}), one pass, {:.2f} s'.format(
+                n, R, w['name'], 'fwd+bwd' if w['dy'] is not None else 'fwd only', dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=30)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--workload', default='cfg2', choices=['cfg1', 'cfg2', 'cfg3', 'cfg4'])
+    ap.add_argument('--impl', default='auto', choices=['auto', 'tiled', 'naive'])
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py: this build measures one GPU only (the path shards by image with no '
+                 'exchange; see DESIGN.md); run with --gpus 1')
+
+    import torch
+    from mobulaop_amd import workloads
+    import abi_util as abi
+    assert torch.cuda.is_available(), 'bench.py needs a GPU'
+
+    w = workloads.make_workload(args.workload)
+    pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
+    x = abi.to_dev(w['data'])
+    rois = abi.to_dev(w['rois'])
+    has_bwd = w['dy'] is not None
+    dy = abi.to_dev(w['dy']) if has_bwd else None
+    R = rois.shape[0]
+    abi.set_impl(args.impl)
+    stream = torch.cuda.current_stream().cuda_stream  # launches and events share this stream
+
+    dx = torch.empty_like(x) if has_bwd else None
+
+    def step(events=None):
+        if events is not None:
+            events[0].record()
+        y = abi.forward(x, rois, pooled, scale, S, stream=stream)
+        if events is not None:
+            events[1].record()
+        if has_bwd:
+            abi.backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream)
+        if events is not None:
+            events[2].record()
+        return y
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(evs[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps if has_bwd else 0.0
+    ms_per_step = wall * 1e3 / args.steps
+    b_fwd, b_bwd = workloads.algorithmic_bytes(w)
+
+    def gbs(nbytes, ms):
+        return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+
+    dominant = 'backward' if bwd_ms > fwd_ms else 'forward'
+    dom_bytes, dom_ms = (b_bwd, bwd_ms) if dominant == 'backward' else (b_fwd, fwd_ms)
+    passes = {'forward': {'ms': fwd_ms, 'GB/s': gbs(b_fwd, fwd_ms), 'frac': gbs(b_fwd, fwd_ms) / HBM_PEAK_GBS,
+                          'rois_per_s': R / (fwd_ms * 1e-3)}}
+    total_bytes = b_fwd
+    if has_bwd:
+        passes['backward'] = {'ms': bwd_ms, 'GB/s': gbs(b_bwd, bwd_ms),
+                              'frac': gbs(b_bwd, bwd_ms) / HBM_PEAK_GBS}
+        total_bytes += b_bwd
+    gpu_ms = fwd_ms + bwd_ms
+    passes['fwd_bwd' if has_bwd else 'fwd'] = {
+        'ms': gpu_ms, 'GB/s': gbs(total_bytes, gpu_ms), 'frac': gbs(total_bytes, gpu_ms) / HBM_PEAK_GBS}
+
+    out = {
+        'metric': 'roialign_fwd_bwd_rois_per_sec' if has_bwd else 'roialign_fwd_rois_per_sec',
+        'value': R / (ms_per_step * 1e-3), 'unit': 'ROIs/s', 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': ms_per_step, 'higher_is_better': True,
+        'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'f16 storage, f32 accumulate' if w['data'].dtype.itemsize == 2 else 'f32',
+        'data': 'synthetic',
+        'config': {'workload': '{}: data {} rois {} pooled {} scale {} sampling_ratio {}'.format(
+            w['name'], 'x'.join(map(str, w['data'].shape)), R, 'x'.join(map(str, pooled)), scale, S),
+            'impl': args.impl, 'step': 'forward + backward(assign)' if has_bwd else 'forward'},
+        'roofline': {'bound': 'hbm', 'kernel': dominant + ' pass', 'achieved': gbs(dom_bytes, dom_ms),
+                     'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': gbs(dom_bytes, dom_ms) / HBM_PEAK_GBS,
+                     'traffic': None, 'algorithmic_bytes': dom_bytes, 'avg_ms': dom_ms},
+        'passes': passes,
+    }
+    if not args.no_cpu_baseline:
+        out['cpu_baseline'] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

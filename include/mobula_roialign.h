@@ -1,0 +1,108 @@
+/*
+ * C ABI of the MI355X (gfx950) ROIAlign launcher library, libmobula_hip.so.
+ *
+ * The first two functions are, name for name and argument for argument, what
+ * the reference's Python binding resolves with ctypes for the float
+ * instantiation of its ROIAlign kernels:
+ *   - symbol name  <func>_<md5(argument C type list)[:8]>   mobula/func.py:13-50
+ *   - signature    (device_id, kernel arguments...)          mobula/op/templates/kernel_code.cpp:1-5
+ *   - kernel arguments                                       opzoo/ROIAlign/ROIAlign.cpp:10-16, 79-83
+ *   - call site    func(dev_id, *raw_pointers)               mobula/func.py:155-156
+ *
+ * Conventions (all entry points):
+ *   device_id >= 0  every pointer is device memory of that GPU; the launch
+ *                   goes to the stream set with mobula_hip_set_stream() on the
+ *                   calling thread (default: the null stream, and the call
+ *                   returns only when the result is complete, like the
+ *                   reference, context/hip_ctx.h:62-93).
+ *   device_id == -1 every pointer is host memory; the library stages the
+ *                   buffers through GPU memory and returns when the result is
+ *                   in the host buffers.  There is no CPU implementation.
+ *   Tensors are dense: data/bottom_diff NCHW [N,C,H,W], rois [R,5] rows
+ *   [batch_idx, x1, y1, x2, y2], top [R,C,PH,PW]; R = nthreads/(C*PH*PW).
+ *   N is not an argument of the reference ABI: it is taken from the element
+ *   count declared with mobula_hip_set_arg_extents(), else read back from the
+ *   largest batch index (one blocking copy).
+ *   No return codes: a failed call leaves a message for
+ *   mobula_hip_last_error() and does not terminate the process (the reference
+ *   prints and calls exit(-1), mobula/cpp/include/logging.h:23-26).
+ */
+#ifndef MOBULA_ROIALIGN_H_
+#define MOBULA_ROIALIGN_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* top_data[r,c,ph,pw] = mean over the sampling grid of bilinear samples.
+ * Replaces: roi_align_forward_kernel<float>, opzoo/ROIAlign/ROIAlign.cpp:9-76. */
+void roi_align_forward_ab78de3c(const int device_id, const int nthreads,
+                                const float* bottom_data, const float spatial_scale,
+                                const int channels, const int height, const int width,
+                                const int pooled_height, const int pooled_width,
+                                const int sampling_ratio, const float* bottom_rois,
+                                float* top_data);
+
+/* bottom_diff += scatter of top_diff (accumulates; the caller zeroes).
+ * Replaces: roi_align_backward_kernel<float>, opzoo/ROIAlign/ROIAlign.cpp:78-161.
+ * Note the argument order: bottom_diff before bottom_rois. */
+void roi_align_backward_f318a24e(const int device_id, const int nthreads, const float* top_diff,
+                                 const float spatial_scale, const int channels, const int height,
+                                 const int width, const int pooled_height, const int pooled_width,
+                                 const int sampling_ratio, float* bottom_diff,
+                                 const float* bottom_rois);
+
+/* Makes device_id the current device.
+ * Replaces: set_device, mobula/cpp/include/context/context.h:15-17. */
+void set_device(const int device_id);
+
+/* ---- Extensions: no counterpart in the reference ------------------------ */
+
+/* bottom_diff = scatter of top_diff: overwrites all N*C*H*W elements (zero
+ * where no ROI contributes).  Fuses the operator's zero-fill
+ * (opzoo/ROIAlign/ROIAlign.py:33-34) with the scatter. */
+void roi_align_backward_assign_a8793cbe(const int device_id, const int nthreads,
+                                        const float* top_diff, const float spatial_scale,
+                                        const int channels, const int height, const int width,
+                                        const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        float* bottom_diff, const float* bottom_rois);
+
+/* Forward with IEEE binary16 storage of bottom_data / top_data (passed as
+ * 16-bit patterns), fp32 rois and fp32 accumulation. */
+void roi_align_forward_e874c59a(const int device_id, const int nthreads,
+                                const unsigned short* bottom_data, const float spatial_scale,
+                                const int channels, const int height, const int width,
+                                const int pooled_height, const int pooled_width,
+                                const int sampling_ratio, const float* bottom_rois,
+                                unsigned short* top_data);
+
+/* Per-thread launch stream (a hipStream_t) for subsequent calls; synchronous
+ * != 0 makes each call wait for its result before returning. */
+void mobula_hip_set_stream(void* stream, int synchronous);
+
+/* Element counts of the NEXT call's arguments, in argument order without the
+ * device id, -1 for scalars.  Used to derive N and to reject calls whose
+ * buffers cannot hold the problem the scalars describe. */
+void mobula_hip_set_arg_extents(const long long* numel, int n);
+
+/* Message of the calling thread's last failed call, or NULL; cleared by
+ * mobula_hip_clear_error(). */
+const char* mobula_hip_last_error(void);
+void mobula_hip_clear_error(void);
+
+/* Named integer switches ("roialign_impl": 0 auto, 1 tiled, 2 naive;
+ * "host_staging_device").  set returns 0, or -1 for an unknown name; get
+ * returns -1 for a name never set. */
+int mobula_hip_set_option(const char* name, long long value);
+long long mobula_hip_get_option(const char* name);
+
+int mobula_hip_device_count(void);
+
+/* Space-separated list of the operator entry points in this build. */
+const char* mobula_hip_exports(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOBULA_ROIALIGN_H_ */

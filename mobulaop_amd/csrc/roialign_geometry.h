@@ -1,0 +1,80 @@
+// ROI and sample geometry, evaluated in fp32 in exactly the operation order of
+// the reference (opzoo/ROIAlign/ROIAlign.cpp:24-65, opzoo/ROIAlign/bilinear.h:
+// 15-48).  The validity cut-offs are discontinuous (a sample at y == height
+// counts, one a single ulp above does not), so these expressions must not be
+// re-associated or fused: the translation unit is compiled with
+// -ffp-contract=off and IEEE division.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+namespace roialign {
+
+struct RoiGeom {
+  int batch;
+  float start_w, start_h;
+  float bin_w, bin_h;
+  int grid_h, grid_w;
+  float count;
+};
+
+__device__ __forceinline__ RoiGeom roi_geometry(const float* __restrict__ roi, float scale,
+                                                int pooled_h, int pooled_w, int sampling_ratio) {
+  RoiGeom g;
+  g.batch = static_cast<int>(roi[0]);  // truncation toward zero
+  g.start_w = roi[1] * scale;
+  g.start_h = roi[2] * scale;
+  const float end_w = roi[3] * scale;
+  const float end_h = roi[4] * scale;
+  const float roi_w = fmaxf(end_w - g.start_w, 1.0f);  // malformed boxes become 1x1
+  const float roi_h = fmaxf(end_h - g.start_h, 1.0f);
+  g.bin_h = roi_h / static_cast<float>(pooled_h);
+  g.bin_w = roi_w / static_cast<float>(pooled_w);
+  g.grid_h = sampling_ratio > 0 ? sampling_ratio
+                                : static_cast<int>(ceilf(roi_h / static_cast<float>(pooled_h)));
+  g.grid_w = sampling_ratio > 0 ? sampling_ratio
+                                : static_cast<int>(ceilf(roi_w / static_cast<float>(pooled_w)));
+  g.count = static_cast<float>(g.grid_h * g.grid_w);
+  return g;
+}
+
+// start + p*bin + ((i + .5)*bin)/grid, left to right.
+__device__ __forceinline__ float sample_coord(float start, int p, float bin, int i, int grid) {
+  const float a = static_cast<float>(p) * bin;
+  float b = (static_cast<float>(i) + 0.5f) * bin;
+  b = b / static_cast<float>(grid);
+  return (start + a) + b;
+}
+
+struct AxisSample {
+  int low, high;  // the two neighbouring rows (or columns)
+  float l, h;     // weight of `high` and of `low`
+  bool valid;     // false: the whole sample contributes nothing
+};
+
+__device__ __forceinline__ AxisSample axis_sample(float v, int size) {
+  AxisSample s;
+  s.valid = !(v < -1.0f || v > static_cast<float>(size));
+  if (v <= 0.0f) v = 0.0f;
+  int lo = static_cast<int>(v);
+  if (lo >= size - 1) {
+    lo = size - 1;
+    s.high = lo;
+    v = static_cast<float>(lo);
+  } else {
+    s.high = lo + 1;
+  }
+  s.low = lo;
+  s.l = v - static_cast<float>(lo);
+  s.h = 1.0f - s.l;
+  if (!s.valid) { s.low = s.high = 0; s.l = s.h = 0.0f; }
+  return s;
+}
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(__half v) { return __half2float(v); }
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ __half from_float<__half>(float v) { return __float2half_rn(v); }
+
+}  // namespace roialign

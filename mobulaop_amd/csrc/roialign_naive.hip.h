@@ -1,0 +1,91 @@
+// Straightforward ROIAlign kernels: one thread per output element, every
+// expression in the reference's order (opzoo/ROIAlign/ROIAlign.cpp:17-75,
+// 84-160).  They are the library's correctness anchor on the GPU (bit-close to
+// the reference arithmetic, including the order of the four-term weighted sum)
+// and the fallback for shapes the tiled kernels do not take.
+#pragma once
+#include "roialign_geometry.h"
+
+namespace roialign {
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+forward_naive_kernel(long long n_out, const T* __restrict__ x, float scale, int C, int H, int W,
+                     int PH, int PW, int S, const float* __restrict__ rois, T* __restrict__ y,
+                     long long num_images) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  const int bins = PH * PW;
+  for (long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; idx < n_out;
+       idx += stride) {
+    const int pw = static_cast<int>(idx % PW);
+    const int ph = static_cast<int>((idx / PW) % PH);
+    const int c = static_cast<int>((idx / bins) % C);
+    const long long r = idx / (static_cast<long long>(bins) * C);
+    const RoiGeom g = roi_geometry(rois + r * 5, scale, PH, PW, S);
+    float acc = 0.0f;
+    if (g.batch >= 0 && g.batch < num_images) {
+      const T* plane = x + (static_cast<long long>(g.batch) * C + c) * H * W;
+      for (int iy = 0; iy < g.grid_h; ++iy) {
+        const AxisSample sy = axis_sample(sample_coord(g.start_h, ph, g.bin_h, iy, g.grid_h), H);
+        for (int ix = 0; ix < g.grid_w; ++ix) {
+          const AxisSample sx = axis_sample(sample_coord(g.start_w, pw, g.bin_w, ix, g.grid_w), W);
+          float val = 0.0f;
+          if (sy.valid && sx.valid) {
+            const float v1 = to_float(plane[sy.low * W + sx.low]);
+            const float v2 = to_float(plane[sy.low * W + sx.high]);
+            const float v3 = to_float(plane[sy.high * W + sx.low]);
+            const float v4 = to_float(plane[sy.high * W + sx.high]);
+            const float w1 = sy.h * sx.h, w2 = sy.h * sx.l, w3 = sy.l * sx.h, w4 = sy.l * sx.l;
+            val = w1 * v1 + w2 * v2 + w3 * v3 + w4 * v4;
+          }
+          acc += val;
+        }
+      }
+    }
+    y[idx] = from_float<T>(acc / g.count);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+backward_naive_kernel(long long n_out, const float* __restrict__ dy, float scale, int C, int H,
+                      int W, int PH, int PW, int S, float* __restrict__ dx,
+                      const float* __restrict__ rois, long long num_images) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  const int bins = PH * PW;
+  for (long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; idx < n_out;
+       idx += stride) {
+    const int pw = static_cast<int>(idx % PW);
+    const int ph = static_cast<int>((idx / PW) % PH);
+    const int c = static_cast<int>((idx / bins) % C);
+    const long long r = idx / (static_cast<long long>(bins) * C);
+    const RoiGeom g = roi_geometry(rois + r * 5, scale, PH, PW, S);
+    if (g.batch < 0 || g.batch >= num_images) continue;
+    float* plane = dx + (static_cast<long long>(g.batch) * C + c) * H * W;
+    const float top = dy[idx];
+    for (int iy = 0; iy < g.grid_h; ++iy) {
+      const AxisSample sy = axis_sample(sample_coord(g.start_h, ph, g.bin_h, iy, g.grid_h), H);
+      if (!sy.valid) continue;
+      for (int ix = 0; ix < g.grid_w; ++ix) {
+        const AxisSample sx = axis_sample(sample_coord(g.start_w, pw, g.bin_w, ix, g.grid_w), W);
+        if (!sx.valid) continue;
+        const float w1 = sy.h * sx.h, w2 = sy.h * sx.l, w3 = sy.l * sx.h, w4 = sy.l * sx.l;
+        atomicAdd(plane + sy.low * W + sx.low, top * w1 / g.count);
+        atomicAdd(plane + sy.low * W + sx.high, top * w2 / g.count);
+        atomicAdd(plane + sy.high * W + sx.low, top * w3 / g.count);
+        atomicAdd(plane + sy.high * W + sx.high, top * w4 / g.count);
+      }
+    }
+  }
+}
+
+// max(batch index)+1 over all ROIs, for callers that did not say how many
+// images the feature map holds.
+__global__ void max_batch_kernel(const float* __restrict__ rois, int R, int* __restrict__ out) {
+  int m = 0;
+  for (int r = blockIdx.x * blockDim.x + threadIdx.x; r < R; r += gridDim.x * blockDim.x)
+    m = max(m, static_cast<int>(rois[r * 5]) + 1);
+  for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off));
+  if ((threadIdx.x & 63) == 0) atomicMax(out, m);
+}
+
+}  // namespace roialign

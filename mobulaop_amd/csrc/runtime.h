@@ -1,0 +1,88 @@
+// Launcher runtime shared by every operator in the library: per-thread call
+// state (stream, argument extents, error text), per-device scratch memory and
+// staging of host buffers through device memory.
+//
+// Replaces the reference's HIP "context" (mobula/cpp/include/context/hip_ctx.h:
+// 36-106): that one creates, synchronises and destroys a stream around every
+// launch and terminates the process on a HIP error; this one launches on a
+// caller-chosen stream, synchronises only when asked to, and records errors
+// for the caller to pick up.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace mobula_hip {
+
+struct CallState {
+  hipStream_t stream = nullptr;
+  bool synchronous = true;          // wait for completion before returning
+  std::vector<long long> extents;   // element count per argument, -1 = unknown
+  std::string error;                // empty = no error
+};
+
+CallState& call_state();
+
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+inline bool failed() { return !call_state().error.empty(); }
+
+// Element count the caller declared for argument `index` (0-based, device id
+// not counted); -1 if it declared none.  Consumed extents are cleared by
+// finish_call().
+long long arg_extent(int index);
+
+// Grow-only scratch buffer of the current device.  The pointer stays valid
+// until a later call asks for more bytes on the same device.
+void* workspace(size_t bytes);
+
+long long option(const char* name, long long fallback);
+
+// Makes `device` current for the lifetime of the object (no-op for -1).
+class DeviceScope {
+ public:
+  explicit DeviceScope(int device);
+  ~DeviceScope();
+  bool ok() const { return ok_; }
+
+ private:
+  int previous_ = -1;
+  bool changed_ = false;
+  bool ok_ = true;
+};
+
+// Device mirrors of host buffers for calls that arrive with device id -1.
+class HostStaging {
+ public:
+  ~HostStaging();
+  // Device copy of `bytes` bytes at `host` (uploaded when `upload`).
+  void* in(const void* host, size_t bytes, bool upload = true);
+  // Device buffer that is downloaded to `host` by flush().
+  void* inout(void* host, size_t bytes, bool upload);
+  bool flush(hipStream_t stream);  // download outputs, wait for completion
+
+ private:
+  struct Item { void* dev; void* host; size_t bytes; bool download; };
+  std::vector<Item> items_;
+};
+
+// Synchronises if the call is synchronous and clears the per-call extents.
+void finish_call();
+
+}  // namespace mobula_hip
+
+#define MOBULA_HIP_TRY(expr)                                                        \
+  do {                                                                              \
+    hipError_t mobula_hip_status_ = (expr);                                         \
+    if (mobula_hip_status_ != hipSuccess) {                                         \
+      ::mobula_hip::set_error("%s failed: %s (%s:%d)", #expr,                       \
+                              hipGetErrorString(mobula_hip_status_), __FILE__, __LINE__); \
+    }                                                                               \
+  } while (0)
+
+// Launcher functions are ordinary host functions; the macro only marks them
+// for the Python-side declaration scanner.
+#define MOBULA_KERNEL void
+#define MOBULA_FUNC

@@ -1,0 +1,165 @@
+// See runtime.h.
+#include "runtime.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+
+namespace mobula_hip {
+
+CallState& call_state() {
+  static thread_local CallState state;
+  return state;
+}
+
+void set_error(const char* fmt, ...) {
+  CallState& st = call_state();
+  if (!st.error.empty()) return;  // keep the first error of a call
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  st.error = buf;
+}
+
+long long arg_extent(int index) {
+  const auto& e = call_state().extents;
+  return (index >= 0 && index < static_cast<int>(e.size())) ? e[index] : -1;
+}
+
+namespace {
+struct Scratch { void* ptr = nullptr; size_t bytes = 0; };
+std::mutex g_mutex;
+std::map<int, Scratch> g_scratch;
+std::map<std::string, long long> g_options;
+}  // namespace
+
+void* workspace(size_t bytes) {
+  int device = 0;
+  MOBULA_HIP_TRY(hipGetDevice(&device));
+  if (failed()) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  Scratch& s = g_scratch[device];
+  if (s.bytes < bytes) {
+    if (s.ptr != nullptr) MOBULA_HIP_TRY(hipFree(s.ptr));  // waits for pending work
+    s.ptr = nullptr;
+    s.bytes = 0;
+    size_t want = bytes + bytes / 4 + (1u << 20);
+    MOBULA_HIP_TRY(hipMalloc(&s.ptr, want));
+    if (failed()) { s.ptr = nullptr; return nullptr; }
+    s.bytes = want;
+  }
+  return s.ptr;
+}
+
+long long option(const char* name, long long fallback) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto it = g_options.find(name);
+  return it == g_options.end() ? fallback : it->second;
+}
+
+DeviceScope::DeviceScope(int device) {
+  if (device < 0) return;
+  MOBULA_HIP_TRY(hipGetDevice(&previous_));
+  if (failed()) { ok_ = false; return; }
+  if (previous_ != device) {
+    MOBULA_HIP_TRY(hipSetDevice(device));
+    if (failed()) { ok_ = false; return; }
+    changed_ = true;
+  }
+}
+
+DeviceScope::~DeviceScope() {
+  if (changed_) (void)hipSetDevice(previous_);
+}
+
+HostStaging::~HostStaging() {
+  for (auto& it : items_) (void)hipFree(it.dev);
+}
+
+void* HostStaging::in(const void* host, size_t bytes, bool upload) {
+  void* dev = inout(const_cast<void*>(host), bytes, upload);
+  items_.back().download = false;
+  return dev;
+}
+
+void* HostStaging::inout(void* host, size_t bytes, bool upload) {
+  Item item{nullptr, host, bytes, true};
+  MOBULA_HIP_TRY(hipMalloc(&item.dev, bytes > 0 ? bytes : 1));
+  if (!failed() && upload && bytes > 0)
+    MOBULA_HIP_TRY(hipMemcpy(item.dev, host, bytes, hipMemcpyHostToDevice));
+  items_.push_back(item);
+  return item.dev;
+}
+
+bool HostStaging::flush(hipStream_t stream) {
+  MOBULA_HIP_TRY(hipStreamSynchronize(stream));
+  for (auto& it : items_) {
+    if (failed()) break;
+    if (it.download && it.bytes > 0)
+      MOBULA_HIP_TRY(hipMemcpy(it.host, it.dev, it.bytes, hipMemcpyDeviceToHost));
+  }
+  return !failed();
+}
+
+void finish_call() {
+  CallState& st = call_state();
+  if (st.synchronous && !failed()) MOBULA_HIP_TRY(hipStreamSynchronize(st.stream));
+  st.extents.clear();
+}
+
+}  // namespace mobula_hip
+
+using mobula_hip::call_state;
+
+extern "C" {
+
+void mobula_hip_set_stream(void* stream, int synchronous) {
+  auto& st = call_state();
+  st.stream = static_cast<hipStream_t>(stream);
+  st.synchronous = synchronous != 0;
+}
+
+void mobula_hip_set_arg_extents(const long long* numel, int n) {
+  auto& st = call_state();
+  st.extents.assign(numel, numel + (n > 0 ? n : 0));
+}
+
+const char* mobula_hip_last_error(void) {
+  auto& st = call_state();
+  return st.error.empty() ? nullptr : st.error.c_str();
+}
+
+void mobula_hip_clear_error(void) { call_state().error.clear(); }
+
+int mobula_hip_set_option(const char* name, long long value) {
+  static const char* known[] = {"roialign_impl", "host_staging_device", "roialign_fwd_variant",
+                                "roialign_bwd_variant", nullptr};
+  for (int i = 0; known[i] != nullptr; ++i) {
+    if (std::strcmp(known[i], name) == 0) {
+      std::lock_guard<std::mutex> lock(mobula_hip::g_mutex);
+      mobula_hip::g_options[name] = value;
+      return 0;
+    }
+  }
+  return -1;
+}
+
+long long mobula_hip_get_option(const char* name) { return mobula_hip::option(name, -1); }
+
+int mobula_hip_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+  return n;
+}
+
+// Reference: mobula/cpp/src/context.cpp:9-15.
+void set_device(const int device_id) {
+  int current = -1;
+  MOBULA_HIP_TRY(hipGetDevice(&current));
+  if (current != device_id) MOBULA_HIP_TRY(hipSetDevice(device_id));
+}
+}

@@ -1,0 +1,323 @@
+// ROIAlign launchers for gfx950 and their C-ABI entry points.
+//
+// The MOBULA_KERNEL declarations below are what `mobula.op.load('ROIAlign')`
+// scans to bind `mobula.func.roi_align_forward / roi_align_backward /
+// roi_align_backward_assign`; argument lists and meaning are those of the
+// reference kernels (opzoo/ROIAlign/ROIAlign.cpp:9-16, 78-83).  The extern "C"
+// functions at the end carry the names the reference's loader derives for the
+// same instantiations (mobula/func.py:13-50, op/templates/kernel_code.cpp:1-5).
+#include <algorithm>
+#include <type_traits>
+
+#include "runtime.h"
+#include "roialign_naive.hip.h"
+
+namespace {
+
+using mobula_hip::arg_extent;
+using mobula_hip::call_state;
+using mobula_hip::failed;
+using mobula_hip::set_error;
+
+enum Impl { kAuto = 0, kTiled = 1, kNaive = 2 };
+
+struct Problem {
+  long long n_out;  // R*C*PH*PW
+  int R, C, H, W, PH, PW, S;
+  long long N;      // images in the feature map
+  float scale;
+};
+
+// Shape checks shared by every entry point.  Returns false (with the error
+// text set) if the arguments cannot describe a valid problem.  `ext_*` are
+// the positions of the pointer arguments in the call, for the extents the
+// caller may have declared.
+bool describe(Problem* p, const char* what, int nthreads, float scale, int C, int H, int W,
+              int PH, int PW, int S, int ext_map, int ext_rois, int ext_pooled,
+              long long num_images_hint) {
+  if (nthreads < 0 || C <= 0 || H <= 0 || W <= 0 || PH <= 0 || PW <= 0) {
+    set_error("%s: non-positive dimension (nthreads=%d C=%d H=%d W=%d PH=%d PW=%d)", what,
+              nthreads, C, H, W, PH, PW);
+    return false;
+  }
+  const long long per_roi = static_cast<long long>(C) * PH * PW;
+  if (nthreads % per_roi != 0) {
+    set_error("%s: nthreads=%d is not a multiple of C*PH*PW=%lld", what, nthreads, per_roi);
+    return false;
+  }
+  const long long plane = static_cast<long long>(H) * W;
+  if (plane * C >= (1ll << 31)) {
+    set_error("%s: C*H*W=%lld does not fit 32-bit indexing", what, plane * C);
+    return false;
+  }
+  p->n_out = nthreads;
+  p->R = static_cast<int>(nthreads / per_roi);
+  p->C = C; p->H = H; p->W = W; p->PH = PH; p->PW = PW; p->S = S;
+  p->scale = scale;
+  p->N = num_images_hint;
+  const long long e_map = arg_extent(ext_map), e_rois = arg_extent(ext_rois),
+                  e_pool = arg_extent(ext_pooled);
+  if (e_rois >= 0 && e_rois != 5ll * p->R) {
+    set_error("%s: rois holds %lld values, expected R*5=%lld", what, e_rois, 5ll * p->R);
+    return false;
+  }
+  if (e_pool >= 0 && e_pool != p->n_out) {
+    set_error("%s: pooled tensor holds %lld values, expected %lld", what, e_pool, p->n_out);
+    return false;
+  }
+  if (e_map >= 0) {
+    if (e_map % (plane * C) != 0) {
+      set_error("%s: feature map holds %lld values, not a multiple of C*H*W=%lld", what, e_map,
+                plane * C);
+      return false;
+    }
+    const long long n = e_map / (plane * C);
+    if (p->N >= 0 && p->N != n) {
+      set_error("%s: num_images=%lld but the feature map holds %lld images", what, p->N, n);
+      return false;
+    }
+    p->N = n;
+  }
+  return true;
+}
+
+// Number of images when the caller gave neither extents nor a count: read the
+// largest batch index back from the device (one blocking copy).
+long long images_from_rois(const float* d_rois, int R, hipStream_t stream) {
+  if (R == 0) return 0;
+  int* d_max = static_cast<int*>(mobula_hip::workspace(256));
+  if (failed()) return 0;
+  MOBULA_HIP_TRY(hipMemsetAsync(d_max, 0, sizeof(int), stream));
+  roialign::max_batch_kernel<<<std::min(64, (R + 255) / 256), 256, 0, stream>>>(d_rois, R, d_max);
+  int h = 0;
+  MOBULA_HIP_TRY(hipMemcpyAsync(&h, d_max, sizeof(int), hipMemcpyDeviceToHost, stream));
+  MOBULA_HIP_TRY(hipStreamSynchronize(stream));
+  return h;
+}
+
+int grid_for(long long n, int block) {
+  return static_cast<int>(std::min<long long>((n + block - 1) / block, 256ll * 64));
+}
+
+template <typename T>
+void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipStream_t stream) {
+  if (p.n_out == 0) return;
+  roialign::forward_naive_kernel<T><<<grid_for(p.n_out, 256), 256, 0, stream>>>(
+      p.n_out, x, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, rois, y, p.N);
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+void backward_device(const Problem& p, const float* dy, const float* rois, float* dx, bool assign,
+                     hipStream_t stream) {
+  if (assign && p.N > 0)
+    MOBULA_HIP_TRY(hipMemsetAsync(dx, 0, sizeof(float) * p.N * p.C * p.H * p.W, stream));
+  if (p.n_out == 0) return;
+  roialign::backward_naive_kernel<<<grid_for(p.n_out, 256), 256, 0, stream>>>(
+      p.n_out, dy, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, dx, rois, p.N);
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+long long host_images(const float* rois, int R) {
+  long long n = 0;
+  for (int r = 0; r < R; ++r) n = std::max<long long>(n, static_cast<long long>(rois[5 * r]) + 1);
+  return n;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// Launchers (scanned by the Python loader).
+// ---------------------------------------------------------------------------
+
+template <typename T>
+MOBULA_KERNEL roi_align_forward_kernel(const int nthreads, const T* bottom_data,
+                                       const float spatial_scale, const int channels,
+                                       const int height, const int width,
+                                       const int pooled_height, const int pooled_width,
+                                       const int sampling_ratio, const float* bottom_rois,
+                                       T* top_data) {
+  Problem p;
+  if (!describe(&p, "roi_align_forward", nthreads, spatial_scale, channels, height, width,
+                pooled_height, pooled_width, sampling_ratio, 1, 9, 10, -1))
+    return;
+  hipStream_t stream = call_state().stream;
+  if (p.N < 0) p.N = images_from_rois(bottom_rois, p.R, stream);
+  if (failed()) return;
+  forward_device<T>(p, bottom_data, bottom_rois, top_data, stream);
+}
+
+template <typename T>
+MOBULA_KERNEL roi_align_backward_kernel(const int nthreads, const T* top_diff,
+                                        const float spatial_scale, const int channels,
+                                        const int height, const int width,
+                                        const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, T* bottom_diff,
+                                        const float* bottom_rois) {
+  Problem p;
+  if (!describe(&p, "roi_align_backward", nthreads, spatial_scale, channels, height, width,
+                pooled_height, pooled_width, sampling_ratio, 9, 10, 1, -1))
+    return;
+  hipStream_t stream = call_state().stream;
+  if (p.N < 0) p.N = images_from_rois(bottom_rois, p.R, stream);
+  if (failed()) return;
+  backward_device(p, top_diff, bottom_rois, bottom_diff, /*assign=*/false, stream);
+}
+
+// Not in the reference: backward that OVERWRITES bottom_diff (every element is
+// written exactly once; elements no ROI touches become zero), i.e. the
+// operator's "zero dx, then scatter" (opzoo/ROIAlign/ROIAlign.py:33-39) as one
+// entry point.  num_images is the N of the [N,C,H,W] gradient.
+template <typename T>
+MOBULA_KERNEL roi_align_backward_assign_kernel(const int nthreads, const T* top_diff,
+                                               const float spatial_scale, const int channels,
+                                               const int height, const int width,
+                                               const int pooled_height, const int pooled_width,
+                                               const int sampling_ratio, const int num_images,
+                                               T* bottom_diff, const float* bottom_rois) {
+  Problem p;
+  if (num_images < 0) {
+    set_error("roi_align_backward_assign: num_images=%d", num_images);
+    return;
+  }
+  if (!describe(&p, "roi_align_backward_assign", nthreads, spatial_scale, channels, height, width,
+                pooled_height, pooled_width, sampling_ratio, 10, 11, 1, num_images))
+    return;
+  backward_device(p, top_diff, bottom_rois, bottom_diff, /*assign=*/true, call_state().stream);
+}
+
+// ---------------------------------------------------------------------------
+// Entry-point plumbing: device selection, staging of host buffers (device id
+// -1), completion.
+// ---------------------------------------------------------------------------
+namespace {
+
+int staging_device() { return static_cast<int>(mobula_hip::option("host_staging_device", 0)); }
+
+template <typename T>
+void forward_entry(int device_id, int nthreads, const T* x, float scale, int C, int H, int W,
+                   int PH, int PW, int S, const float* rois, T* y) {
+  if (device_id >= 0) {
+    mobula_hip::DeviceScope scope(device_id);
+    if (scope.ok()) roi_align_forward_kernel<T>(nthreads, x, scale, C, H, W, PH, PW, S, rois, y);
+    mobula_hip::finish_call();
+    return;
+  }
+  // Host memory: mirror the buffers on the staging device.
+  mobula_hip::DeviceScope scope(staging_device());
+  auto& st = call_state();
+  const hipStream_t saved_stream = st.stream;
+  st.stream = nullptr;
+  Problem p;
+  if (scope.ok() && describe(&p, "roi_align_forward", nthreads, scale, C, H, W, PH, PW, S, 1, 9,
+                             10, -1)) {
+    if (p.N < 0) p.N = host_images(rois, p.R);
+    st.extents.assign(11, -1);
+    st.extents[1] = p.N * C * H * W;
+    mobula_hip::HostStaging stage;
+    const T* dx = static_cast<const T*>(stage.in(x, sizeof(T) * p.N * C * H * W));
+    const float* dr = static_cast<const float*>(stage.in(rois, sizeof(float) * 5 * p.R));
+    T* dy = static_cast<T*>(stage.inout(y, sizeof(T) * p.n_out, /*upload=*/false));
+    if (!failed()) roi_align_forward_kernel<T>(nthreads, dx, scale, C, H, W, PH, PW, S, dr, dy);
+    if (!failed()) stage.flush(nullptr);
+  }
+  st.stream = saved_stream;
+  st.extents.clear();
+}
+
+template <typename T>
+void backward_entry(int device_id, int nthreads, const T* dy, float scale, int C, int H, int W,
+                    int PH, int PW, int S, int num_images, T* dx, const float* rois) {
+  const bool assign = num_images >= 0;
+  if (device_id >= 0) {
+    mobula_hip::DeviceScope scope(device_id);
+    if (scope.ok()) {
+      if (assign)
+        roi_align_backward_assign_kernel<T>(nthreads, dy, scale, C, H, W, PH, PW, S, num_images,
+                                            dx, rois);
+      else
+        roi_align_backward_kernel<T>(nthreads, dy, scale, C, H, W, PH, PW, S, dx, rois);
+    }
+    mobula_hip::finish_call();
+    return;
+  }
+  mobula_hip::DeviceScope scope(staging_device());
+  auto& st = call_state();
+  const hipStream_t saved_stream = st.stream;
+  st.stream = nullptr;
+  Problem p;
+  const int e_map = assign ? 10 : 9, e_rois = assign ? 11 : 10;
+  if (scope.ok() && describe(&p, "roi_align_backward", nthreads, scale, C, H, W, PH, PW, S, e_map,
+                             e_rois, 1, assign ? num_images : -1)) {
+    if (p.N < 0) p.N = host_images(rois, p.R);
+    mobula_hip::HostStaging stage;
+    const T* ddy = static_cast<const T*>(stage.in(dy, sizeof(T) * p.n_out));
+    const float* dr = static_cast<const float*>(stage.in(rois, sizeof(float) * 5 * p.R));
+    T* ddx = static_cast<T*>(stage.inout(dx, sizeof(T) * p.N * C * H * W, /*upload=*/!assign));
+    st.extents.assign(12, -1);
+    st.extents[e_map] = p.N * C * H * W;
+    if (!failed()) {
+      if (assign)
+        roi_align_backward_assign_kernel<T>(nthreads, ddy, scale, C, H, W, PH, PW, S,
+                                            static_cast<int>(p.N), ddx, dr);
+      else
+        roi_align_backward_kernel<T>(nthreads, ddy, scale, C, H, W, PH, PW, S, ddx, dr);
+    }
+    if (!failed()) stage.flush(nullptr);
+  }
+  st.stream = saved_stream;
+  st.extents.clear();
+}
+
+}  // namespace
+
+extern "C" {
+
+// float instantiations: the symbols the reference binding resolves.
+void roi_align_forward_ab78de3c(const int device_id, const int nthreads, const float* bottom_data,
+                                const float spatial_scale, const int channels, const int height,
+                                const int width, const int pooled_height, const int pooled_width,
+                                const int sampling_ratio, const float* bottom_rois,
+                                float* top_data) {
+  forward_entry<float>(device_id, nthreads, bottom_data, spatial_scale, channels, height, width,
+                       pooled_height, pooled_width, sampling_ratio, bottom_rois, top_data);
+}
+
+void roi_align_backward_f318a24e(const int device_id, const int nthreads, const float* top_diff,
+                                 const float spatial_scale, const int channels, const int height,
+                                 const int width, const int pooled_height, const int pooled_width,
+                                 const int sampling_ratio, float* bottom_diff,
+                                 const float* bottom_rois) {
+  backward_entry<float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+                        pooled_height, pooled_width, sampling_ratio, -1, bottom_diff, bottom_rois);
+}
+
+// Extensions (no counterpart in the reference); names follow the same scheme.
+void roi_align_backward_assign_a8793cbe(const int device_id, const int nthreads,
+                                        const float* top_diff, const float spatial_scale,
+                                        const int channels, const int height, const int width,
+                                        const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        float* bottom_diff, const float* bottom_rois) {
+  if (num_images < 0) {
+    set_error("roi_align_backward_assign: num_images=%d", num_images);
+    return;
+  }
+  backward_entry<float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+                        pooled_height, pooled_width, sampling_ratio, num_images, bottom_diff,
+                        bottom_rois);
+}
+
+void roi_align_forward_e874c59a(const int device_id, const int nthreads, const __half* bottom_data,
+                                const float spatial_scale, const int channels, const int height,
+                                const int width, const int pooled_height, const int pooled_width,
+                                const int sampling_ratio, const float* bottom_rois,
+                                __half* top_data) {
+  forward_entry<__half>(device_id, nthreads, bottom_data, spatial_scale, channels, height, width,
+                        pooled_height, pooled_width, sampling_ratio, bottom_rois, top_data);
+}
+
+const char* mobula_hip_exports(void) {
+  return "roi_align_forward_ab78de3c roi_align_backward_f318a24e "
+         "roi_align_backward_assign_a8793cbe roi_align_forward_e874c59a set_device";
+}
+}

@@ -1,0 +1,85 @@
+"""Direct ctypes calls into the launcher library's C ABI with torch-owned device
+memory (test helper: no Python binding in between)."""
+import ctypes
+
+import numpy as np
+import torch
+
+from mobulaop_amd import native
+
+IMPL = {'auto': 0, 'tiled': 1, 'naive': 2}
+
+
+def _ptr(t):
+    assert t.is_contiguous()
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _begin(extents, stream=None):
+    lib = native.library()
+    if stream is None:
+        lib.mobula_hip_set_stream(None, 1)
+    else:
+        lib.mobula_hip_set_stream(ctypes.c_void_p(stream), 0)
+    if extents is not None:
+        arr = (ctypes.c_longlong * len(extents))(*extents)
+        lib.mobula_hip_set_arg_extents(arr, len(extents))
+    return lib
+
+
+def _end(lib):
+    msg = lib.mobula_hip_last_error()
+    if msg:
+        lib.mobula_hip_clear_error()
+        raise RuntimeError(msg.decode())
+
+
+def _geom(scale, C, H, W, PH, PW, S):
+    return [ctypes.c_float(scale)] + [ctypes.c_int(v) for v in (C, H, W, PH, PW, S)]
+
+
+def forward(x, rois, pooled, scale, S, declare_extents=True, stream=None, dev=0):
+    """x: torch cuda tensor [N,C,H,W] (fp32 or fp16), rois: cuda fp32 [R,5]."""
+    N, C, H, W = x.shape
+    PH, PW = pooled
+    R = rois.shape[0]
+    y = torch.empty((R, C, PH, PW), dtype=x.dtype, device=x.device)
+    ext = [-1, x.numel(), -1, -1, -1, -1, -1, -1, -1, rois.numel(), y.numel()]
+    lib = _begin(ext if declare_extents else [], stream)
+    fn = lib.roi_align_forward_ab78de3c if x.dtype == torch.float32 else lib.roi_align_forward_e874c59a
+    fn(ctypes.c_int(dev), ctypes.c_int(y.numel()), _ptr(x), *_geom(scale, C, H, W, PH, PW, S),
+       _ptr(rois), _ptr(y))
+    _end(lib)
+    return y
+
+
+def backward(dy, rois, shape, scale, S, dx=None, assign=False, declare_extents=True, stream=None,
+             dev=0):
+    N, C, H, W = shape
+    PH, PW = dy.shape[2], dy.shape[3]
+    if dx is None:
+        dx = (torch.full(shape, float('nan'), dtype=dy.dtype, device=dy.device) if assign
+              else torch.zeros(shape, dtype=dy.dtype, device=dy.device))
+    lib = native.library()
+    if assign:
+        ext = [-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()]
+        _begin(ext if declare_extents else [], stream)
+        lib.roi_align_backward_assign_a8793cbe(
+            ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
+            ctypes.c_int(N), _ptr(dx), _ptr(rois))
+    else:
+        ext = [-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()]
+        _begin(ext if declare_extents else [], stream)
+        lib.roi_align_backward_f318a24e(
+            ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
+            _ptr(dx), _ptr(rois))
+    _end(lib)
+    return dx
+
+
+def set_impl(name):
+    native.set_option('roialign_impl', IMPL[name])
+
+
+def to_dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()

@@ -1,0 +1,131 @@
+"""GPU tests of the Python surface: `mobula.op.ROIAlign` through the torch and
+NumPy glues and `mobula.func.*` directly, checked against the CPU oracle."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip('torch')
+
+from mobulaop_amd import workloads  # noqa: E402
+from mobulaop_amd.testing import assert_parity  # noqa: E402
+from oracle import roialign as oracle  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+FWD_TOL, BWD_TOL = 1e-5, 1e-4
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    print('\n[case] {}'.format(request.node.nodeid), flush=True)
+
+
+def _small():
+    w = workloads.make_workload('cfg2', scale_down=32)
+    want_y = oracle.forward(w['data'], w['rois'], w['pooled_size'], w['spatial_scale'],
+                            w['sampling_ratio'])
+    want_dx = oracle.backward(w['dy'], w['rois'], w['data'].shape, w['spatial_scale'],
+                              w['sampling_ratio'], impl='ordered')
+    return w, want_y, want_dx
+
+
+def test_reference_example_through_torch(mobula):
+    # examples/RunROIAlign.py:12-26 with torch tensors on the GPU
+    x = torch.arange(2 * 3 * 4 * 4, dtype=torch.float32, device='cuda').reshape(2, 3, 4, 4)
+    x.requires_grad_(True)
+    rois = torch.tensor([[0, 1, 1, 3, 3]], dtype=torch.float32, device='cuda')
+    out = mobula.op.ROIAlign(data=x, rois=rois, pooled_size=(2, 2), spatial_scale=1.0,
+                             sampling_ratio=1)
+    out.backward(torch.ones_like(out))
+    want = torch.tensor([[7.5, 8.5], [11.5, 12.5]], device='cuda')
+    for c in range(3):
+        assert torch.equal(out[0, c].detach(), want + 16 * c)
+    k = torch.tensor([[.25, .5, .25], [.5, 1, .5], [.25, .5, .25]], device='cuda')
+    assert torch.equal(x.grad[0, 0, 1:4, 1:4], k) and float(x.grad[1].abs().sum()) == 0
+
+
+def test_torch_autograd_path(mobula):
+    w, want_y, want_dx = _small()
+    x = torch.from_numpy(w['data']).cuda().requires_grad_(True)
+    rois = torch.from_numpy(w['rois']).cuda().requires_grad_(True)
+    y = mobula.op.ROIAlign(x, rois, pooled_size=w['pooled_size'],
+                           spatial_scale=w['spatial_scale'], sampling_ratio=w['sampling_ratio'])
+    assert y.requires_grad and y.shape == want_y.shape
+    y.backward(torch.from_numpy(w['dy']).cuda())
+    assert_parity(y, want_y, FWD_TOL, 'y')
+    assert_parity(x.grad, want_dx, BWD_TOL, 'dx')
+    assert float(rois.grad.abs().max()) == 0      # no gradient to the boxes
+    # a second backward accumulates into .grad exactly once
+    y2 = mobula.op.ROIAlign(x, rois, pooled_size=w['pooled_size'],
+                            spatial_scale=w['spatial_scale'], sampling_ratio=w['sampling_ratio'])
+    y2.backward(torch.from_numpy(w['dy']).cuda())
+    assert_parity(x.grad, 2 * want_dx, BWD_TOL, 'dx twice')
+
+
+def test_numpy_path_stages_through_the_gpu(mobula):
+    w, want_y, want_dx = _small()
+    op = mobula.op.ROIAlign[np.ndarray](pooled_size=w['pooled_size'],
+                                        spatial_scale=w['spatial_scale'],
+                                        sampling_ratio=w['sampling_ratio'])
+    y = op(w['data'], w['rois'])
+    assert isinstance(y, np.ndarray)
+    assert_parity(y, want_y, FWD_TOL, 'y')
+    dx, drois = op.backward(w['dy'])
+    assert_parity(dx, want_dx, BWD_TOL, 'dx')
+    assert not drois.any()
+    # req = add accumulates into the caller's gradient, req = null leaves it alone
+    base = np.ones_like(w['data'])
+    op.backward(w['dy'], in_grad=[base, np.zeros_like(w['rois'])], req=['add', 'null'])
+    assert_parity(base, want_dx + 1, BWD_TOL, 'dx add')
+
+
+def test_direct_function_calls_kwargs_and_strided_tensors(mobula):
+    w, want_y, want_dx = _small()
+    N, C, H, W = w['data'].shape
+    PH, PW = w['pooled_size']
+    x = torch.from_numpy(w['data']).cuda()
+    rois = torch.from_numpy(w['rois']).cuda()
+    # output written through a non-contiguous view: copied back after the call
+    backing = torch.zeros(want_y.shape[0], C, PH, 2 * PW, device='cuda')
+    y_view = backing[..., ::2]
+    assert not y_view.is_contiguous()
+    mobula.func.roi_align_forward(
+        nthreads=y_view.numel(), bottom_data=x, spatial_scale=w['spatial_scale'], channels=C,
+        height=H, width=W, pooled_height=PH, pooled_width=PW, sampling_ratio=w['sampling_ratio'],
+        bottom_rois=rois, top_data=y_view)
+    assert_parity(backing[..., ::2], want_y, FWD_TOL, 'strided y')
+    assert float(backing[..., 1::2].abs().sum()) == 0
+    # strided input
+    x_t = torch.from_numpy(np.ascontiguousarray(w['data'].transpose(0, 1, 3, 2))).cuda().transpose(2, 3)
+    assert not x_t.is_contiguous()
+    y = torch.empty(want_y.shape, device='cuda')
+    mobula.func.roi_align_forward(y.numel(), x_t, w['spatial_scale'], C, H, W, PH, PW,
+                                  w['sampling_ratio'], rois, y)
+    assert_parity(y, want_y, FWD_TOL, 'strided x')
+    dx = torch.zeros(N, C, H, W, device='cuda')
+    mobula.func.roi_align_backward(y.numel(), torch.from_numpy(w['dy']).cuda(), w['spatial_scale'],
+                                   C, H, W, PH, PW, w['sampling_ratio'], dx, rois)
+    assert_parity(dx, want_dx, BWD_TOL, 'dx')
+
+
+def test_errors_surface_as_python_exceptions(mobula):
+    x = torch.rand(1, 2, 4, 4, device='cuda')
+    rois = torch.zeros(2, 5, device='cuda')
+    y = torch.empty(3, 2, 2, 2, device='cuda')  # claims 3 ROIs, rois has 2
+    with pytest.raises(RuntimeError):
+        mobula.func.roi_align_forward(y.numel(), x, 1.0, 2, 4, 4, 2, 2, 2, rois, y)
+    with pytest.raises(AssertionError):          # host and device tensor in one call
+        mobula.func.roi_align_forward(8, x, 1.0, 2, 4, 4, 2, 2, 2, rois.cpu().numpy(), y)
+
+
+def test_runs_on_the_callers_stream(mobula):
+    w, want_y, _ = _small()
+    x = torch.from_numpy(w['data']).cuda()
+    rois = torch.from_numpy(w['rois']).cuda()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        y = mobula.op.ROIAlign(x, rois, pooled_size=w['pooled_size'],
+                               spatial_scale=w['spatial_scale'],
+                               sampling_ratio=w['sampling_ratio'])
+        doubled = y * 2          # ordered after the kernel on the same stream
+    side.synchronize()
+    assert_parity(doubled, 2 * want_y, FWD_TOL, 'stream')

@@ -1,0 +1,224 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI, against the CPU
+oracle and the committed golden vectors on the same seeded inputs.
+
+Tolerances (stated by the task for this path): forward 1e-5, backward 1e-4
+(atomic / tile summation order differs), fp16 storage 2e-3; measured as
+|a-b| <= tol*|b| + tol*max|b|.
+"""
+import os
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip('torch')
+
+from mobulaop_amd import workloads  # noqa: E402
+from mobulaop_amd.testing import assert_parity  # noqa: E402
+from oracle import roialign as oracle  # noqa: E402
+import abi_util as abi  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), 'golden')
+FWD_TOL, BWD_TOL, FP16_TOL = 1e-5, 1e-4, 2e-3
+IMPLS = ['naive', 'tiled']
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    print('\n[case] {}'.format(request.node.nodeid), flush=True)
+    yield
+    abi.set_impl('auto')
+
+
+@pytest.mark.parametrize('impl', IMPLS)
+def test_golden_vectors(impl):
+    abi.set_impl(impl)
+    for name in sorted(f for f in os.listdir(GOLDEN) if f.endswith('.npz')):
+        z = np.load(os.path.join(GOLDEN, name))
+        pooled = tuple(int(v) for v in z['pooled_size'])
+        scale, S = float(z['spatial_scale']), int(z['sampling_ratio'])
+        x, rois, dy = abi.to_dev(z['data']), abi.to_dev(z['rois']), abi.to_dev(z['dy'])
+        y = abi.forward(x, rois, pooled, scale, S).cpu().numpy()
+        assert_parity(y, z['y'], FWD_TOL, name + ' fwd')
+        dx = abi.backward(dy, rois, x.shape, scale, S).cpu().numpy()
+        assert_parity(dx, z['dx'], BWD_TOL, name + ' bwd')
+        dx2 = abi.backward(dy, rois, x.shape, scale, S, assign=True).cpu().numpy()
+        assert_parity(dx2, z['dx'], BWD_TOL, name + ' bwd assign')
+
+
+@pytest.mark.parametrize('impl', IMPLS)
+@pytest.mark.parametrize('cfg,down', [('cfg1', 8), ('cfg2', 16), ('cfg3', 32)])
+def test_scaled_configs_against_oracle(impl, cfg, down):
+    abi.set_impl(impl)
+    w = workloads.make_workload(cfg, scale_down=down)
+    pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
+    x, rois, dy = abi.to_dev(w['data']), abi.to_dev(w['rois']), abi.to_dev(w['dy'])
+    y = abi.forward(x, rois, pooled, scale, S).cpu().numpy()
+    assert_parity(y, oracle.forward(w['data'], w['rois'], pooled, scale, S), FWD_TOL, cfg + ' fwd')
+    want_dx = oracle.backward(w['dy'], w['rois'], w['data'].shape, scale, S, impl='ordered')
+    dx = abi.backward(dy, rois, x.shape, scale, S).cpu().numpy()
+    assert_parity(dx, want_dx, BWD_TOL, cfg + ' bwd')
+    dx = abi.backward(dy, rois, x.shape, scale, S, assign=True).cpu().numpy()
+    assert_parity(dx, want_dx, BWD_TOL, cfg + ' bwd assign')
+
+
+@pytest.mark.parametrize('impl', IMPLS)
+def test_backward_accumulates_into_existing_gradient(impl):
+    abi.set_impl(impl)
+    w = workloads.make_workload('cfg1', scale_down=16)
+    scale, S = w['spatial_scale'], w['sampling_ratio']
+    rois, dy = abi.to_dev(w['rois']), abi.to_dev(w['dy'])
+    base = np.random.default_rng(3).standard_normal(w['data'].shape).astype(np.float32)
+    dx = abi.backward(dy, rois, base.shape, scale, S, dx=abi.to_dev(base)).cpu().numpy()
+    want = oracle.backward(w['dy'], w['rois'], base.shape, scale, S, impl='ordered', dx=base.copy())
+    assert_parity(dx, want, BWD_TOL, 'accumulate')
+
+
+@pytest.mark.parametrize('impl', IMPLS)
+def test_fp16_storage_forward(impl):
+    abi.set_impl(impl)
+    w = workloads.make_workload('cfg4', scale_down=16)
+    pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
+    x16 = w['data']
+    y = abi.forward(abi.to_dev(x16), abi.to_dev(w['rois']), pooled, scale, S).cpu().numpy()
+    assert y.dtype == np.float16
+    want = oracle.forward(x16.astype(np.float32), w['rois'], pooled, scale, S)
+    assert_parity(y.astype(np.float32), want.astype(np.float16).astype(np.float32), FP16_TOL, 'fp16')
+
+
+@pytest.mark.parametrize('impl', IMPLS)
+@pytest.mark.parametrize('shape', [
+    # N, C, H, W, R, pooled, scale, S
+    (1, 1, 1, 1, 3, (1, 1), 1.0, 1),        # single-pixel map
+    (2, 3, 5, 7, 11, (2, 3), 0.5, 0),       # tiny odd sizes, adaptive grid
+    (3, 65, 33, 47, 37, (7, 7), 0.25, 2),   # channel count just over one block
+    (2, 130, 18, 70, 50, (14, 14), 0.125, 2),
+    (1, 7, 64, 64, 20, (5, 9), 0.3, 3),     # non-square pooling, S=3
+    (2, 4, 40, 40, 25, (7, 7), 1.0, 5),     # dense grid
+])
+def test_ragged_shapes(impl, shape):
+    abi.set_impl(impl)
+    N, C, H, W, R, pooled, scale, S = shape
+    rng = np.random.default_rng(hash(shape) & 0xffff)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    ext_w, ext_h = W / scale, H / scale
+    c = np.stack([rng.uniform(-0.2 * ext_w, 1.2 * ext_w, R), rng.uniform(-0.2 * ext_h, 1.2 * ext_h, R)], 1)
+    wh = np.stack([rng.uniform(0, ext_w, R), rng.uniform(0, ext_h, R)], 1)
+    rois = np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+    dy = rng.standard_normal((R, C) + pooled).astype(np.float32)
+    y = abi.forward(abi.to_dev(x), abi.to_dev(rois), pooled, scale, S).cpu().numpy()
+    assert_parity(y, oracle.forward(x, rois, pooled, scale, S), FWD_TOL, 'fwd')
+    want = oracle.backward(dy, rois, x.shape, scale, S, impl='ordered')
+    for assign in (False, True):
+        dx = abi.backward(abi.to_dev(dy), abi.to_dev(rois), x.shape, scale, S, assign=assign)
+        assert_parity(dx.cpu().numpy(), want, BWD_TOL, 'bwd assign=%s' % assign)
+
+
+@pytest.mark.parametrize('impl', IMPLS)
+def test_empty_roi_list_and_out_of_range_batch(impl):
+    abi.set_impl(impl)
+    x = torch.rand(2, 4, 8, 8, device='cuda')
+    none = torch.zeros(0, 5, device='cuda')
+    assert abi.forward(x, none, (7, 7), 1.0, 2).shape == (0, 4, 7, 7)
+    dy0 = torch.zeros(0, 4, 7, 7, device='cuda')
+    assert float(abi.backward(dy0, none, x.shape, 1.0, 2, assign=True).abs().sum()) == 0
+    # a batch index beyond the map reads nothing and scatters nothing
+    rois = torch.tensor([[0, 1, 1, 6, 6], [5, 1, 1, 6, 6], [-3, 1, 1, 6, 6]], device='cuda',
+                        dtype=torch.float32)
+    y = abi.forward(x, rois, (2, 2), 1.0, 2)
+    assert float(y[1:].abs().sum()) == 0 and float(y[0].abs().sum()) > 0
+    dy = torch.ones(3, 4, 2, 2, device='cuda')
+    dx = abi.backward(dy, rois, x.shape, 1.0, 2, assign=True)
+    assert abs(float(dx.sum()) - 16.0) < 1e-4 and float(dx[1].abs().sum()) == 0
+
+
+@pytest.mark.parametrize('impl', IMPLS)
+def test_without_declared_extents(impl):
+    # plain C callers do not say how many images there are: N comes from the rois
+    abi.set_impl(impl)
+    w = workloads.make_workload('cfg1', scale_down=32)
+    pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
+    x, rois, dy = abi.to_dev(w['data']), abi.to_dev(w['rois']), abi.to_dev(w['dy'])
+    y = abi.forward(x, rois, pooled, scale, S, declare_extents=False).cpu().numpy()
+    assert_parity(y, oracle.forward(w['data'], w['rois'], pooled, scale, S), FWD_TOL, 'fwd')
+    dx = abi.backward(dy, rois, x.shape, scale, S, declare_extents=False).cpu().numpy()
+    assert_parity(dx, oracle.backward(w['dy'], w['rois'], x.shape, scale, S, impl='ordered'),
+                  BWD_TOL, 'bwd')
+
+
+def test_shape_errors_are_reported_not_fatal():
+    x = torch.rand(2, 4, 8, 8, device='cuda')
+    rois = torch.zeros(3, 5, device='cuda')
+    with pytest.raises(RuntimeError, match='rois holds'):
+        _bad_rois_call(x)
+    # the library is still usable afterwards
+    assert abi.forward(x, rois, (2, 2), 1.0, 2).shape == (3, 4, 2, 2)
+
+
+def _bad_rois_call(x):
+    import ctypes
+    from mobulaop_amd import native
+    lib = native.library()
+    rois = torch.zeros(2, 5, device='cuda')
+    y = torch.empty(3, 4, 2, 2, device='cuda')
+    ext = [-1, x.numel(), -1, -1, -1, -1, -1, -1, -1, rois.numel(), y.numel()]
+    abi._begin(ext)
+    lib.roi_align_forward_ab78de3c(ctypes.c_int(0), ctypes.c_int(y.numel()), abi._ptr(x),
+                                   *abi._geom(1.0, 4, 8, 8, 2, 2, 2), abi._ptr(rois), abi._ptr(y))
+    abi._end(lib)
+
+
+# ---------------------------------------------------------------------------
+# Full benchmark sizes: size-independent properties + oracle on a ROI subset.
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize('cfg', ['cfg2', 'cfg3'])
+def test_full_size_properties(cfg):
+    w = workloads.make_workload(cfg)
+    pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
+    x, rois, dy = abi.to_dev(w['data']), abi.to_dev(w['rois']), abi.to_dev(w['dy'])
+    abi.set_impl('auto')
+    y = abi.forward(x, rois, pooled, scale, S)
+    dx = abi.backward(dy, rois, x.shape, scale, S, assign=True)
+    # (1) oracle on a subset of the ROIs (forward rows are independent)
+    pick = np.random.default_rng(0).choice(w['rois'].shape[0], 48, replace=False)
+    want = oracle.forward(w['data'], w['rois'][pick], pooled, scale, S)
+    assert_parity(y[torch.from_numpy(pick).cuda()].cpu().numpy(), want, FWD_TOL, cfg + ' fwd subset')
+    # (2) adjoint identity ties backward to forward at full size
+    lhs = float((y.double() * dy.double()).sum())
+    rhs = float((x.double() * dx.double()).sum())
+    assert abs(lhs - rhs) <= 1e-6 * float((y.double().abs() * dy.double().abs()).sum())
+    # (3) the straightforward kernels give the same answers
+    abi.set_impl('naive')
+    y_n = abi.forward(x, rois, pooled, scale, S)
+    assert_parity(y.cpu().numpy(), y_n.cpu().numpy(), FWD_TOL, cfg + ' fwd vs naive')
+    del y_n
+    dx_n = abi.backward(dy, rois, x.shape, scale, S)
+    assert_parity(dx.cpu().numpy(), dx_n.cpu().numpy(), BWD_TOL, cfg + ' bwd vs naive')
+    # (4) oracle backward on a few (image, channel) planes via the channel-sliced problem
+    ch = [0, w['data'].shape[1] // 2, w['data'].shape[1] - 1]
+    want_dx = oracle.backward(np.ascontiguousarray(w['dy'][:, ch]), w['rois'],
+                              (x.shape[0], len(ch)) + tuple(x.shape[2:]), scale, S, impl='ordered')
+    assert_parity(dx[:, ch].cpu().numpy(), want_dx, BWD_TOL, cfg + ' bwd planes')
+    # (5) on a constant map every output is the fraction of valid samples, in [0, 1]
+    abi.set_impl('auto')
+    ones = torch.ones_like(x)
+    frac = abi.forward(ones, rois, pooled, scale, S)
+    assert float(frac.min()) >= 0 and float(frac.max()) <= 1 + 1e-6
+    # (6) run-to-run difference of the backward pass stays inside the tolerance
+    dx2 = abi.backward(dy, rois, x.shape, scale, S, assign=True)
+    diff = float((dx - dx2).abs().max())
+    print('{}: backward run-to-run max abs diff {:.3e} (max |dx| {:.3e})'.format(
+        cfg, diff, float(dx.abs().max())), flush=True)
+    assert diff <= BWD_TOL * float(dx.abs().max())
+
+
+def test_fp16_full_size_subset():
+    w = workloads.make_workload('cfg4')
+    pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
+    x, rois = abi.to_dev(w['data']), abi.to_dev(w['rois'])
+    y = abi.forward(x, rois, pooled, scale, S)
+    pick = np.random.default_rng(1).choice(w['rois'].shape[0], 32, replace=False)
+    want = oracle.forward(w['data'].astype(np.float32), w['rois'][pick], pooled, scale, S)
+    got = y[torch.from_numpy(pick).cuda()].float().cpu().numpy()
+    assert_parity(got, want.astype(np.float16).astype(np.float32), FP16_TOL, 'cfg4 subset')
