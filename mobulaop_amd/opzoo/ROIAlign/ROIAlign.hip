@@ -11,6 +11,7 @@
 
 #include "runtime.h"
 #include "roialign_naive.hip.h"
+#include "roialign_backward_tiled.hip.h"
 
 namespace {
 
@@ -107,9 +108,76 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
   MOBULA_HIP_TRY(hipGetLastError());
 }
 
+// Scratch layout of the tile pre-pass, carved out of the device workspace.
+struct TilePlan {
+  roialign::TileGrid grid;
+  roialign::RoiRec* recs;
+  int* tile_count;
+  int* tile_offset;
+  int* tile_rois;
+};
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Runs the pre-pass (ROI records, per-tile ROI lists) for tiles of th x tw
+// pixels.  Returns false if the problem is too large for the list buffers (or
+// on error); the caller then uses the straightforward kernels.
+bool plan_tiles(const Problem& p, const float* rois, int th, int tw, hipStream_t stream,
+                TilePlan* plan) {
+  roialign::TileGrid& g = plan->grid;
+  g.th = th; g.tw = tw;
+  g.ty = (p.H + th - 1) / th;
+  g.tx = (p.W + tw - 1) / tw;
+  g.per_image = g.ty * g.tx;
+  g.total = static_cast<long long>(g.per_image) * p.N;
+  const long long list_cap = static_cast<long long>(p.R) * g.per_image;  // every ROI in every tile
+  if (g.total <= 0 || g.total > (1ll << 24) || list_cap > (1ll << 27)) return false;
+  const size_t b_recs = align_up(sizeof(roialign::RoiRec) * std::max(p.R, 1), 256);
+  const size_t b_cnt = align_up(sizeof(int) * (g.total + 1), 256);
+  const size_t b_list = align_up(sizeof(int) * std::max<long long>(list_cap, 1), 256);
+  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list));
+  if (failed()) return false;
+  plan->recs = reinterpret_cast<roialign::RoiRec*>(base);
+  plan->tile_count = reinterpret_cast<int*>(base + b_recs);
+  plan->tile_offset = reinterpret_cast<int*>(base + b_recs + b_cnt);
+  plan->tile_rois = reinterpret_cast<int*>(base + b_recs + 2 * b_cnt);
+  MOBULA_HIP_TRY(hipMemsetAsync(plan->tile_count, 0, sizeof(int) * (g.total + 1), stream));
+  if (p.R > 0) {
+    roialign::roi_prepare_kernel<<<(p.R + 255) / 256, 256, 0, stream>>>(
+        rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->recs, plan->tile_count);
+  }
+  roialign::tile_scan_kernel<<<1, 1024, 0, stream>>>(plan->tile_count, g.total, plan->tile_offset);
+  if (p.R > 0) {
+    const long long threads = g.total * 64;
+    roialign::tile_fill_kernel<<<static_cast<int>((threads + 255) / 256), 256, 0, stream>>>(
+        plan->recs, p.R, g, plan->tile_offset, plan->tile_rois);
+  }
+  MOBULA_HIP_TRY(hipGetLastError());
+  return !failed();
+}
+
+bool use_tiled() { return mobula_hip::option("roialign_impl", kAuto) != kNaive; }
+
 void backward_device(const Problem& p, const float* dy, const float* rois, float* dx, bool assign,
                      hipStream_t stream) {
-  if (assign && p.N > 0)
+  if (p.N <= 0) return;
+  using BT = roialign::BwdTile;
+  TilePlan plan;
+  if (use_tiled() && roialign::backward_tiled_supports(p.PH, p.PW, p.S) &&
+      plan_tiles(p, rois, BT::TH, BT::TW, stream, &plan)) {
+    const int cblocks = (p.C + BT::CH - 1) / BT::CH;
+    const long long jobs = plan.grid.total * cblocks;
+    const long long grid = (jobs + 7) / 8 * 8;
+    if (grid < (1ll << 31)) {
+      roialign::backward_tiled_kernel<<<static_cast<unsigned>(grid), BT::NT, 0, stream>>>(
+          dy, dx, plan.recs, plan.tile_offset, plan.tile_rois, plan.grid, p.C, p.H, p.W, p.PH,
+          p.PW, cblocks, jobs, assign ? 1 : 0);
+      MOBULA_HIP_TRY(hipGetLastError());
+      return;
+    }
+  }
+  if (failed()) return;
+  if (assign)
     MOBULA_HIP_TRY(hipMemsetAsync(dx, 0, sizeof(float) * p.N * p.C * p.H * p.W, stream));
   if (p.n_out == 0) return;
   roialign::backward_naive_kernel<<<grid_for(p.n_out, 256), 256, 0, stream>>>(
