@@ -2,25 +2,28 @@
 // workgroup, accumulated in LDS and written to memory exactly once -- no global
 // atomics and no separate zero-fill pass.
 //
-// LDS layout: acc[c][1 + row*33 + col], channel stride odd, so the 64 lanes of
+// LDS layout: acc[c][1 + row*34 + col], channel stride odd, so the 64 lanes of
 // a wavefront (one channel each) always hit 64 different banks; weights and
-// pixel positions are the same for all lanes.  Column 32 of row r and column
-// -1 of row r+1 are one shared dummy cell, which lets every column unit be a
-// two-cell read-modify-write even at the tile border.
+// pixel positions are the same for all lanes.  Each row has a dummy cell on
+// either side (columns -1 and 32), which lets every column unit be a two-cell
+// read-modify-write even at the tile border and gives dead units (weights 0,
+// position 32) somewhere harmless to go.
 // LDS float atomics are not used (they run at a few lanes per clock on this
-// part): each of the eight compute wavefronts owns two tile rows instead.
+// part): each of the sixteen wavefronts owns one tile row instead, and there
+// is no barrier between the initial clear and the final store -- every
+// wavefront walks the tile's ROI list on its own.
 //
-// Pipeline per ROI of the tile's list: a ninth wavefront lists the sample
-// units of the next ROI while the compute wavefronts work on the current one.
-// The dy blocks [roi, c0:c0+64, ph_a:ph_b, :] (contiguous in memory) of the
-// next DEPTH iterations are in flight in registers -- one workgroup per CU
-// cannot hide a memory round trip any other way -- and each is dropped into
-// LDS between two barriers when its turn comes.  The geometry records of the
-// tile's ROIs are copied to LDS up front, 128 at a time.
+// Everything uniform stays off the vector ALU, which is what bounds the inner
+// loop: the column units of a ROI come through scalar loads (they are written
+// once per (ROI, tile column) by the pre-pass, see roialign_taps.hip.h), loop
+// control and liveness tests run on scalar registers.  Per (row tap, pooled
+// column) the vector work is one multiply plus, per unit, one address add and
+// two fused multiply-adds around a two-cell LDS read/write.
 //
-// The inner loops are bound by vector-ALU issue, so everything uniform stays
-// off the vector ALU: units are fetched with broadcast LDS reads, loop control
-// and ownership tests run on scalar registers, no integer division per ROI.
+// dy is read straight from memory, one channel per lane: the PW floats of one
+// pooled row are contiguous (28 bytes for PW = 7), the other rows of the same
+// 64-channel block are fetched by the wavefronts that own the rows they land
+// on, so the lines are reused out of L1/L2 while the ROI is being processed.
 //
 // Arithmetic per cell: dx += (dy * (wy / count)) * wx, against the reference's
 // (dy * (wy*wx)) / count (opzoo/ROIAlign/ROIAlign.cpp:143-157): same samples
@@ -32,126 +35,70 @@ namespace roialign {
 
 struct BwdTile {
   static constexpr int TH = 16, TW = 32, CH = 64;
-  static constexpr int NWC = 8;                  // compute wavefronts
-  static constexpr int NTC = NWC * 64;           // compute threads
-  static constexpr int NT = NTC + 64;            // + one producer wavefront
-  static constexpr int ROWS_PER_WAVE = TH / NWC;
-  static constexpr int RS = TW + 1;              // row stride (one dummy cell per row)
+  static constexpr int NW = TH;                  // one wavefront per tile row
+  static constexpr int NT = NW * 64;
+  static constexpr int RS = TW + 2;              // row stride: dummy cell, 32 columns, dummy cell
   static constexpr int CS = TH * RS + 1;         // channel stride, odd
-  static constexpr int DYS = 63;                 // channel stride of the staged dy, odd
-  static constexpr int RU_CAP = 64, CU_CAP = 128;  // axis units per (tile, ROI): rows, columns
-  static constexpr int DEPTH = 4;                // dy blocks in flight per thread
-  static constexpr int REC_CHUNK = 128;          // ROI records held in LDS at a time
-  static constexpr int STAGE_ITERS = (CH * DYS + NTC - 1) / NTC;
-  static constexpr int MAX_PW = 32, MAX_PH = 64;
-  static_assert(CS % 2 == 1 && ROWS_PER_WAVE == 2, "layout");
+  static constexpr int PWB = 8;                  // pooled columns handled per register block
+  static_assert(CS % 2 == 1, "channel stride must be odd");
 };
 
-// Host-side gate: can the tiled backward kernel take this problem?  The unit
-// lists of one (tile, ROI) pair must fit their LDS arrays for any box.  With a
-// fixed grid all PH*S sample rows may fall into one tile; with the adaptive
-// grid samples are more than half a pixel apart (or there is one per pooled
-// row), so a tile sees at most 2*(T+2) + PH of them.
-inline bool backward_tiled_supports(int PH, int PW, int S) {
-  using K = BwdTile;
-  if (PW > K::MAX_PW || PH > K::MAX_PH) return false;
-  const long long rows = S > 0 ? static_cast<long long>(PH) * S : 2 * (K::TH + 2) + PH;
-  const long long cols = S > 0 ? static_cast<long long>(PW) * S : 2 * (K::TW + 2) + PW;
-  return rows <= K::RU_CAP && cols <= K::CU_CAP;
-}
+// Host-side gate: the tiled backward kernel takes fixed sampling grids with
+// S <= 2 whose lists fit the pre-pass layout.
+inline bool backward_tiled_supports(int PH, int PW, int S) { return lists_supported(PH, PW, S); }
 
-// Bit 16 of AxisUnit::bin of a column unit: its cells overlap those of the
-// NEXT unit in the list (set by the producer).
-constexpr int kOverlapsNext = 1 << 16;
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef float float2u __attribute__((ext_vector_type(2), aligned(4)));
 
-// Adds one row tap (NR == 1) or one tap for each of two different tile rows
-// (NR == 2) to the accumulator rows ra / rb: for every column unit u,
-//   row[u.pos] += dy[u.bin]*wy*u.w0,  row[u.pos+1] += dy[u.bin]*wy*u.w1.
-// Units are taken two at a time; when their cells are disjoint all loads are
-// issued before the stores, otherwise unit after unit (LDS accesses of one
-// wavefront complete in program order).  `units` is the same address in every
-// lane, so the unit fetches are broadcast reads and their fields are uniform.
-template <int NR>
-__device__ __forceinline__ void scatter_rows(float* ra, float* rb, const float* dy_a,
-                                             const float* dy_b, float wy_a, float wy_b,
-                                             const AxisUnit* units, int n_units) {
-  int k = 0;
-  for (; k + 1 < n_units; k += 2) {
-    const AxisUnit u0 = units[k], u1 = units[k + 1];
-    const int pw0 = u0.bin & 0xffff, pw1 = u1.bin & 0xffff;
-    const float ga0 = dy_a[pw0] * wy_a, ga1 = dy_a[pw1] * wy_a;
-    float gb0 = 0.0f, gb1 = 0.0f;
-    if (NR == 2) { gb0 = dy_b[pw0] * wy_b; gb1 = dy_b[pw1] * wy_b; }
-    float* const pa0 = ra + u0.pos;
-    float* const pa1 = ra + u1.pos;
-    float* const pb0 = rb + u0.pos;
-    float* const pb1 = rb + u1.pos;
-    if ((__builtin_amdgcn_readfirstlane(u0.bin) & kOverlapsNext) == 0) {
-      const float xa0 = pa0[0], ya0 = pa0[1], xa1 = pa1[0], ya1 = pa1[1];
-      float xb0 = 0.0f, yb0 = 0.0f, xb1 = 0.0f, yb1 = 0.0f;
-      if (NR == 2) { xb0 = pb0[0]; yb0 = pb0[1]; xb1 = pb1[0]; yb1 = pb1[1]; }
-      pa0[0] = fmaf(ga0, u0.w0, xa0); pa0[1] = fmaf(ga0, u0.w1, ya0);
-      pa1[0] = fmaf(ga1, u1.w0, xa1); pa1[1] = fmaf(ga1, u1.w1, ya1);
-      if (NR == 2) {
-        pb0[0] = fmaf(gb0, u0.w0, xb0); pb0[1] = fmaf(gb0, u0.w1, yb0);
-        pb1[0] = fmaf(gb1, u1.w0, xb1); pb1[1] = fmaf(gb1, u1.w1, yb1);
-      }
-    } else {
-      const float xa0 = pa0[0], ya0 = pa0[1];
-      float xb0 = 0.0f, yb0 = 0.0f;
-      if (NR == 2) { xb0 = pb0[0]; yb0 = pb0[1]; }
-      pa0[0] = fmaf(ga0, u0.w0, xa0); pa0[1] = fmaf(ga0, u0.w1, ya0);
-      if (NR == 2) { pb0[0] = fmaf(gb0, u0.w0, xb0); pb0[1] = fmaf(gb0, u0.w1, yb0); }
-      const float xa1 = pa1[0], ya1 = pa1[1];
-      float xb1 = 0.0f, yb1 = 0.0f;
-      if (NR == 2) { xb1 = pb1[0]; yb1 = pb1[1]; }
-      pa1[0] = fmaf(ga1, u1.w0, xa1); pa1[1] = fmaf(ga1, u1.w1, ya1);
-      if (NR == 2) { pb1[0] = fmaf(gb1, u1.w0, xb1); pb1[1] = fmaf(gb1, u1.w1, yb1); }
-    }
-  }
-  if (k < n_units) {
-    const AxisUnit u0 = units[k];
-    const int pw0 = u0.bin & 0xffff;
-    const float ga0 = dy_a[pw0] * wy_a;
-    float* const pa0 = ra + u0.pos;
-    const float xa0 = pa0[0], ya0 = pa0[1];
-    pa0[0] = fmaf(ga0, u0.w0, xa0); pa0[1] = fmaf(ga0, u0.w1, ya0);
-    if (NR == 2) {
-      const float gb0 = dy_b[pw0] * wy_b;
-      float* const pb0 = rb + u0.pos;
-      const float xb0 = pb0[0], yb0 = pb0[1];
-      pb0[0] = fmaf(gb0, u0.w0, xb0); pb0[1] = fmaf(gb0, u0.w1, yb0);
-    }
+// The (up to) eight dy values of one pooled row for this lane's channel.
+__device__ __forceinline__ void load_dy_row(const float* __restrict__ p, int n, float (&d)[8]) {
+  if (n == 7) {
+    const float4u a = *reinterpret_cast<const float4u*>(p);
+    const float2u b = *reinterpret_cast<const float2u*>(p + 4);
+    d[0] = a.x; d[1] = a.y; d[2] = a.z; d[3] = a.w; d[4] = b.x; d[5] = b.y; d[6] = p[6]; d[7] = 0.0f;
+  } else if (n == 8) {
+    const float4u a = *reinterpret_cast<const float4u*>(p);
+    const float4u b = *reinterpret_cast<const float4u*>(p + 4);
+    d[0] = a.x; d[1] = a.y; d[2] = a.z; d[3] = a.w; d[4] = b.x; d[5] = b.y; d[6] = b.z; d[7] = b.w;
+  } else {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) d[k] = k < n ? p[k] : 0.0f;
   }
 }
 
-struct alignas(16) BwdHeader { int n_ru; int n_cu; float inv_count; int pad; };
+// row[u.pos] += g*u.w0, row[u.pos+1] += g*u.w1 for the 2*NPW column units of NPW
+// pooled columns.  BATCH: the cells are pairwise disjoint (or dummy cells), so
+// all loads are issued before the first store -- one LDS round trip.
+// Otherwise unit after unit; LDS accesses of a wavefront complete in program
+// order, so a store is seen by the loads that follow it.
+template <int NPW, bool BATCH>
+__device__ __forceinline__ void add_units(float* row, const float (&g)[8], const AxisUnit* __restrict__ u) {
+  if (BATCH) {
+    float x[2 * NPW], y[2 * NPW];
+#pragma unroll
+    for (int k = 0; k < 2 * NPW; ++k) { x[k] = row[u[k].pos]; y[k] = row[u[k].pos + 1]; }
+#pragma unroll
+    for (int k = 0; k < 2 * NPW; ++k) {
+      row[u[k].pos] = fmaf(g[k >> 1], u[k].w0, x[k]);
+      row[u[k].pos + 1] = fmaf(g[k >> 1], u[k].w1, y[k]);
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < 2 * NPW; ++k) {
+      const float x = row[u[k].pos], y = row[u[k].pos + 1];
+      row[u[k].pos] = fmaf(g[k >> 1], u[k].w0, x);
+      row[u[k].pos + 1] = fmaf(g[k >> 1], u[k].w1, y);
+    }
+  }
+}
 
 __global__ void __launch_bounds__(BwdTile::NT)
 backward_tiled_kernel(const float* __restrict__ dy, float* __restrict__ dx,
-                      const RoiRec* __restrict__ recs, const int* __restrict__ tile_offset,
-                      const int* __restrict__ tile_rois, TileGrid tg, int C, int H, int W, int PH,
-                      int PW, int cblocks, long long num_jobs, int assign
-#ifdef ROIALIGN_PROFILE
-                      , unsigned long long* prof
-#endif
-                      ) {
+                      const int* __restrict__ tile_offset, const int* __restrict__ tile_rois,
+                      const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll, int C, int H,
+                      int W, int PH, int PW, int cblocks, long long num_jobs, int assign) {
   using K = BwdTile;
-#ifdef ROIALIGN_PROFILE
-  long long pt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  const long long t_start = clock64();
-#define PROF_T(var) const long long var = clock64()
-#define PROF_ADD(i, a, b) pt[i] += (b) - (a)
-#else
-#define PROF_T(var)
-#define PROF_ADD(i, a, b)
-#endif
   __shared__ float acc[K::CH * K::CS];
-  __shared__ float dyb[K::CH * K::DYS + 4];   // + a trash word for masked staging stores
-  __shared__ AxisUnit runit[2][K::RU_CAP];
-  __shared__ AxisUnit cunit[2][K::CU_CAP];
-  __shared__ BwdHeader header[2];
-  __shared__ TileRoi rec_s[K::REC_CHUNK];
 
   // XCD-aware job order: consecutive workgroup ids go round-robin to the 8
   // XCDs, so give each XCD a contiguous run of logical jobs (neighbouring
@@ -163,18 +110,17 @@ backward_tiled_kernel(const float* __restrict__ dy, float* __restrict__ dx,
   const int cb = static_cast<int>((job / tg.per_image) % cblocks);
   const int n = static_cast<int>(job / (static_cast<long long>(tg.per_image) * cblocks));
   const long long tile = static_cast<long long>(n) * tg.per_image + t_in_img;
-  const int r0 = (t_in_img / tg.tx) * K::TH, q0 = (t_in_img % tg.tx) * K::TW;
+  const int ty = t_in_img / tg.tx, tx = t_in_img % tg.tx;
+  const int r0 = ty * K::TH, q0 = tx * K::TW;
   const int c0 = cb * K::CH;
   const int nch = min(K::CH, C - c0);
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const bool producer = wave == K::NWC;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // = the tile row this wavefront owns
   const int rows = min(K::TH, H - r0), cols = min(K::TW, W - q0);
   float* const plane0 = dx + (static_cast<size_t>(n) * C + c0) * H * W;
 
   const int list_begin = tile_offset[tile], list_end = tile_offset[tile + 1];
-  const int n_rois = list_end - list_begin;
-  if (n_rois == 0) {
+  if (list_begin == list_end) {
     if (assign) {
       for (int i = tid; i < nch * K::TH * K::TW; i += K::NT) {
         const int col = i % K::TW, row = (i / K::TW) % K::TH, c = i / (K::TW * K::TH);
@@ -186,189 +132,108 @@ backward_tiled_kernel(const float* __restrict__ dy, float* __restrict__ dx,
   }
 
   for (int i = tid; i < K::CH * K::CS; i += K::NT) acc[i] = 0.0f;
+  __syncthreads();
 
-  // dy staging map of the compute threads: element idx = tid + k*NTC of a
-  // [CH][seg] block, seg = words per channel and chunk.  Fixed for the kernel:
-  // st_src = offset inside the ROI's dy block, st_dst = LDS word (the trash
-  // word for elements this thread does not stage).
   const int bins = PH * PW;
-  const int nphc = min(PH, K::DYS / PW);   // pooled rows per staged chunk
-  const int nchunks = (PH + nphc - 1) / nphc;
-  const int seg = nphc * PW;
-  const int last_valid = (PH - (nchunks - 1) * nphc) * PW;  // words/channel of the last chunk
-  int st_src[K::STAGE_ITERS], st_dst[K::STAGE_ITERS], st_j[K::STAGE_ITERS];
-  float st_v[K::DEPTH][K::STAGE_ITERS];
-#pragma unroll
-  for (int k = 0; k < K::STAGE_ITERS; ++k) {
-    const int idx = tid + k * K::NTC;
-    const int c = idx / seg, j = idx - c * seg;
-    const bool mine = !producer && c < nch;
-    st_j[k] = mine ? j : 0x7fffffff;
-    st_src[k] = mine ? c * bins + j : 0;
-    st_dst[k] = mine ? c * K::DYS + j : K::CH * K::DYS;
-  }
+  const int ch = min(lane, nch - 1);                 // lanes past the last channel shadow it
+  float* const row = acc + ch * K::CS + 1 + wave * K::RS;
+  const float* const dy_lane = dy + static_cast<size_t>(c0 + ch) * bins;
+  const size_t roi_dy_stride = static_cast<size_t>(C) * bins;
+  const AxisUnit* const row_lists = lists + static_cast<long long>(ty) * ll.row_stride;
+  const AxisUnit* const col_lists =
+      lists + static_cast<long long>(ll.ty) * ll.row_stride + static_cast<long long>(tx) * ll.col_stride;
+  const AxisUnit kDead = AxisUnit{0, -4, 0.0f, 0.0f};
 
-  auto load_recs = [&](int first) {   // records [first, first+REC_CHUNK) of the list -> LDS
-    for (int i = tid; i < K::REC_CHUNK && first + i < n_rois; i += K::NT) {
-      const int roi = tile_rois[list_begin + first + i];
-      const RoiRec r = recs[roi];
-      rec_s[i] = TileRoi{r.start_h, r.start_w, r.bin_h, r.bin_w, r.grid_h, r.grid_w, r.count, roi};
-    }
+  // Software pipeline over the tile's ROI list, per wavefront:
+  //   stage 1 (ROI it+2): fetch row unit `lane` of its row list
+  //   stage 2 (ROI it+1): which sample rows land on my tile row?  fetch the dy
+  //                       row of the first of them
+  //   stage 3 (ROI it)  : fold all taps into g[pw], walk the column units
+  auto fetch_ru = [&](int it) -> AxisUnit {
+    if (it >= list_end || lane >= kRowSlots) return kDead;
+    return row_lists[static_cast<long long>(tile_rois[it]) * ll.roi_stride + lane];
   };
-  // issue the global loads of one iteration: ROI slot `slot` of rec_s, pooled-row chunk `chunk`
-  auto prefetch = [&](int slot, int chunk, float (&dst)[K::STAGE_ITERS]) {
-    const int roi = __builtin_amdgcn_readfirstlane(rec_s[slot].roi);
-    const float* src = dy + (static_cast<size_t>(roi) * C + c0) * bins + chunk * seg;
-    if (chunk == nchunks - 1 && last_valid != seg) {
-#pragma unroll
-      for (int k = 0; k < K::STAGE_ITERS; ++k) dst[k] = src[st_j[k] < last_valid ? st_src[k] : 0];
-    } else {
-#pragma unroll
-      for (int k = 0; k < K::STAGE_ITERS; ++k) dst[k] = src[st_src[k]];
-    }
+  auto mine_of = [&](const AxisUnit& ru) -> float {
+    return ru.pos == wave ? ru.w0 : ru.pos + 1 == wave ? ru.w1 : 0.0f;
   };
-  auto produce = [&](int slot, int b) {
-#ifdef LAB_NO_PRODUCE
-    if (lane == 0) header[b] = BwdHeader{0, 0, 1.0f, 0};
-    return;
-#endif
-    const TileRoi t = rec_s[slot];
-    const int n_ru = build_axis_units(t.start_h, t.bin_h, PH, t.grid_h, H, r0, K::TH, lane,
-                                      runit[b], K::RU_CAP);
-    const int n_cu = build_axis_units(t.start_w, t.bin_w, PW, t.grid_w, W, q0, K::TW, lane,
-                                      cunit[b], K::CU_CAP);
-    if (lane == 0) header[b] = BwdHeader{n_ru, n_cu, 1.0f / t.count, 0};
-    // mark column units whose cells overlap the next unit's
-    for (int k = lane; k + 1 < n_cu; k += 64) {
-      const int d = cunit[b][k + 1].pos - cunit[b][k].pos;
-      if (d >= -1 && d <= 1) cunit[b][k].bin |= kOverlapsNext;
+  if (wave < rows) {
+    AxisUnit ru_cur = fetch_ru(list_begin), ru_nx = fetch_ru(list_begin + 1);
+    float w_cur = mine_of(ru_cur);
+    unsigned long long taps_cur = __ballot(w_cur != 0.0f);
+    float d_cur[8];
+    {
+      const int ph0 = __builtin_amdgcn_readlane(ru_cur.bin, taps_cur ? __builtin_ctzll(taps_cur) : 0);
+      load_dy_row(dy_lane + tile_rois[list_begin] * roi_dy_stride + ph0 * PW, min(K::PWB, PW), d_cur);
     }
-  };
-
-  // One pipeline step of iteration (slot, chunk); `mine` is the register set
-  // that holds its dy block, (nslot, nchunk) the iteration DEPTH steps ahead.
-  auto step = [&](int slot, int chunk, int b, bool more_rois, bool refill, int nslot, int nchunk,
-                  float (&mine)[K::STAGE_ITERS]) {
-    PROF_T(t0);
-    __syncthreads();  // A: previous iteration fully consumed, dyb is free
-    PROF_T(t1);
+    for (int it = list_begin; it < list_end; ++it) {
+      const int roi_now = tile_rois[it];
+      // stage 1
+      const AxisUnit ru_n2 = fetch_ru(it + 2);
+      // stage 2
+      const float w_nx = mine_of(ru_nx);
+      const unsigned long long taps_nx = __ballot(w_nx != 0.0f);
+      float d_nx[8];
+      if (taps_nx != 0) {
+        const int ph0 = __builtin_amdgcn_readlane(ru_nx.bin, __builtin_ctzll(taps_nx));
+        load_dy_row(dy_lane + tile_rois[it + 1] * roi_dy_stride + ph0 * PW, min(K::PWB, PW), d_nx);
+      }
+      // stage 3
+      if (taps_cur != 0) {
+        const AxisUnit* const cl = col_lists + static_cast<long long>(roi_now) * ll.roi_stride;
+        const float* const dy_roi = dy_lane + roi_now * roi_dy_stride;
+        const bool overlaps = (cl[0].bin & kListOverlaps) != 0;
+        for (int pwb = 0; pwb < PW; pwb += K::PWB) {
+          const int nb = min(K::PWB, PW - pwb);
+          float g[8];
+          unsigned long long taps = taps_cur;
+          bool first = true;
+          while (taps != 0) {
+            const int i = __builtin_ctzll(taps);
+            taps &= taps - 1;
+            const int ph = __builtin_amdgcn_readlane(ru_cur.bin, i);
+            const float wy = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_cur), i));
+            float d[8];
+            if (first && pwb == 0) {
 #pragma unroll
-    for (int k = 0; k < K::STAGE_ITERS; ++k) dyb[st_dst[k]] = mine[k];
-    PROF_T(t2);
-    __syncthreads();  // B: dyb and the unit lists of this ROI are visible
-    PROF_T(t3);
-    PROF_ADD(0, t0, t1); PROF_ADD(1, t1, t2); PROF_ADD(2, t2, t3);
-    if (producer) {
-      if (chunk == nchunks - 1 && more_rois) produce(slot + 1, b ^ 1);
-      PROF_T(t4);
-      PROF_ADD(4, t3, t4);
-      return;
-    }
-    if (refill) prefetch(nslot, nchunk, mine);
-
-    const BwdHeader hd = header[b];
-    const int n_ru = __builtin_amdgcn_readfirstlane(hd.n_ru);
-    const int n_cu = __builtin_amdgcn_readfirstlane(hd.n_cu);
-    if (n_ru > 0 && n_cu > 0) {
-      const int ph_a = chunk * nphc, ph_b = min(PH, ph_a + nphc);
-      // Lane i looks at row unit i: which part of it lands on the two tile rows
-      // this wavefront owns (row_a, row_a + 1)?
-      const AxisUnit ru = lane < n_ru ? runit[b][lane] : AxisUnit{0, -4, 0.0f, 0.0f};
-      const int row_a = wave * K::ROWS_PER_WAVE;
-      const bool in_chunk = ru.bin >= ph_a && ru.bin < ph_b;
-      const float w_a = !in_chunk ? 0.0f : ru.pos == row_a ? ru.w0 : ru.pos + 1 == row_a ? ru.w1 : 0.0f;
-      const float w_b = !in_chunk ? 0.0f : ru.pos == row_a + 1 ? ru.w0 : ru.pos == row_a ? ru.w1 : 0.0f;
-      unsigned long long m_a = __ballot(w_a != 0.0f), m_b = __ballot(w_b != 0.0f);
-      if (lane < nch) {
-        float* const row_ptr_a = acc + lane * K::CS + 1 + row_a * K::RS;
-        float* const row_ptr_b = row_ptr_a + K::RS;
-        const float* const dy_lane = dyb + lane * K::DYS - ph_a * PW;
-        const AxisUnit* const units = cunit[b];
-        while ((m_a | m_b) != 0) {
-          // next tap of each owned row; a row without one sits this round out
-          const bool has_a = m_a != 0, has_b = m_b != 0;
-          const int i_a = has_a ? __builtin_ctzll(m_a) : 0, i_b = has_b ? __builtin_ctzll(m_b) : 0;
-          m_a &= m_a - 1; m_b &= m_b - 1;
-          const float wy_a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_a), i_a)) * hd.inv_count;
-          const float wy_b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_b), i_b)) * hd.inv_count;
-          const float* const dy_a = dy_lane + __builtin_amdgcn_readlane(ru.bin, i_a) * PW;
-          const float* const dy_b = dy_lane + __builtin_amdgcn_readlane(ru.bin, i_b) * PW;
-#ifdef LAB_NO_SCATTER
-          if (wy_a == 12345.f) acc[lane] = wy_b + dy_a[0] + dy_b[0];
-          continue;
-#endif
-          if (has_a && has_b)
-            scatter_rows<2>(row_ptr_a, row_ptr_b, dy_a, dy_b, wy_a, wy_b, units, n_cu);
-          else if (has_a)
-            scatter_rows<1>(row_ptr_a, row_ptr_a, dy_a, dy_a, wy_a, wy_a, units, n_cu);
-          else
-            scatter_rows<1>(row_ptr_b, row_ptr_b, dy_b, dy_b, wy_b, wy_b, units, n_cu);
+              for (int k = 0; k < 8; ++k) d[k] = d_cur[k];
+            } else {
+              load_dy_row(dy_roi + ph * PW + pwb, nb, d);
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) g[k] = first ? d[k] * wy : fmaf(d[k], wy, g[k]);
+            first = false;
+          }
+          const AxisUnit* const u = cl + 2 * pwb;
+          if (lane < nch) {
+#define ROIALIGN_ADD_CASE(N)                                                            \
+  case N:                                                                                \
+    if (overlaps) add_units<N, false>(row, g, u); else add_units<N, true>(row, g, u);    \
+    break;
+            switch (nb) {
+              ROIALIGN_ADD_CASE(8) ROIALIGN_ADD_CASE(7) ROIALIGN_ADD_CASE(6) ROIALIGN_ADD_CASE(5)
+              ROIALIGN_ADD_CASE(4) ROIALIGN_ADD_CASE(3) ROIALIGN_ADD_CASE(2) ROIALIGN_ADD_CASE(1)
+            }
+#undef ROIALIGN_ADD_CASE
+          }
         }
       }
-    }
-    PROF_T(t5);
-    PROF_ADD(3, t3, t5);
-  };
-
-  // Driver: records are (re)loaded every REC_CHUNK ROIs and the pipeline is
-  // refilled after each reload.  Iterations run over (ROI, chunk), chunk fastest.
-  for (int first = 0; first < n_rois; first += K::REC_CHUNK) {
-    __syncthreads();
-    load_recs(first);
-    __syncthreads();
-    const int here = min(K::REC_CHUNK, n_rois - first);   // ROIs in this batch
-    // (slot, chunk) of the iteration being executed and of the one DEPTH ahead
-    int slot = 0, chunk = 0, nslot = 0, nchunk = 0;
-    if (producer) {
-      produce(0, 0);
-    } else {
+      // rotate
+      ru_cur = ru_nx; ru_nx = ru_n2; w_cur = w_nx; taps_cur = taps_nx;
 #pragma unroll
-      for (int s = 0; s < K::DEPTH; ++s) {
-        if (nslot < here) prefetch(nslot, nchunk, st_v[s]);
-        if (++nchunk == nchunks) { nchunk = 0; ++nslot; }
-      }
-    }
-    while (slot < here) {
-#pragma unroll
-      for (int s = 0; s < K::DEPTH; ++s) {
-        if (slot < here) {
-          step(slot, chunk, slot & 1, slot + 1 < here, nslot < here, nslot, nchunk, st_v[s]);
-          if (++chunk == nchunks) { chunk = 0; ++slot; }
-          if (++nchunk == nchunks) { nchunk = 0; ++nslot; }
-        }
-      }
+      for (int k = 0; k < 8; ++k) d_cur[k] = d_nx[k];
     }
   }
-  PROF_T(t_w0);
   __syncthreads();
 
   // Owner writes its tile: two 32-pixel rows per wavefront access.
   for (int i = tid; i < nch * K::TH * K::TW; i += K::NT) {
-    const int col = i % K::TW, row = (i / K::TW) % K::TH, c = i / (K::TW * K::TH);
-    if (row < rows && col < cols) {
-      float* p = plane0 + static_cast<size_t>(c) * H * W + static_cast<size_t>(r0 + row) * W + q0 + col;
-      const float v = acc[c * K::CS + 1 + row * K::RS + col];
+    const int col = i % K::TW, row_i = (i / K::TW) % K::TH, c = i / (K::TW * K::TH);
+    if (row_i < rows && col < cols) {
+      float* p = plane0 + static_cast<size_t>(c) * H * W + static_cast<size_t>(r0 + row_i) * W + q0 + col;
+      const float v = acc[c * K::CS + 1 + row_i * K::RS + col];
       *p = assign ? v : *p + v;
     }
   }
-#ifdef ROIALIGN_PROFILE
-  const long long t_end = clock64();
-  if (lane == 0 && (wave == 0 || producer)) {
-    if (wave == 0) {
-      atomicAdd(prof + 0, (unsigned long long)(t_end - t_start));
-      atomicAdd(prof + 1, (unsigned long long)pt[0]);
-      atomicAdd(prof + 2, (unsigned long long)pt[1]);
-      atomicAdd(prof + 3, (unsigned long long)pt[2]);
-      atomicAdd(prof + 4, (unsigned long long)pt[3]);
-      atomicAdd(prof + 5, (unsigned long long)(t_end - t_w0));
-    } else {
-      atomicAdd(prof + 6, (unsigned long long)pt[4]);
-      atomicAdd(prof + 7, (unsigned long long)(pt[0] + pt[2]));
-    }
-  }
-#endif
-#undef PROF_T
-#undef PROF_ADD
 }
 
 }  // namespace roialign

@@ -1,15 +1,24 @@
-// Per-(tile, ROI) sample lists shared by the tiled forward and backward kernels.
+// Per-ROI sample lists shared by the tiled kernels.
 //
 // A sample at (y, x) touches rows {y_low, y_high} with weights {hy, ly} and
 // columns {x_low, x_high} with weights {hx, lx}; the weight of a pixel is the
 // product, and a sample outside [-1, size] on either axis contributes nothing
 // (opzoo/ROIAlign/bilinear.h:15-48).  Because of this product structure the
 // contribution of one ROI to one tile is fully described by two short lists,
-//   axis units along y:  (pooled row ph,  local row r,  weights of rows r, r+1)
-//   axis units along x:  (pooled col pw,  local col c,  weights of cols c, c+1)
-// one unit per sample row / sample column that has a corner inside the tile.
-// A corner outside the tile gets weight 0 here (its owner tile accounts for
-// it), so local positions range over [-1, T-1].
+//   units along y:  (pooled row ph,  local row r,  weights of rows r, r+1)
+//   units along x:  (pooled col pw,  local col c,  weights of cols c, c+1)
+// one unit per sample row / sample column.  A corner outside the tile gets
+// weight 0 (its owner tile accounts for it), so local positions range over
+// [-1, T-1]; a unit with both weights 0 is dead.
+//
+// The lists depend only on (ROI, tile row) and (ROI, tile column), so the
+// pre-pass writes them once to memory and every tile owner that needs them
+// reads them back:
+//   row list  of (roi, ty): kRowSlots units, slot = sample row index
+//                           ph*S + iy; weights already divided by the sample
+//                           count of the bin
+//   col list  of (roi, tx): PW*2 units, slot = pw*2 + ix
+// Only fixed sampling grids with S <= 2 use this path.
 // Sample coordinates come from roialign_geometry.h (reference operation order).
 #pragma once
 #include "roialign_tiles.hip.h"
@@ -19,42 +28,118 @@ namespace roialign {
 // `bin` is the pooled row/column; `pos` the local position of the low corner.
 struct alignas(16) AxisUnit { int bin; int pos; float w0, w1; };
 
-// What the tile owners need of a RoiRec, plus the ROI index: 32 bytes.
-struct alignas(16) TileRoi {
-  float start_h, start_w, bin_h, bin_w;
-  int grid_h, grid_w;
-  float count;
-  int roi;
+// Bit 16 of `bin` of the first column unit of a pooled column: the cells of
+// its two units overlap.  Bit 17: this pooled column's cells overlap the next
+// pooled column's.
+// Bit 18 of `bin` of slot 0 of a column list: some cells of the list overlap
+// (otherwise all of its live units may be processed in any order, or at once).
+constexpr int kPairOverlaps = 1 << 16;
+constexpr int kNextOverlaps = 1 << 17;
+constexpr int kListOverlaps = 1 << 18;
+
+constexpr int kRowSlots = 32;   // PH * S <= 32
+constexpr int kMaxListPW = 16;  // PW <= 16, S <= 2
+
+struct ListLayout {
+  int ty, tx;            // tiles per image
+  int row_stride;        // units per (roi, ty) row list   = kRowSlots
+  int col_stride;        // units per (roi, tx) column list = 2 * PW
+  long long roi_stride;  // units per ROI: ty*row_stride + tx*col_stride
 };
 
-// One wavefront lists the units of one axis: samples (p, i), p < pooled,
-// i < grid, whose low or high corner lies in [t0, t0+tsize).  Order = sample
-// order.  Returns the (lane-uniform) count, clamped to `cap`.
-__device__ __forceinline__ int build_axis_units(float start, float bin, int pooled, int grid,
-                                                int size, int t0, int tsize, int lane,
-                                                AxisUnit* out, int cap) {
-  const int total = pooled * grid;
-  int n = 0;
-  for (int s0 = 0; s0 < total; s0 += 64) {
-    const int s = s0 + lane;
-    AxisUnit u;
-    bool live = false;
-    if (s < total) {
-      u.bin = s / grid;
-      const AxisSample a = axis_sample(sample_coord(start, u.bin, bin, s - u.bin * grid, grid), size);
-      u.pos = a.low - t0;
-      const bool lo_in = u.pos >= 0 && u.pos < tsize;
-      const bool hi_in = a.high != a.low && u.pos + 1 >= 0 && u.pos + 1 < tsize;
-      u.w0 = lo_in ? a.h : 0.0f;
-      u.w1 = hi_in ? a.l : 0.0f;
-      live = a.valid && (u.w0 != 0.0f || u.w1 != 0.0f);
-    }
-    const unsigned long long m = __ballot(live);
-    const int idx = n + __popcll(m & ((1ull << lane) - 1ull));
-    if (live && idx < cap) out[idx] = u;
-    n += __popcll(m);
+inline ListLayout make_list_layout(const TileGrid& tg, int PW) {
+  ListLayout l;
+  l.ty = tg.ty; l.tx = tg.tx;
+  l.row_stride = kRowSlots;
+  l.col_stride = 2 * PW;
+  l.roi_stride = static_cast<long long>(l.ty) * l.row_stride + static_cast<long long>(l.tx) * l.col_stride;
+  return l;
+}
+
+inline bool lists_supported(int PH, int PW, int S) {
+  return S >= 1 && S <= 2 && PH * S <= kRowSlots && PW <= kMaxListPW;
+}
+
+__device__ __forceinline__ AxisUnit clip_unit(int bin, const AxisSample& a, int t0, int tsize,
+                                              float scale) {
+  AxisUnit u;
+  u.bin = bin;
+  u.pos = a.low - t0;
+  const bool lo_in = a.valid && u.pos >= 0 && u.pos < tsize;
+  const bool hi_in = a.valid && a.high != a.low && u.pos + 1 >= 0 && u.pos + 1 < tsize;
+  u.w0 = lo_in ? a.h * scale : 0.0f;
+  u.w1 = hi_in ? a.l * scale : 0.0f;
+  // dead units point at the two dummy cells to the right of a tile row
+  if (!(lo_in || hi_in) || (u.w0 == 0.0f && u.w1 == 0.0f)) { u.pos = tsize; u.w0 = u.w1 = 0.0f; }
+  return u;
+}
+
+// One wavefront per ROI: lane s < PH*S evaluates sample row s once and clips it
+// against every tile row of the ROI's box; likewise for sample columns.
+__global__ void __launch_bounds__(256)
+build_lists_kernel(const RoiRec* __restrict__ recs, int R, int PH, int PW, int S, int H, int W,
+                   TileGrid tg, ListLayout ll, AxisUnit* __restrict__ lists) {
+  const int roi = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  if (roi >= R) return;
+  const int lane = threadIdx.x & 63;
+  const RoiRec rec = recs[roi];
+  if (rec.row_lo > rec.row_hi) return;
+  AxisUnit* const base = lists + static_cast<long long>(roi) * ll.roi_stride;
+  const float inv_count = 1.0f / rec.count;
+  {
+    const int ph = lane / S, iy = lane - ph * S;
+    const bool real = lane < PH * S;
+    AxisSample a = axis_sample(sample_coord(rec.start_h, ph, rec.bin_h, iy, S), H);
+    a.valid = a.valid && real;
+    for (int ty = rec.row_lo / tg.th; ty <= rec.row_hi / tg.th; ++ty)
+      if (lane < kRowSlots)
+        base[ty * ll.row_stride + lane] = clip_unit(ph, a, ty * tg.th, tg.th, inv_count);
   }
-  return min(n, cap);
+  {
+    const int pw = lane / S, ix = lane - pw * S;
+    const bool real = lane < PW * S;
+    AxisSample a = axis_sample(sample_coord(rec.start_w, pw, rec.bin_w, ix, S), W);
+    a.valid = a.valid && real;
+    AxisUnit* const cols = base + static_cast<long long>(ll.ty) * ll.row_stride;
+    for (int tx = rec.col_lo / tg.tw; tx <= rec.col_hi / tg.tw; ++tx) {
+      AxisUnit u = clip_unit(pw, a, tx * tg.tw, tg.tw, 1.0f);
+      const bool live = u.w0 != 0.0f || u.w1 != 0.0f;
+      // neighbours: the other unit of this pooled column, the units of the next one
+      const int pos_next = __shfl_down(u.pos, 1), pos_next2 = __shfl_down(u.pos, 2);
+      const bool live_next = __shfl_down(live ? 1 : 0, 1) != 0;
+      const bool live_next2 = __shfl_down(live ? 1 : 0, 2) != 0;
+      auto near = [](int p, int q) { return p - q >= -1 && p - q <= 1; };
+      if (S == 2) {
+        // lane = 2*pw + ix.  Flags live in the ix == 0 unit.
+        const bool pair = live && live_next && near(u.pos, pos_next);
+        // this column's units vs the next column's two units
+        const int pos_next3 = __shfl_down(u.pos, 3);
+        const bool live_next3 = __shfl_down(live ? 1 : 0, 3) != 0;
+        bool next = false;
+        if (ix == 0) {
+          next = (live && live_next2 && near(u.pos, pos_next2)) ||
+                 (live && live_next3 && near(u.pos, pos_next3)) ||
+                 (live_next && live_next2 && near(pos_next, pos_next2)) ||
+                 (live_next && live_next3 && near(pos_next, pos_next3));
+          if (pair) u.bin |= kPairOverlaps;
+          if (next) u.bin |= kNextOverlaps;
+        }
+        const unsigned long long any_overlap = __ballot(ix == 0 && (pair || next));
+        if (lane == 0 && any_overlap != 0) u.bin |= kListOverlaps;
+        if (real) cols[tx * ll.col_stride + lane] = u;
+      } else {
+        // S == 1: slot 2*pw holds the unit, slot 2*pw + 1 is dead
+        const bool next = live && live_next && near(u.pos, pos_next);
+        if (next) u.bin |= kNextOverlaps;
+        const unsigned long long any_overlap = __ballot(next);
+        if (lane == 0 && any_overlap != 0) u.bin |= kListOverlaps;
+        if (real) {
+          cols[tx * ll.col_stride + 2 * lane] = u;
+          cols[tx * ll.col_stride + 2 * lane + 1] = AxisUnit{pw, tg.tw, 0.0f, 0.0f};
+        }
+      }
+    }
+  }
 }
 
 }  // namespace roialign

@@ -115,6 +115,8 @@ struct TilePlan {
   int* tile_count;
   int* tile_offset;
   int* tile_rois;
+  roialign::ListLayout layout;
+  roialign::AxisUnit* lists;   // null unless requested
 };
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -122,8 +124,8 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // Runs the pre-pass (ROI records, per-tile ROI lists) for tiles of th x tw
 // pixels.  Returns false if the problem is too large for the list buffers (or
 // on error); the caller then uses the straightforward kernels.
-bool plan_tiles(const Problem& p, const float* rois, int th, int tw, hipStream_t stream,
-                TilePlan* plan) {
+bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_lists,
+                hipStream_t stream, TilePlan* plan) {
   roialign::TileGrid& g = plan->grid;
   g.th = th; g.tw = tw;
   g.ty = (p.H + th - 1) / th;
@@ -135,8 +137,14 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, hipStream_t
   const size_t b_recs = align_up(sizeof(roialign::RoiRec) * std::max(p.R, 1), 256);
   const size_t b_cnt = align_up(sizeof(int) * (g.total + 1), 256);
   const size_t b_list = align_up(sizeof(int) * std::max<long long>(list_cap, 1), 256);
-  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list));
+  plan->layout = roialign::make_list_layout(g, p.PW);
+  const long long n_units = with_lists ? plan->layout.roi_stride * p.R : 0;
+  if (n_units > (1ll << 25)) return false;   // 512 MiB of sample lists: not worth it
+  const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256);
+  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list + b_units));
   if (failed()) return false;
+  plan->lists = with_lists ? reinterpret_cast<roialign::AxisUnit*>(base + b_recs + 2 * b_cnt + b_list)
+                           : nullptr;
   plan->recs = reinterpret_cast<roialign::RoiRec*>(base);
   plan->tile_count = reinterpret_cast<int*>(base + b_recs);
   plan->tile_offset = reinterpret_cast<int*>(base + b_recs + b_cnt);
@@ -151,6 +159,9 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, hipStream_t
     const long long threads = g.total * 64;
     roialign::tile_fill_kernel<<<static_cast<int>((threads + 255) / 256), 256, 0, stream>>>(
         plan->recs, p.R, g, plan->tile_offset, plan->tile_rois);
+    if (with_lists)
+      roialign::build_lists_kernel<<<(p.R * 64 + 255) / 256, 256, 0, stream>>>(
+          plan->recs, p.R, p.PH, p.PW, p.S, p.H, p.W, g, plan->layout, plan->lists);
   }
   MOBULA_HIP_TRY(hipGetLastError());
   return !failed();
@@ -164,14 +175,14 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
   using BT = roialign::BwdTile;
   TilePlan plan;
   if (use_tiled() && roialign::backward_tiled_supports(p.PH, p.PW, p.S) &&
-      plan_tiles(p, rois, BT::TH, BT::TW, stream, &plan)) {
+      plan_tiles(p, rois, BT::TH, BT::TW, /*with_lists=*/true, stream, &plan)) {
     const int cblocks = (p.C + BT::CH - 1) / BT::CH;
     const long long jobs = plan.grid.total * cblocks;
     const long long grid = (jobs + 7) / 8 * 8;
     if (grid < (1ll << 31)) {
       roialign::backward_tiled_kernel<<<static_cast<unsigned>(grid), BT::NT, 0, stream>>>(
-          dy, dx, plan.recs, plan.tile_offset, plan.tile_rois, plan.grid, p.C, p.H, p.W, p.PH,
-          p.PW, cblocks, jobs, assign ? 1 : 0);
+          dy, dx, plan.tile_offset, plan.tile_rois, plan.lists, plan.grid, plan.layout, p.C, p.H,
+          p.W, p.PH, p.PW, cblocks, jobs, assign ? 1 : 0);
       MOBULA_HIP_TRY(hipGetLastError());
       return;
     }
