@@ -31,11 +31,13 @@ struct alignas(16) AxisUnit { int bin; int pos; float w0, w1; };
 // Bit 16 of `bin` of the first column unit of a pooled column: the cells of
 // its two units overlap.  Bit 17: this pooled column's cells overlap the next
 // pooled column's.
-// Bit 18 of `bin` of slot 0 of a column list: some cells of the list overlap
-// (otherwise all of its live units may be processed in any order, or at once).
+// Bits 18..20 of `bin` of slot 0 of a column list: log2 of the smallest power
+// of two s such that units k and k+s of the list never share a cell.  Units
+// k, k+s, k+2s, ... can then be processed together (loads before stores).
 constexpr int kPairOverlaps = 1 << 16;
 constexpr int kNextOverlaps = 1 << 17;
-constexpr int kListOverlaps = 1 << 18;
+constexpr int kStrideShift = 18;
+constexpr int kStrideMask = 7;
 
 constexpr int kRowSlots = 32;   // PH * S <= 32
 constexpr int kMaxListPW = 16;  // PW <= 16, S <= 2
@@ -124,15 +126,35 @@ build_lists_kernel(const RoiRec* __restrict__ recs, int R, int PH, int PW, int S
           if (pair) u.bin |= kPairOverlaps;
           if (next) u.bin |= kNextOverlaps;
         }
-        const unsigned long long any_overlap = __ballot(ix == 0 && (pair || next));
-        if (lane == 0 && any_overlap != 0) u.bin |= kListOverlaps;
+        {
+          // smallest power-of-two stride at which no two live units share a cell
+          int lg = 0;
+#pragma unroll
+          for (int d = 1; d <= 16; d <<= 1) {
+            const int pos_d = __shfl_down(u.pos, d);
+            const bool live_d = __shfl_down(live ? 1 : 0, d) != 0;
+            const bool clash = live && live_d && lane + d < PW * S && near(u.pos, pos_d);
+            if (__ballot(clash) != 0) lg = (d == 16) ? 5 : __builtin_ctz(d) + 1;
+          }
+          if (lane == 0) u.bin |= lg << kStrideShift;
+        }
         if (real) cols[tx * ll.col_stride + lane] = u;
       } else {
         // S == 1: slot 2*pw holds the unit, slot 2*pw + 1 is dead
         const bool next = live && live_next && near(u.pos, pos_next);
         if (next) u.bin |= kNextOverlaps;
-        const unsigned long long any_overlap = __ballot(next);
-        if (lane == 0 && any_overlap != 0) u.bin |= kListOverlaps;
+        {
+          int lg = 0;
+#pragma unroll
+          for (int d = 1; d <= 16; d <<= 1) {
+            const int pos_d = __shfl_down(u.pos, d);
+            const bool live_d = __shfl_down(live ? 1 : 0, d) != 0;
+            const bool clash = live && live_d && lane + d < PW && near(u.pos, pos_d);
+            // slots are 2 apart for S == 1
+            if (__ballot(clash) != 0) lg = (d == 16) ? 5 : __builtin_ctz(d) + 2;
+          }
+          if (lane == 0) u.bin |= min(lg, 5) << kStrideShift;
+        }
         if (real) {
           cols[tx * ll.col_stride + 2 * lane] = u;
           cols[tx * ll.col_stride + 2 * lane + 1] = AxisUnit{pw, tg.tw, 0.0f, 0.0f};

@@ -117,6 +117,7 @@ struct TilePlan {
   int* tile_rois;
   roialign::ListLayout layout;
   roialign::AxisUnit* lists;   // null unless requested
+  float* dyt;                  // [R][PH][C][8] copy of dy, with the lists
 };
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -140,9 +141,11 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   plan->layout = roialign::make_list_layout(g, p.PW);
   const long long n_units = with_lists ? plan->layout.roi_stride * p.R : 0;
   if (n_units > (1ll << 25)) return false;   // 512 MiB of sample lists: not worth it
-  const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256);
-  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list + b_units));
+  const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256) + 256;  // blocks are read whole
+  const size_t b_dyt = with_lists ? align_up(sizeof(float) * 8 * p.R * p.PH * p.C, 256) : 0;
+  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list + b_units + b_dyt));
   if (failed()) return false;
+  plan->dyt = with_lists ? reinterpret_cast<float*>(base + b_recs + 2 * b_cnt + b_list + b_units) : nullptr;
   plan->lists = with_lists ? reinterpret_cast<roialign::AxisUnit*>(base + b_recs + 2 * b_cnt + b_list)
                            : nullptr;
   plan->recs = reinterpret_cast<roialign::RoiRec*>(base);
@@ -180,8 +183,11 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
     const long long jobs = plan.grid.total * cblocks;
     const long long grid = (jobs + 7) / 8 * 8;
     if (grid < (1ll << 31)) {
+      if (p.R > 0)
+        roialign::transpose_dy_kernel<<<p.R * cblocks, 256, 0, stream>>>(dy, plan.dyt, p.C, p.PH,
+                                                                         p.PW, cblocks);
       roialign::backward_tiled_kernel<<<static_cast<unsigned>(grid), BT::NT, 0, stream>>>(
-          dy, dx, plan.tile_offset, plan.tile_rois, plan.lists, plan.grid, plan.layout, p.C, p.H,
+          plan.dyt, dx, plan.tile_offset, plan.tile_rois, plan.lists, plan.grid, plan.layout, p.C, p.H,
           p.W, p.PH, p.PW, cblocks, jobs, assign ? 1 : 0);
       MOBULA_HIP_TRY(hipGetLastError());
       return;
