@@ -40,8 +40,9 @@ struct BwdTile {
   static constexpr int RS = TW + 2;              // row stride: dummy cell, 32 columns, dummy cell
   static constexpr int CS = TH * RS + 1;         // channel stride, odd
   static constexpr int PWB = 8;                  // pooled columns per dy register block
-  static constexpr int UB = 4;                   // pooled columns per scalar unit block (8 units)
-  static_assert(CS % 2 == 1, "channel stride must be odd");
+  static constexpr int UB = 4;                   // pooled columns per unit block (8 units)
+  static constexpr int G = 4;                    // work entries per group
+  static_assert(CS % 2 == 1 && TH == kTileRows, "layout");
 };
 
 // Host-side gate: the tiled backward kernel takes fixed sampling grids with
@@ -74,6 +75,22 @@ struct UnitBlock {
   }
 };
 
+// Eight column units fetched with broadcast LDS reads (same address in every
+// lane): the fields are uniform but live in vector registers.
+struct LdsUnitBlock {
+  AxisUnit u[8];
+  __device__ __forceinline__ int pos(int k) const { return u[k].pos; }
+  __device__ __forceinline__ float w0(int k) const { return u[k].w0; }
+  __device__ __forceinline__ float w1(int k) const { return u[k].w1; }
+};
+
+__device__ __forceinline__ LdsUnitBlock load_unit_block_lds(const AxisUnit* u) {
+  LdsUnitBlock b;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) b.u[k] = u[k];
+  return b;
+}
+
 __device__ __forceinline__ UnitBlock load_unit_block(const AxisUnit* __restrict__ u) {
   const int16v* p = reinterpret_cast<const int16v*>(u);
   UnitBlock b;
@@ -89,8 +106,8 @@ __device__ __forceinline__ UnitBlock load_unit_block(const AxisUnit* __restrict_
 // (or are dead and sit on dummy cells), so each such group issues all its
 // loads before its first store -- one LDS round trip per group.  LDS accesses
 // of a wavefront complete in program order, so the next group sees the stores.
-template <int G0, int NV, int ST>
-__device__ __forceinline__ void add_block_n(float* row, const float (&g)[8], const UnitBlock& u) {
+template <int G0, int NV, int ST, typename Block>
+__device__ __forceinline__ void add_block_n(float* row, const float (&g)[8], const Block& u) {
 #pragma unroll
   for (int p = 0; p < ST && p < 2 * NV; ++p) {
     float x[8], y[8];
@@ -104,8 +121,8 @@ __device__ __forceinline__ void add_block_n(float* row, const float (&g)[8], con
   }
 }
 
-template <int G0, int NV>
-__device__ __forceinline__ void add_block_s(float* row, const float (&g)[8], const UnitBlock& u, int lg) {
+template <int G0, int NV, typename Block>
+__device__ __forceinline__ void add_block_s(float* row, const float (&g)[8], const Block& u, int lg) {
   switch (lg) {
     case 0: add_block_n<G0, NV, 1>(row, g, u); break;
     case 1: add_block_n<G0, NV, 2>(row, g, u); break;
@@ -114,8 +131,8 @@ __device__ __forceinline__ void add_block_s(float* row, const float (&g)[8], con
   }
 }
 
-template <int G0>
-__device__ __forceinline__ void add_block(float* row, const float (&g)[8], const UnitBlock& u,
+template <int G0, typename Block>
+__device__ __forceinline__ void add_block(float* row, const float (&g)[8], const Block& u,
                                           int nv, int lg) {
   switch (nv) {
     case 4: add_block_s<G0, 4>(row, g, u, lg); break;
@@ -162,11 +179,13 @@ transpose_dy_kernel(const float* __restrict__ dy, float* __restrict__ dyt, int C
 
 __global__ void __launch_bounds__(BwdTile::NT)
 backward_tiled_kernel(const float* __restrict__ dyt, float* __restrict__ dx,
-                      const int* __restrict__ tile_offset, const int* __restrict__ tile_rois,
-                      const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll, int C, int H,
-                      int W, int PH, int PW, int cblocks, long long num_jobs, int assign) {
+                      const int* __restrict__ tile_offset, const WorkRange* __restrict__ ranges,
+                      const WorkEntry* __restrict__ entries, const AxisUnit* __restrict__ lists,
+                      TileGrid tg, ListLayout ll, int C, int H, int W, int PH, int PW, int cblocks,
+                      long long num_jobs, int assign) {
   using K = BwdTile;
   __shared__ float acc[K::CH * K::CS];
+  __shared__ AxisUnit ubuf[K::NW][K::G * 16];   // per wavefront: the column lists of one group
 
   // XCD-aware job order: consecutive workgroup ids go round-robin to the 8
   // XCDs, so give each XCD a contiguous run of logical jobs (neighbouring
@@ -206,91 +225,89 @@ backward_tiled_kernel(const float* __restrict__ dyt, float* __restrict__ dx,
   float* const row = acc + ch * K::CS + 1 + wave * K::RS;
   const float* const dy_lane = dyt + static_cast<size_t>(c0 + ch) * 8;   // dyt[r][ph][c][8]
   const size_t roi_dy_stride = static_cast<size_t>(PH) * C * 8, ph_dy_stride = static_cast<size_t>(C) * 8;
-  const AxisUnit* const row_lists = lists + static_cast<long long>(ty) * ll.row_stride;
   const AxisUnit* const col_lists =
       lists + static_cast<long long>(ll.ty) * ll.row_stride + static_cast<long long>(tx) * ll.col_stride;
-  const AxisUnit kDead = AxisUnit{0, -4, 0.0f, 0.0f};
 
-  // Software pipeline over the tile's ROI list, per wavefront:
-  //   stage 1 (ROI it+2): fetch row unit `lane` of its row list
-  //   stage 2 (ROI it+1): which sample rows land on my tile row?  fetch the dy
-  //                       row of the first of them
-  //   stage 3 (ROI it)  : fold all taps into g[pw], walk the column units
-  auto fetch_ru = [&](int it) -> AxisUnit {
-    if (it >= list_end || lane >= kRowSlots) return kDead;
-    return row_lists[static_cast<long long>(tile_rois[it]) * ll.roi_stride + lane];
-  };
-  auto mine_of = [&](const AxisUnit& ru) -> float {
-    return ru.pos == wave ? ru.w0 : ru.pos + 1 == wave ? ru.w1 : 0.0f;
-  };
+  // Each wavefront streams through the work list of its tile row: entries
+  // (ROI, pooled row, weight) in ROI order, four at a time.  Software pipeline:
+  //   entries of group k+2   scalar load in flight
+  //   group k+1              dy rows (two 16-byte loads per entry and lane) and the
+  //                          four column lists (one 16-byte load per lane) in flight
+  //   group k                fold the taps of a ROI into g[pw]; at its last entry
+  //                          walk the ROI's column units (staged through this
+  //                          wavefront's private LDS slot and read back as broadcasts)
   if (wave < rows) {
-    int roi_cur = tile_rois[list_begin];
-    int roi_nx = list_begin + 1 < list_end ? tile_rois[list_begin + 1] : roi_cur;
-    AxisUnit ru_cur = fetch_ru(list_begin), ru_nx = fetch_ru(list_begin + 1);
-    float w_cur = mine_of(ru_cur);
-    unsigned long long taps_cur = __ballot(w_cur != 0.0f);
-    float d_cur[8];
-    {
-      const int ph0 = __builtin_amdgcn_readlane(ru_cur.bin, taps_cur ? __builtin_ctzll(taps_cur) : 0);
-      load_dy_row(dy_lane + roi_cur * roi_dy_stride + ph0 * ph_dy_stride, d_cur);
-    }
-    for (int it = list_begin; it < list_end; ++it) {
-      // stage 1
-      const int roi_n2 = it + 2 < list_end ? tile_rois[it + 2] : roi_nx;
-      const AxisUnit ru_n2 =
-          (it + 2 < list_end && lane < kRowSlots)
-              ? row_lists[static_cast<long long>(roi_n2) * ll.roi_stride + lane] : kDead;
-      // stage 2
-      const float w_nx = mine_of(ru_nx);
-      const unsigned long long taps_nx = __ballot(w_nx != 0.0f);
-      float d_nx[8];
-      if (taps_nx != 0) {
-        const int ph0 = __builtin_amdgcn_readlane(ru_nx.bin, __builtin_ctzll(taps_nx));
-        load_dy_row(dy_lane + roi_nx * roi_dy_stride + ph0 * ph_dy_stride, d_nx);
-      }
-      // stage 3
-      if (taps_cur != 0) {
-        const AxisUnit* const cl = col_lists + static_cast<long long>(roi_cur) * ll.roi_stride;
-        const float* const dy_roi = dy_lane + roi_cur * roi_dy_stride;
-        const UnitBlock ub0 = load_unit_block(cl);
-        const int lg = (ub0.lo[0] >> kStrideShift) & kStrideMask;
-        for (int pwb = 0; pwb < PW; pwb += K::PWB) {
-          const int nb = min(K::PWB, PW - pwb);
-          const UnitBlock ub_a = pwb == 0 ? ub0 : load_unit_block(cl + 2 * pwb);
-          float g[8];
-          unsigned long long taps = taps_cur;
-          bool first = true;
-          while (taps != 0) {
-            const int i = __builtin_ctzll(taps);
-            taps &= taps - 1;
-            const int ph = __builtin_amdgcn_readlane(ru_cur.bin, i);
-            const float wy = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_cur), i));
-            float d[8];
-            if (first && pwb == 0) {
+    const WorkRange wr = ranges[tile * kTileRows + wave];
+    const int n = wr.count;
+    const int16v* const wl = reinterpret_cast<const int16v*>(entries + wr.begin);
+    AxisUnit* const my_units = ubuf[wave];
+    const int lane_list = lane >> 4, lane_unit = lane & 15;
+
+    auto issue = [&](const int16v& e, int e0, float (&d)[K::G][8], AxisUnit& uv) {
+      int my_roi = e[0];
 #pragma unroll
-              for (int k = 0; k < 8; ++k) d[k] = d_cur[k];
-            } else {
-              load_dy_row(dy_roi + ph * ph_dy_stride, d);
-            }
-#pragma unroll
-            for (int k = 0; k < 8; ++k) g[k] = first ? d[k] * wy : fmaf(d[k], wy, g[k]);
-            first = false;
-          }
-#ifdef LAB_NO_ADD
-          if (g[0] == 12345.f && g[3] == 3.f && g[6] == 1.f) row[ub_a.pos(0)] = g[1] + g[2] + g[4] + g[5] + g[7];
-          continue;
+      for (int j = 0; j < K::G; ++j) {
+#ifdef LAB_NO_DY
+        for (int k = 0; k < 8; ++k) d[j][k] = 1.0f + lane;
+#else
+        if (e0 + j < n) load_dy_row(dy_lane + e[4 * j] * roi_dy_stride + e[4 * j + 1] * ph_dy_stride, d[j]);
 #endif
-          if (lane < nch) {
-            add_block<0>(row, g, ub_a, min(nb, K::UB), lg);
-            if (nb > K::UB) add_block<4>(row, g, load_unit_block(cl + 2 * (pwb + K::UB)), nb - K::UB, lg);
+        my_roi = (lane_list == j && e0 + j < n) ? e[4 * j] : my_roi;
+      }
+#ifdef LAB_NO_UNITS
+      uv = AxisUnit{0, lane_unit, 0.5f, 0.5f};
+#else
+      uv = col_lists[static_cast<long long>(my_roi) * ll.roi_stride + lane_unit];
+#endif
+    };
+    float g[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    auto process = [&](const int16v& e, int e0, const float (&d)[K::G][8], const AxisUnit& uv) {
+      my_units[lane] = uv;
+#pragma unroll
+      for (int j = 0; j < K::G; ++j) {
+        if (e0 + j < n) {
+          const float wy = __int_as_float(e[4 * j + 2]);
+          const int fl = e[4 * j + 3];
+          if ((fl & 1) == 0) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) g[k] = d[j][k] * wy;
+          } else {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) g[k] = fmaf(d[j][k], wy, g[k]);
+          }
+          if ((fl & 2) != 0 && lane < nch) {
+            const AxisUnit* const ul = my_units + 16 * j;
+            const LdsUnitBlock ub_a = load_unit_block_lds(ul);
+            const int lg = (__builtin_amdgcn_readfirstlane(ub_a.u[0].bin) >> kStrideShift) & kStrideMask;
+#ifndef LAB_NO_ADD
+            add_block<0>(row, g, ub_a, min(PW, K::UB), lg);
+            if (PW > K::UB) add_block<4>(row, g, load_unit_block_lds(ul + 8), PW - K::UB, lg);
+#else
+            if (g[0] == 12345.f && g[3] == 3.f && g[6] == 1.f) row[ub_a.pos(0) + lg] = g[1] + g[2] + g[4] + g[5] + g[7];
+#endif
           }
         }
       }
-      // rotate
-      ru_cur = ru_nx; ru_nx = ru_n2; w_cur = w_nx; taps_cur = taps_nx;
-      roi_cur = roi_nx; roi_nx = roi_n2;
-#pragma unroll
-      for (int k = 0; k < 8; ++k) d_cur[k] = d_nx[k];
+    };
+
+    if (n > 0) {
+      int16v e_cur = wl[0], e_nx = wl[1], e_n2;
+      float d_a[K::G][8], d_b[K::G][8];
+      AxisUnit uv_a, uv_b;
+      issue(e_cur, 0, d_a, uv_a);
+      for (int e0 = 0; e0 < n; e0 += 2 * K::G) {
+        // group at e0 lives in set a, group at e0 + G in set b
+        e_n2 = wl[(e0 >> 2) + 2];
+        if (e0 + K::G < n) issue(e_nx, e0 + K::G, d_b, uv_b);
+        process(e_cur, e0, d_a, uv_a);
+        e_cur = e_nx; e_nx = e_n2;
+        if (e0 + K::G < n) {
+          e_n2 = wl[(e0 >> 2) + 3];
+          if (e0 + 2 * K::G < n) issue(e_nx, e0 + 2 * K::G, d_a, uv_a);
+          process(e_cur, e0 + K::G, d_b, uv_b);
+          e_cur = e_nx; e_nx = e_n2;
+        }
+      }
     }
   }
   __syncthreads();

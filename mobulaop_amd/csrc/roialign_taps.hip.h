@@ -14,9 +14,11 @@
 // The lists depend only on (ROI, tile row) and (ROI, tile column), so the
 // pre-pass writes them once to memory and every tile owner that needs them
 // reads them back:
-//   row list  of (roi, ty): kRowSlots units, slot = sample row index
-//                           ph*S + iy; weights already divided by the sample
-//                           count of the bin
+//   row taps  of (roi, ty): for each of the tile's rows the (pooled row, weight)
+//                           pairs that land on it, weights already divided by
+//                           the sample count of the bin: a 16-entry index
+//                           (start | count << 8) followed by the taps, sorted
+//                           by tile row, then by sample order
 //   col list  of (roi, tx): PW*2 units, slot = pw*2 + ix
 // Only fixed sampling grids with S <= 2 use this path.
 // Sample coordinates come from roialign_geometry.h (reference operation order).
@@ -39,12 +41,21 @@ constexpr int kNextOverlaps = 1 << 17;
 constexpr int kStrideShift = 18;
 constexpr int kStrideMask = 7;
 
-constexpr int kRowSlots = 32;   // PH * S <= 32
+constexpr int kRowSlots = 32;   // PH * S <= 32 sample rows per ROI
 constexpr int kMaxListPW = 16;  // PW <= 16, S <= 2
+constexpr int kTileRows = 16;   // rows of a tile (fixed by the row-tap index)
+
+struct RowTap { int ph; float wy; };
+// Row taps of one (roi, tile row): 32-byte index + up to 2*kRowSlots taps.
+struct alignas(16) RowTapTable {
+  unsigned short index[kTileRows];   // start | count << 8, per tile row
+  RowTap taps[2 * kRowSlots];
+};
+constexpr int kRowTableUnits = sizeof(RowTapTable) / 16;   // in 16-byte units
 
 struct ListLayout {
   int ty, tx;            // tiles per image
-  int row_stride;        // units per (roi, ty) row list   = kRowSlots
+  int row_stride;        // 16-byte units per (roi, ty) row-tap table
   int col_stride;        // units per (roi, tx) column list = 2 * PW
   long long roi_stride;  // units per ROI: ty*row_stride + tx*col_stride
 };
@@ -52,7 +63,7 @@ struct ListLayout {
 inline ListLayout make_list_layout(const TileGrid& tg, int PW) {
   ListLayout l;
   l.ty = tg.ty; l.tx = tg.tx;
-  l.row_stride = kRowSlots;
+  l.row_stride = kRowTableUnits;
   l.col_stride = 2 * PW;
   l.roi_stride = static_cast<long long>(l.ty) * l.row_stride + static_cast<long long>(l.tx) * l.col_stride;
   return l;
@@ -90,12 +101,25 @@ build_lists_kernel(const RoiRec* __restrict__ recs, int R, int PH, int PW, int S
   const float inv_count = 1.0f / rec.count;
   {
     const int ph = lane / S, iy = lane - ph * S;
-    const bool real = lane < PH * S;
     AxisSample a = axis_sample(sample_coord(rec.start_h, ph, rec.bin_h, iy, S), H);
-    a.valid = a.valid && real;
-    for (int ty = rec.row_lo / tg.th; ty <= rec.row_hi / tg.th; ++ty)
-      if (lane < kRowSlots)
-        base[ty * ll.row_stride + lane] = clip_unit(ph, a, ty * tg.th, tg.th, inv_count);
+    a.valid = a.valid && lane < PH * S;
+    for (int ty = rec.row_lo / tg.th; ty <= rec.row_hi / tg.th; ++ty) {
+      const AxisUnit u = clip_unit(ph, a, ty * tg.th, tg.th, inv_count);
+      RowTapTable* const table = reinterpret_cast<RowTapTable*>(base + ty * ll.row_stride);
+      // each unit lands on up to two tile rows; order the taps by row, then by lane
+      const int row0 = u.w0 != 0.0f ? u.pos : -1, row1 = u.w1 != 0.0f ? u.pos + 1 : -1;
+      int start = 0;
+      for (int r = 0; r < kTileRows; ++r) {
+        const unsigned long long m0 = __ballot(row0 == r), m1 = __ballot(row1 == r);
+        const unsigned long long below = (1ull << lane) - 1ull;
+        // a unit's high row is the next unit's low row: high parts first keeps sample order
+        const int n1 = __popcll(m1), n0 = __popcll(m0);
+        if (row1 == r) table->taps[start + __popcll(m1 & below)] = RowTap{ph, u.w1};
+        if (row0 == r) table->taps[start + n1 + __popcll(m0 & below)] = RowTap{ph, u.w0};
+        if (lane == 0) table->index[r] = static_cast<unsigned short>(start | ((n0 + n1) << 8));
+        start += n0 + n1;
+      }
+    }
   }
   {
     const int pw = lane / S, ix = lane - pw * S;
@@ -161,6 +185,70 @@ build_lists_kernel(const RoiRec* __restrict__ recs, int R, int PH, int PW, int S
         }
       }
     }
+  }
+}
+
+
+// One wavefront's share of a tile: the (ROI, pooled row, weight) taps that land
+// on one tile row, in ROI order, so that the owner of that row streams through
+// them without looking anything up.
+struct alignas(16) WorkEntry {
+  int roi;
+  int ph;
+  float wy;
+  int flags;   // bit 0: continues the previous entry's ROI; bit 1: last entry of its ROI
+};
+struct WorkRange { int begin; int count; };
+
+// One wavefront per (tile, tile row): lane j looks at ROI j of the tile's list,
+// takes its taps for this row from the row-tap table, and all lanes append
+// theirs in list order.  Space comes from a bump pointer (*cursor).
+__global__ void __launch_bounds__(256)
+build_worklists_kernel(const int* __restrict__ tile_offset, const int* __restrict__ tile_rois,
+                       const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll,
+                       int* __restrict__ cursor, WorkRange* __restrict__ ranges,
+                       WorkEntry* __restrict__ entries) {
+  const long long wid = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+  if (wid >= tg.total * kTileRows) return;
+  const int lane = threadIdx.x & 63;
+  const long long tile = wid / kTileRows;
+  const int row = static_cast<int>(wid % kTileRows);
+  const int ty = static_cast<int>(tile % tg.per_image) / tg.tx;
+  const int begin = tile_offset[tile], end = tile_offset[tile + 1];
+  auto table_of = [&](int roi) {
+    return reinterpret_cast<const RowTapTable*>(lists + static_cast<long long>(roi) * ll.roi_stride +
+                                                static_cast<long long>(ty) * ll.row_stride);
+  };
+  int total = 0;
+  for (int base = begin; base < end; base += 64) {
+    int c = 0;
+    if (base + lane < end) c = table_of(tile_rois[base + lane])->index[row] >> 8;
+    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
+    total += c;
+  }
+  int out = 0;
+  if (lane == 0 && total > 0) out = atomicAdd(cursor, total);
+  out = __shfl(out, 0);
+  if (lane == 0) ranges[wid] = WorkRange{out, total};
+  for (int base = begin; base < end; base += 64) {
+    int c = 0, roi = 0;
+    const RowTap* taps = nullptr;
+    if (base + lane < end) {
+      roi = tile_rois[base + lane];
+      const RowTapTable* tb = table_of(roi);
+      const unsigned idx = tb->index[row];
+      c = idx >> 8;
+      taps = tb->taps + (idx & 0xffu);
+    }
+    int incl = c;
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off);
+      if (lane >= off) incl += up;
+    }
+    WorkEntry* dst = entries + out + incl - c;
+    for (int q = 0; q < c; ++q)
+      dst[q] = WorkEntry{roi, taps[q].ph, taps[q].wy, (q > 0 ? 1 : 0) | (q == c - 1 ? 2 : 0)};
+    out += __shfl(incl, 63);
   }
 }
 

@@ -118,6 +118,9 @@ struct TilePlan {
   roialign::ListLayout layout;
   roialign::AxisUnit* lists;   // null unless requested
   float* dyt;                  // [R][PH][C][8] copy of dy, with the lists
+  int* cursor;                 // bump pointer of the work lists (zeroed with tile_count)
+  roialign::WorkRange* ranges; // per (tile, tile row)
+  roialign::WorkEntry* entries;
 };
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -143,15 +146,29 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   if (n_units > (1ll << 25)) return false;   // 512 MiB of sample lists: not worth it
   const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256) + 256;  // blocks are read whole
   const size_t b_dyt = with_lists ? align_up(sizeof(float) * 8 * p.R * p.PH * p.C, 256) : 0;
-  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list + b_units + b_dyt));
+  // work lists: every tap of every ROI once per tile column it spans
+  const long long n_entries =
+      with_lists ? static_cast<long long>(p.R) * 2 * p.PH * std::max(p.S, 1) * g.tx : 0;
+  if (n_entries > (1ll << 27)) return false;
+  const size_t b_ranges = with_lists ? align_up(sizeof(roialign::WorkRange) * g.total * roialign::kTileRows, 256) : 0;
+  const size_t b_entries = with_lists ? align_up(sizeof(roialign::WorkEntry) * n_entries, 256) + 512 : 0;
+  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list + b_units + b_dyt +
+                                                        b_ranges + b_entries + 256));
   if (failed()) return false;
-  plan->dyt = with_lists ? reinterpret_cast<float*>(base + b_recs + 2 * b_cnt + b_list + b_units) : nullptr;
-  plan->lists = with_lists ? reinterpret_cast<roialign::AxisUnit*>(base + b_recs + 2 * b_cnt + b_list)
-                           : nullptr;
   plan->recs = reinterpret_cast<roialign::RoiRec*>(base);
   plan->tile_count = reinterpret_cast<int*>(base + b_recs);
   plan->tile_offset = reinterpret_cast<int*>(base + b_recs + b_cnt);
   plan->tile_rois = reinterpret_cast<int*>(base + b_recs + 2 * b_cnt);
+  plan->cursor = plan->tile_count + g.total;   // spare slot of the zeroed counter array
+  plan->lists = with_lists ? reinterpret_cast<roialign::AxisUnit*>(base + b_recs + 2 * b_cnt + b_list)
+                           : nullptr;
+  char* cur = base + b_recs + 2 * b_cnt + b_list + b_units;
+  plan->dyt = with_lists ? reinterpret_cast<float*>(cur) : nullptr;
+  cur += b_dyt;
+  plan->ranges = reinterpret_cast<roialign::WorkRange*>(cur);
+  cur += b_ranges;
+  plan->entries = reinterpret_cast<roialign::WorkEntry*>(cur);
+  cur += b_entries;
   MOBULA_HIP_TRY(hipMemsetAsync(plan->tile_count, 0, sizeof(int) * (g.total + 1), stream));
   if (p.R > 0) {
     roialign::roi_prepare_kernel<<<(p.R + 255) / 256, 256, 0, stream>>>(
@@ -165,6 +182,12 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
     if (with_lists)
       roialign::build_lists_kernel<<<(p.R * 64 + 255) / 256, 256, 0, stream>>>(
           plan->recs, p.R, p.PH, p.PW, p.S, p.H, p.W, g, plan->layout, plan->lists);
+  }
+  if (with_lists) {
+    const long long threads = g.total * roialign::kTileRows * 64;
+    roialign::build_worklists_kernel<<<static_cast<int>((threads + 255) / 256), 256, 0, stream>>>(
+        plan->tile_offset, plan->tile_rois, plan->lists, g, plan->layout, plan->cursor,
+        plan->ranges, plan->entries);
   }
   MOBULA_HIP_TRY(hipGetLastError());
   return !failed();
@@ -187,8 +210,8 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
         roialign::transpose_dy_kernel<<<p.R * cblocks, 256, 0, stream>>>(dy, plan.dyt, p.C, p.PH,
                                                                          p.PW, cblocks);
       roialign::backward_tiled_kernel<<<static_cast<unsigned>(grid), BT::NT, 0, stream>>>(
-          plan.dyt, dx, plan.tile_offset, plan.tile_rois, plan.lists, plan.grid, plan.layout, p.C, p.H,
-          p.W, p.PH, p.PW, cblocks, jobs, assign ? 1 : 0);
+          plan.dyt, dx, plan.tile_offset, plan.ranges, plan.entries, plan.lists, plan.grid,
+          plan.layout, p.C, p.H, p.W, p.PH, p.PW, cblocks, jobs, assign ? 1 : 0);
       MOBULA_HIP_TRY(hipGetLastError());
       return;
     }
