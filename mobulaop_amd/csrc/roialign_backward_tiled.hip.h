@@ -145,35 +145,42 @@ __device__ __forceinline__ void add_block(float* row, const float (&g)[8], const
 // dy[r][c][ph][pw] -> dyt[r][ph][c][8] (pw padded to 8 with zeros, requires
 // PW <= 8): the form in which one lane per channel can fetch the PW values of
 // a pooled row with two 16-byte loads while the wavefront reads one
-// contiguous 2 KB segment.  One workgroup per (ROI, 64 channels).
+// contiguous 2 KB segment.  One workgroup per (ROI, 64 channels): the 64*PH*PW
+// input words are contiguous, and so are the 64*8 output words of each pooled
+// row.
 __global__ void __launch_bounds__(256)
 transpose_dy_kernel(const float* __restrict__ dy, float* __restrict__ dyt, int C, int PH, int PW,
                     int cblocks) {
-  __shared__ float buf[64 * 65];
+  extern __shared__ float tbuf[];   // [64][PH*PW]
   const int r = blockIdx.x / cblocks, cb = blockIdx.x % cblocks;
   const int c0 = cb * 64, nch = min(64, C - c0);
   const int bins = PH * PW;
   const float* src = dy + (static_cast<size_t>(r) * C + c0) * bins;
-  float* dst = dyt + static_cast<size_t>(r) * PH * C * 8;
-  for (int b0 = 0; b0 < bins; b0 += 64) {
-    const int nb = min(64, bins - b0);
-    __syncthreads();
-    for (int i = threadIdx.x; i < nch * nb; i += 256) {
-      const int c = i / nb, b = i - c * nb;
-      buf[c * 65 + b] = src[static_cast<size_t>(c) * bins + b0 + b];
+  const int n_in = nch * bins;
+  if ((reinterpret_cast<size_t>(src) & 15) == 0) {
+    for (int i = threadIdx.x * 4; i < n_in; i += 1024) {
+      if (i + 3 < n_in) {
+        const float4 v = *reinterpret_cast<const float4*>(src + i);
+        tbuf[i] = v.x; tbuf[i + 1] = v.y; tbuf[i + 2] = v.z; tbuf[i + 3] = v.w;
+      } else {
+        for (int k = i; k < n_in; ++k) tbuf[k] = src[k];
+      }
     }
-    __syncthreads();
-    // bins [b0, b0+nb) of every channel -> rows ph = bin / PW, slot k = bin % PW
-    for (int i = threadIdx.x; i < nch * nb; i += 256) {
-      const int b = i / nch, c = i - b * nch;
-      const int bin = b0 + b, ph = bin / PW, k = bin - ph * PW;
-      dst[(static_cast<size_t>(ph) * C + c0 + c) * 8 + k] = buf[c * 65 + b];
-    }
+  } else {
+    for (int i = threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
   }
-  // zero the padding slots
-  for (int i = threadIdx.x; i < PH * nch * (8 - PW); i += 256) {
-    const int k = PW + i % (8 - PW), c = (i / (8 - PW)) % nch, ph = i / ((8 - PW) * nch);
-    dst[(static_cast<size_t>(ph) * C + c0 + c) * 8 + k] = 0.0f;
+  __syncthreads();
+  // one float4 per thread and step: element e = ((ph * 64) + c) * 8 + k0, k0 in {0, 4}
+  for (int q = threadIdx.x; q < PH * 64 * 2; q += 256) {
+    const int k0 = (q & 1) * 4, c = (q >> 1) & 63, ph = q >> 7;
+    if (c >= nch) continue;
+    const float* in = tbuf + c * bins + ph * PW;
+    float4 v;
+    v.x = k0 + 0 < PW ? in[k0 + 0] : 0.0f;
+    v.y = k0 + 1 < PW ? in[k0 + 1] : 0.0f;
+    v.z = k0 + 2 < PW ? in[k0 + 2] : 0.0f;
+    v.w = k0 + 3 < PW ? in[k0 + 3] : 0.0f;
+    *reinterpret_cast<float4*>(dyt + ((static_cast<size_t>(r) * PH + ph) * C + c0 + c) * 8 + k0) = v;
   }
 }
 
@@ -247,18 +254,10 @@ backward_tiled_kernel(const float* __restrict__ dyt, float* __restrict__ dx,
       int my_roi = e[0];
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
-#ifdef LAB_NO_DY
-        for (int k = 0; k < 8; ++k) d[j][k] = 1.0f + lane;
-#else
         if (e0 + j < n) load_dy_row(dy_lane + e[4 * j] * roi_dy_stride + e[4 * j + 1] * ph_dy_stride, d[j]);
-#endif
         my_roi = (lane_list == j && e0 + j < n) ? e[4 * j] : my_roi;
       }
-#ifdef LAB_NO_UNITS
-      uv = AxisUnit{0, lane_unit, 0.5f, 0.5f};
-#else
       uv = col_lists[static_cast<long long>(my_roi) * ll.roi_stride + lane_unit];
-#endif
     };
     float g[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     auto process = [&](const int16v& e, int e0, const float (&d)[K::G][8], const AxisUnit& uv) {
@@ -279,12 +278,8 @@ backward_tiled_kernel(const float* __restrict__ dyt, float* __restrict__ dx,
             const AxisUnit* const ul = my_units + 16 * j;
             const LdsUnitBlock ub_a = load_unit_block_lds(ul);
             const int lg = (__builtin_amdgcn_readfirstlane(ub_a.u[0].bin) >> kStrideShift) & kStrideMask;
-#ifndef LAB_NO_ADD
             add_block<0>(row, g, ub_a, min(PW, K::UB), lg);
             if (PW > K::UB) add_block<4>(row, g, load_unit_block_lds(ul + 8), PW - K::UB, lg);
-#else
-            if (g[0] == 12345.f && g[3] == 3.f && g[6] == 1.f) row[ub_a.pos(0) + lg] = g[1] + g[2] + g[4] + g[5] + g[7];
-#endif
           }
         }
       }

@@ -200,19 +200,19 @@ struct alignas(16) WorkEntry {
 };
 struct WorkRange { int begin; int count; };
 
-// One wavefront per (tile, tile row): lane j looks at ROI j of the tile's list,
-// takes its taps for this row from the row-tap table, and all lanes append
-// theirs in list order.  Space comes from a bump pointer (*cursor).
-__global__ void __launch_bounds__(256)
+// One workgroup per tile, one wavefront per tile row: lane j looks at ROI j of
+// the tile's list, takes its taps for this row from the row-tap table, and all
+// lanes append theirs in list order.  Space for the tile's sixteen lists comes
+// from one bump-pointer allocation per tile (*cursor).
+__global__ void __launch_bounds__(kTileRows * 64)
 build_worklists_kernel(const int* __restrict__ tile_offset, const int* __restrict__ tile_rois,
                        const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll,
                        int* __restrict__ cursor, WorkRange* __restrict__ ranges,
                        WorkEntry* __restrict__ entries) {
-  const long long wid = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
-  if (wid >= tg.total * kTileRows) return;
-  const int lane = threadIdx.x & 63;
-  const long long tile = wid / kTileRows;
-  const int row = static_cast<int>(wid % kTileRows);
+  __shared__ int row_total[kTileRows];
+  __shared__ int tile_base;
+  const long long tile = blockIdx.x;
+  const int lane = threadIdx.x & 63, row = threadIdx.x >> 6;
   const int ty = static_cast<int>(tile % tg.per_image) / tg.tx;
   const int begin = tile_offset[tile], end = tile_offset[tile + 1];
   auto table_of = [&](int roi) {
@@ -226,10 +226,17 @@ build_worklists_kernel(const int* __restrict__ tile_offset, const int* __restric
     for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
     total += c;
   }
-  int out = 0;
-  if (lane == 0 && total > 0) out = atomicAdd(cursor, total);
-  out = __shfl(out, 0);
-  if (lane == 0) ranges[wid] = WorkRange{out, total};
+  if (lane == 0) row_total[row] = total;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int sum = 0;
+    for (int r = 0; r < kTileRows; ++r) sum += row_total[r];
+    tile_base = sum > 0 ? atomicAdd(cursor, sum) : 0;
+  }
+  __syncthreads();
+  int out = tile_base;
+  for (int r = 0; r < row; ++r) out += row_total[r];
+  if (lane == 0) ranges[tile * kTileRows + row] = WorkRange{out, total};
   for (int base = begin; base < end; base += 64) {
     int c = 0, roi = 0;
     const RowTap* taps = nullptr;

@@ -12,6 +12,7 @@
 #include "runtime.h"
 #include "roialign_naive.hip.h"
 #include "roialign_backward_tiled.hip.h"
+#include "roialign_forward_gather.hip.h"
 
 namespace {
 
@@ -100,9 +101,34 @@ int grid_for(long long n, int block) {
   return static_cast<int>(std::min<long long>((n + block - 1) / block, 256ll * 64));
 }
 
+bool use_tiled();
+
 template <typename T>
 void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipStream_t stream) {
   if (p.n_out == 0) return;
+  using FG = roialign::FwdGather;
+  const long long pixels = static_cast<long long>(p.H) * p.W;
+  const int cblocks = (p.C + FG::CH - 1) / FG::CH;
+  const long long blocks = static_cast<long long>(p.R) * cblocks;
+  if (use_tiled() && p.N > 0 && p.N < 65536 && blocks < (1ll << 31) && cblocks < 65536) {
+    // channel-last copy of the map, then the gather
+    T* xt = static_cast<T*>(mobula_hip::workspace(sizeof(T) * p.N * p.C * pixels));
+    if (failed()) return;
+    const dim3 tgrid(static_cast<unsigned>((pixels + 63) / 64), static_cast<unsigned>(cblocks),
+                     static_cast<unsigned>(p.N));
+    const bool vec = pixels % 4 == 0 && p.C % 4 == 0 &&
+                     (reinterpret_cast<size_t>(x) | reinterpret_cast<size_t>(xt)) % (4 * sizeof(T)) == 0;
+    if (vec)
+      roialign::transpose_to_channel_last_kernel<T, true><<<tgrid, 256, 0, stream>>>(
+          x, xt, p.C, static_cast<int>(pixels));
+    else
+      roialign::transpose_to_channel_last_kernel<T, false><<<tgrid, 256, 0, stream>>>(
+          x, xt, p.C, static_cast<int>(pixels));
+    roialign::forward_gather_kernel<T><<<static_cast<unsigned>(blocks), FG::NT, 0, stream>>>(
+        xt, rois, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblocks);
+    MOBULA_HIP_TRY(hipGetLastError());
+    return;
+  }
   roialign::forward_naive_kernel<T><<<grid_for(p.n_out, 256), 256, 0, stream>>>(
       p.n_out, x, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, rois, y, p.N);
   MOBULA_HIP_TRY(hipGetLastError());
@@ -183,12 +209,10 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
       roialign::build_lists_kernel<<<(p.R * 64 + 255) / 256, 256, 0, stream>>>(
           plan->recs, p.R, p.PH, p.PW, p.S, p.H, p.W, g, plan->layout, plan->lists);
   }
-  if (with_lists) {
-    const long long threads = g.total * roialign::kTileRows * 64;
-    roialign::build_worklists_kernel<<<static_cast<int>((threads + 255) / 256), 256, 0, stream>>>(
+  if (with_lists)
+    roialign::build_worklists_kernel<<<static_cast<unsigned>(g.total), roialign::kTileRows * 64, 0, stream>>>(
         plan->tile_offset, plan->tile_rois, plan->lists, g, plan->layout, plan->cursor,
         plan->ranges, plan->entries);
-  }
   MOBULA_HIP_TRY(hipGetLastError());
   return !failed();
 }
@@ -207,8 +231,8 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
     const long long grid = (jobs + 7) / 8 * 8;
     if (grid < (1ll << 31)) {
       if (p.R > 0)
-        roialign::transpose_dy_kernel<<<p.R * cblocks, 256, 0, stream>>>(dy, plan.dyt, p.C, p.PH,
-                                                                         p.PW, cblocks);
+        roialign::transpose_dy_kernel<<<p.R * cblocks, 256, sizeof(float) * 64 * p.PH * p.PW, stream>>>(
+            dy, plan.dyt, p.C, p.PH, p.PW, cblocks);
       roialign::backward_tiled_kernel<<<static_cast<unsigned>(grid), BT::NT, 0, stream>>>(
           plan.dyt, dx, plan.tile_offset, plan.ranges, plan.entries, plan.lists, plan.grid,
           plan.layout, p.C, p.H, p.W, p.PH, p.PW, cblocks, jobs, assign ? 1 : 0);
