@@ -1,0 +1,326 @@
+// Forward ROIAlign over a channel-blocked copy of the feature map.
+//
+// The map is first rewritten from NCHW to [N][C/32][H][W][32]: the 32 channels
+// of a block at one pixel are one 128-byte line.  A wavefront then computes
+// one (ROI, channel block): its 64 lanes are 8 pooled columns x 8 channel
+// quads, so a single 16-byte load per lane fetches one bilinear corner of
+// eight bins (1 KB), sixteen such loads are in flight per lane, and every lane
+// sums its own bin: no cross-lane traffic.  Row corners are the same for the
+// whole wavefront and live in scalar registers.
+// Channel block b is only ever read by XCD b % 8 and ROIs are visited in
+// spatial order, so what one L2 has to hold is a 128-byte-per-pixel slice of
+// the neighbourhood the XCD is currently working in.
+#pragma once
+#include <type_traits>
+#include "roialign_geometry.h"
+
+namespace roialign {
+
+struct FwdBlocked {
+  static constexpr int CB = 32;        // channels per block of the blocked layout
+  static constexpr int NW = 4;         // independent wavefronts per workgroup
+  static constexpr int MAXT = 128;     // row / column samples per ROI held in LDS
+  static constexpr int STAGE = 1600;   // staged outputs per wavefront
+  static constexpr int PWB = 8;        // pooled columns per step (one per group of 8 lanes)
+  static constexpr int CELL = 32;      // side of the sorting cells in pixels
+  static constexpr int MAXCELLS = 8192;
+};
+
+// Pooled rows staged per pass, 0 if the shape is not taken by this path.
+inline int blocked_rows_per_pass(int C, long long H, long long W, int PH, int PW, size_t elem) {
+  using K = FwdBlocked;
+  if (C % 4 != 0 || PW < 1 || K::CB * PW > K::STAGE) return 0;
+  if (H * W * K::CB * static_cast<long long>(elem) >= (1ll << 31)) return 0;
+  return min(PH, K::STAGE / (K::CB * PW));
+}
+
+// out[n][cb][p][32] = in[n][cb*32 + k][p]; channels past C are written as zero.
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256)
+transpose_to_blocked_kernel(const T* __restrict__ in, T* __restrict__ out, int C, int P) {
+  constexpr int CB = FwdBlocked::CB;
+  struct alignas(4 * sizeof(T)) V4 { T v[4]; };
+  __shared__ T tile[CB][65];
+  const int n = blockIdx.z, cb = blockIdx.y, cblk = gridDim.y;
+  const int p0 = blockIdx.x * 64, c0 = cb * CB;
+  const T* src = in + static_cast<size_t>(n) * C * P;
+  T* dst = out + (static_cast<size_t>(n) * cblk + cb) * P * CB;
+  if (VEC) {
+    const int q = threadIdx.x & 15, r = threadIdx.x >> 4;   // 16 quads of pixels, 16 channels per pass
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int c = c0 + r + 16 * k, p = p0 + 4 * q;
+      V4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v.v[i] = from_float<T>(0.0f);
+      if (c < C && p < P) v = *reinterpret_cast<const V4*>(src + static_cast<size_t>(c) * P + p);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) tile[r + 16 * k][4 * q + i] = v.v[i];
+    }
+  } else {
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int c = c0 + ty + 4 * k, p = p0 + tx;
+      tile[ty + 4 * k][tx] = (c < C && p < P) ? src[static_cast<size_t>(c) * P + p] : from_float<T>(0.0f);
+    }
+  }
+  __syncthreads();
+  const int cq = threadIdx.x & 7, pr = threadIdx.x >> 3;     // 8 channel quads, 32 pixels per pass
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int pl = pr + 32 * k;
+    if (p0 + pl < P) {
+      V4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v.v[i] = tile[4 * cq + i][pl];
+      *reinterpret_cast<V4*>(dst + static_cast<size_t>(p0 + pl) * CB + 4 * cq) = v;
+    }
+  }
+}
+
+// order[] = ROI indices sorted by (image, 32x32-pixel cell of the box centre,
+// rows of cells walked in alternating direction): consecutive wavefronts then
+// read neighbouring parts of the map.  One workgroup; counting sort with the
+// histogram in LDS.  ROIs that name no image sort last.
+__global__ void __launch_bounds__(1024)
+roi_order_kernel(const float* __restrict__ rois, int R, float scale, int H, int W,
+                 long long num_images, int* __restrict__ order) {
+  using K = FwdBlocked;
+  __shared__ int hist[K::MAXCELLS + 1];
+  __shared__ int wave_sum[16];
+  __shared__ int carry;
+  int cell = K::CELL;
+  long long cy = (H + cell - 1) / cell, cx = (W + cell - 1) / cell;
+  while (cy * cx * num_images > K::MAXCELLS && cell < (1 << 20)) {
+    cell *= 2;
+    cy = (H + cell - 1) / cell; cx = (W + cell - 1) / cell;
+  }
+  const int cells = cy * cx * num_images > K::MAXCELLS ? 1 : static_cast<int>(cy * cx * num_images);
+  auto key_of = [&](int r) {
+    const float* q = rois + static_cast<long long>(r) * 5;
+    const int b = static_cast<int>(q[0]);
+    if (b < 0 || b >= num_images) return cells;
+    if (cells == 1) return 0;
+    const float mx = 0.5f * (q[1] + q[3]) * scale, my = 0.5f * (q[2] + q[4]) * scale;
+    const int ix = min(max(static_cast<int>(mx), 0), W - 1) / cell;
+    const int iy = min(max(static_cast<int>(my), 0), H - 1) / cell;
+    const int sx = (iy & 1) ? static_cast<int>(cx) - 1 - ix : ix;
+    return static_cast<int>((b * cy + iy) * cx + sx);
+  };
+  for (int i = threadIdx.x; i <= cells; i += 1024) hist[i] = 0;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (int r = threadIdx.x; r < R; r += 1024) atomicAdd(&hist[key_of(r)], 1);
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int base = 0; base <= cells; base += 1024) {
+    const int i = base + threadIdx.x;
+    const int v = i <= cells ? hist[i] : 0;
+    int incl = v;
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off);
+      if (lane >= off) incl += up;
+    }
+    if (lane == 63) wave_sum[wave] = incl;
+    __syncthreads();
+    int before = carry;
+    for (int w = 0; w < wave; ++w) before += wave_sum[w];
+    if (i <= cells) hist[i] = before + incl - v;
+    __syncthreads();
+    if (threadIdx.x == 1023) carry = before + incl;
+    __syncthreads();
+  }
+  for (int r = threadIdx.x; r < R; r += 1024) order[atomicAdd(&hist[key_of(r)], 1)] = r;
+}
+
+// One row or column sample: byte offset of its low neighbour in a channel
+// block's plane (negative: the sample lies outside the map) and the weight of
+// the high neighbour; the low one weighs 1 - l.  The high neighbour is the next
+// row / column, or the same one at the far edge of the map (where l is 0).
+struct alignas(8) AxisEntry { int off; float l; };
+struct Corner { int off; float w; bool valid; };
+
+// Number of workgroups for R ROIs and cblk channel blocks (see the job decode
+// at the top of forward_blocked_kernel).
+inline long long blocked_grid(long long R, int cblk) {
+  using K = FwdBlocked;
+  long long per_xcd;
+  if (cblk >= 8) per_xcd = R * ((cblk + 7) / 8);
+  else per_xcd = (R + (8 / cblk) - 1) / (8 / cblk);
+  return 8 * ((per_xcd + K::NW - 1) / K::NW);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(FwdBlocked::NW * 64, 4)
+forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
+                       const int* __restrict__ order, T* __restrict__ y, float scale, int C, int H,
+                       int W, int PH, int PW, int S, long long num_images, int cblk,
+                       int rows_per_pass, int R) {
+  using K = FwdBlocked;
+  struct alignas(4 * sizeof(T)) V4 { T v[4]; };
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  __shared__ AxisEntry rows_s[K::NW][K::MAXT];
+  __shared__ AxisEntry cols_s[K::NW][K::MAXT];
+  __shared__ __attribute__((aligned(16))) T stage_s[K::NW][K::STAGE];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // Job decode.  Workgroups are dealt to the 8 XCDs round-robin, so blockIdx % 8
+  // names the XCD: it takes the channel blocks b with b % 8 == xcd and walks
+  // the sorted ROIs; with fewer than 8 blocks the ROIs of a block are split
+  // into 8 / cblk contiguous ranges instead.
+  const int xcd = blockIdx.x & 7;
+  const long long wi = static_cast<long long>(blockIdx.x >> 3) * K::NW + wave;
+  long long slot;
+  int cb;
+  if (cblk >= 8) {
+    const int nx = (cblk - xcd + 7) >> 3;
+    slot = wi / nx;
+    cb = xcd + 8 * static_cast<int>(wi % nx);
+  } else {
+    const int parts = 8 / cblk;
+    cb = xcd % cblk;
+    const int part = xcd / cblk;
+    const long long range = (R + parts - 1) / parts;
+    if (part >= parts || wi >= range) return;
+    slot = part * range + wi;
+  }
+  if (slot >= R) return;
+  const int roi = __builtin_amdgcn_readfirstlane(order[slot]);
+  const int c0 = cb * K::CB, nch = min(K::CB, C - c0);
+  const int grp = lane >> 3, quad = lane & 7;   // pooled column within a step, channel quad
+  const bool quad_on = 4 * quad < nch;
+  const RoiGeom g = roi_geometry(rois + static_cast<long long>(roi) * 5, scale, PH, PW, S);
+  const int bins = PH * PW;
+  const bool image_ok = g.batch >= 0 && g.batch < num_images;
+  const int n_cols = PW * g.grid_w, n_rows = PH * g.grid_h;
+  const bool tables = n_cols <= K::MAXT && n_rows <= K::MAXT;
+  AxisEntry* const rows = rows_s[wave];
+  AxisEntry* const cols = cols_s[wave];
+  T* const stage = stage_s[wave];
+  const int px_bytes = K::CB * static_cast<int>(sizeof(T)), row_bytes = W * px_bytes;
+
+  auto col_entry = [&](int pw, int ix) {
+    const AxisSample a = axis_sample(sample_coord(g.start_w, pw, g.bin_w, ix, g.grid_w), W);
+    return AxisEntry{a.valid ? a.low * px_bytes : -1, a.l};
+  };
+  auto row_entry = [&](int ph, int iy) {
+    const AxisSample a = axis_sample(sample_coord(g.start_h, ph, g.bin_h, iy, g.grid_h), H);
+    return AxisEntry{a.valid ? a.low * row_bytes : -1, a.l};
+  };
+  // low or high corner of a sample along one axis
+  auto corner = [](AxisEntry e, int hi, int stride, int last) {
+    Corner c;
+    c.valid = e.off >= 0;
+    c.off = hi ? e.off + (e.off < last ? stride : 0) : e.off;
+    c.w = hi ? e.l : 1.0f - e.l;
+    return c;
+  };
+  const int last_col = (W - 1) * px_bytes, last_row = (H - 1) * row_bytes;
+  if (image_ok && tables) {
+    for (int s = lane; s < n_cols; s += 64) cols[s] = col_entry(s / g.grid_w, s % g.grid_w);
+    for (int s = lane; s < n_rows; s += 64) rows[s] = row_entry(s / g.grid_h, s % g.grid_h);
+  }
+
+  const char* const base = reinterpret_cast<const char*>(xt) +
+      (static_cast<size_t>(image_ok ? g.batch : 0) * cblk + cb) * H * row_bytes;
+  const int lane_off = quad * 4 * static_cast<int>(sizeof(T));
+  auto uni_i = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  auto uni_f = [](float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); };
+  const int gh = uni_i(g.grid_h), gw = uni_i(g.grid_w);
+
+  for (int ph0 = 0; ph0 < PH; ph0 += rows_per_pass) {
+    const int rp = min(rows_per_pass, PH - ph0), seg = rp * PW;
+    for (int ph = ph0; ph < ph0 + rp; ++ph) {
+      for (int pwb = 0; pwb < PW; pwb += K::PWB) {
+        const int pw = pwb + grp;
+        const bool bin_on = pw < PW && quad_on;
+        const int pwc = min(pw, PW - 1);
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        // two row samples x two column samples = sixteen corners at a time
+        auto gather = [&](auto tables_tag) {
+          constexpr bool TAB = decltype(tables_tag)::value;
+          for (int iy0 = 0; iy0 < gh; iy0 += 2) {
+            Corner rc[4];
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+              const int iy = min(iy0 + a, gh - 1);
+              const AxisEntry e = TAB ? rows[ph * gh + iy] : row_entry(ph, iy);
+              const AxisEntry eu = AxisEntry{uni_i(e.off), uni_f(e.l)};
+#pragma unroll
+              for (int hi = 0; hi < 2; ++hi) {
+                rc[2 * a + hi] = corner(eu, hi, row_bytes, last_row);
+                rc[2 * a + hi].valid = rc[2 * a + hi].valid && iy0 + a < gh;
+              }
+            }
+            for (int ix0 = 0; ix0 < gw; ix0 += 2) {
+              Corner cc[4];
+#pragma unroll
+              for (int a = 0; a < 2; ++a) {
+                const int ix = min(ix0 + a, gw - 1);
+                const AxisEntry e = TAB ? cols[pwc * gw + ix] : col_entry(pwc, ix);
+#pragma unroll
+                for (int hi = 0; hi < 2; ++hi) {
+                  cc[2 * a + hi] = corner(e, hi, px_bytes, last_col);
+                  cc[2 * a + hi].valid = cc[2 * a + hi].valid && ix0 + a < gw && bin_on;
+                  cc[2 * a + hi].off += lane_off;
+                }
+              }
+              V4 v[4][4];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const char* const row_base = base + static_cast<unsigned>(rc[r].off);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+#pragma unroll
+                  for (int i = 0; i < 4; ++i) v[r][c].v[i] = from_float<T>(0.0f);
+                  if (rc[r].valid && cc[c].valid)
+                    v[r][c] = *reinterpret_cast<const V4*>(row_base + static_cast<unsigned>(cc[c].off));
+                }
+              }
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                  const float w = (rc[r].valid && cc[c].valid) ? rc[r].w * cc[c].w : 0.0f;
+#pragma unroll
+                  for (int i = 0; i < 4; ++i) acc[i] = fmaf(w, to_float(v[r][c].v[i]), acc[i]);
+                }
+            }
+          }
+        };
+        if (image_ok) {
+          if (tables) gather(std::true_type{});
+          else gather(std::false_type{});
+        }
+        if (bin_on) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            stage[(4 * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i] / g.count);
+        }
+      }
+    }
+    // the wavefront's outputs of this pass leave LDS in the order of y
+    const int total = nch * seg;
+    if (rp == PH) {
+      T* const dst = y + (static_cast<size_t>(roi) * C + c0) * bins;
+      constexpr int per = 16 / sizeof(T);
+      if (reinterpret_cast<size_t>(dst) % 16 == 0) {
+        const int nvec = total / per;
+        for (int i = lane; i < nvec; i += 64)
+          __builtin_nontemporal_store(reinterpret_cast<const u32x4*>(stage)[i], reinterpret_cast<u32x4*>(dst) + i);
+        for (int i = nvec * per + lane; i < total; i += 64) dst[i] = stage[i];
+      } else {
+        for (int i = lane; i < total; i += 64) dst[i] = stage[i];
+      }
+    } else {
+      for (int i = lane; i < total; i += 64) {
+        const int c = i / seg, j = i - c * seg;
+        y[(static_cast<size_t>(roi) * C + c0 + c) * bins + ph0 * PW + j] = stage[i];
+      }
+    }
+  }
+}
+
+}  // namespace roialign

@@ -12,7 +12,7 @@
 #include "runtime.h"
 #include "roialign_naive.hip.h"
 #include "roialign_backward_tiled.hip.h"
-#include "roialign_forward_gather.hip.h"
+#include "roialign_forward_blocked.hip.h"
 
 namespace {
 
@@ -106,41 +106,30 @@ bool use_tiled();
 template <typename T>
 void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipStream_t stream) {
   if (p.n_out == 0) return;
-  using FG = roialign::FwdGather;
+  using FB = roialign::FwdBlocked;
   const long long pixels = static_cast<long long>(p.H) * p.W;
-  const int cblocks = (p.C + FG::CH - 1) / FG::CH;
-  const long long blocks = static_cast<long long>(p.R) * cblocks;
-  if (use_tiled() && p.N > 0 && p.N < 65536 && blocks < (1ll << 31) && cblocks < 65536) {
-    // channel-last copy of the map, then the gather
-    const size_t xt_bytes = (sizeof(T) * p.N * p.C * pixels + 255) / 256 * 256;
+  const int cblk = (p.C + FB::CB - 1) / FB::CB;
+  const int rpp = roialign::blocked_rows_per_pass(p.C, p.H, p.W, p.PH, p.PW, sizeof(T));
+  const long long grid = roialign::blocked_grid(p.R, cblk);
+  if (use_tiled() && rpp > 0 && p.N > 0 && p.N < 65536 && cblk < 65536 && grid < (1ll << 31)) {
+    // channel-blocked copy of the map, spatial ROI order, then the gather
+    const size_t xt_bytes = (sizeof(T) * p.N * cblk * FB::CB * pixels + 255) / 256 * 256;
     char* const ws = static_cast<char*>(mobula_hip::workspace(xt_bytes + sizeof(int) * p.R));
     if (failed()) return;
     T* const xt = reinterpret_cast<T*>(ws);
     int* const order = reinterpret_cast<int*>(ws + xt_bytes);
-    const dim3 tgrid(static_cast<unsigned>((pixels + 63) / 64), static_cast<unsigned>(cblocks),
+    const dim3 tgrid(static_cast<unsigned>((pixels + 63) / 64), static_cast<unsigned>(cblk),
                      static_cast<unsigned>(p.N));
-    const bool vec = pixels % 4 == 0 && p.C % 4 == 0 &&
-                     (reinterpret_cast<size_t>(x) | reinterpret_cast<size_t>(xt)) % (4 * sizeof(T)) == 0;
+    const bool vec = pixels % 4 == 0 && reinterpret_cast<size_t>(x) % (4 * sizeof(T)) == 0;
     if (vec)
-      roialign::transpose_to_channel_last_kernel<T, true><<<tgrid, 256, 0, stream>>>(
+      roialign::transpose_to_blocked_kernel<T, true><<<tgrid, 256, 0, stream>>>(
           x, xt, p.C, static_cast<int>(pixels));
     else
-      roialign::transpose_to_channel_last_kernel<T, false><<<tgrid, 256, 0, stream>>>(
+      roialign::transpose_to_blocked_kernel<T, false><<<tgrid, 256, 0, stream>>>(
           x, xt, p.C, static_cast<int>(pixels));
-    using G4 = roialign::FwdGather4;
-    const int rpp = roialign::gather4_rows_per_pass(p.C, p.PH, p.PW);
-    const int cblocks4 = (p.C + G4::CW - 1) / G4::CW;
-    const long long jobs4 = static_cast<long long>(p.R) * cblocks4;
-    if (rpp > 0 && jobs4 + 8 < (1ll << 31)) {
-      const int tasks = rpp * ((p.PW + G4::PWB - 1) / G4::PWB);
-      const int nw = std::min(G4::MAXW, tasks);
-      roialign::roi_order_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
-      roialign::forward_gather4_kernel<T><<<static_cast<unsigned>((jobs4 + 7) / 8 * 8), nw * 64, 0, stream>>>(
-          xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblocks4, rpp, jobs4);
-    } else {
-      roialign::forward_gather_kernel<T><<<static_cast<unsigned>(blocks), FG::NT, 0, stream>>>(
-          xt, rois, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblocks);
-    }
+    roialign::roi_order_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
+    roialign::forward_blocked_kernel<T><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+        xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
     MOBULA_HIP_TRY(hipGetLastError());
     return;
   }
