@@ -11,7 +11,6 @@
 // spatial order, so what one L2 has to hold is a 128-byte-per-pixel slice of
 // the neighbourhood the XCD is currently working in.
 #pragma once
-#include <type_traits>
 #include "roialign_geometry.h"
 
 namespace roialign {
@@ -19,7 +18,8 @@ namespace roialign {
 struct FwdBlocked {
   static constexpr int CB = 32;        // channels per block of the blocked layout
   static constexpr int NW = 4;         // independent wavefronts per workgroup
-  static constexpr int MAXT = 128;     // row / column samples per ROI held in LDS
+  static constexpr int MAXT = 128;     // column samples held in LDS (16 for each of 8 pooled columns)
+  static constexpr int ROWT = 96;      // row samples held in LDS
   static constexpr int STAGE = 1600;   // staged outputs per wavefront
   static constexpr int PWB = 8;        // pooled columns per step (one per group of 8 lanes)
   static constexpr int CELL = 32;      // side of the sorting cells in pixels
@@ -134,12 +134,30 @@ roi_order_kernel(const float* __restrict__ rois, int R, float scale, int H, int 
   for (int r = threadIdx.x; r < R; r += 1024) order[atomicAdd(&hist[key_of(r)], 1)] = r;
 }
 
-// One row or column sample: byte offset of its low neighbour in a channel
-// block's plane (negative: the sample lies outside the map) and the weight of
-// the high neighbour; the low one weighs 1 - l.  The high neighbour is the next
-// row / column, or the same one at the far edge of the map (where l is 0).
-struct alignas(8) AxisEntry { int off; float l; };
-struct Corner { int off; float w; bool valid; };
+// A row sample: byte offsets of its low and high row in a channel block's
+// plane (lo negative: the sample lies outside the map) and their weights.
+struct alignas(16) RowEntry { int lo, hi; float wl, wh; };
+// A column sample, likewise, with the offsets in bytes along a row.
+struct alignas(16) ColEntry { int lo, hi; float wl, wh; };
+
+// Four consecutive elements (16 or 8 bytes) at byte offset lane_off + row_off of
+// a raw buffer; lane offsets outside the buffer read as zero without an access.
+__device__ __forceinline__ void buffer_load4(__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_off,
+                                             float (&out)[4]) {
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  const u32x4 raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off, row_off, 0);
+  out[0] = __uint_as_float(raw.x); out[1] = __uint_as_float(raw.y);
+  out[2] = __uint_as_float(raw.z); out[3] = __uint_as_float(raw.w);
+}
+__device__ __forceinline__ void buffer_load4(__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_off,
+                                             __half (&out)[4]) {
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_off, row_off, 0);
+  out[0] = __ushort_as_half(static_cast<unsigned short>(raw.x & 0xffffu));
+  out[1] = __ushort_as_half(static_cast<unsigned short>(raw.x >> 16));
+  out[2] = __ushort_as_half(static_cast<unsigned short>(raw.y & 0xffffu));
+  out[3] = __ushort_as_half(static_cast<unsigned short>(raw.y >> 16));
+}
 
 // Number of workgroups for R ROIs and cblk channel blocks (see the job decode
 // at the top of forward_blocked_kernel).
@@ -158,14 +176,16 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
                        int W, int PH, int PW, int S, long long num_images, int cblk,
                        int rows_per_pass, int R) {
   using K = FwdBlocked;
-  struct alignas(4 * sizeof(T)) V4 { T v[4]; };
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-  __shared__ AxisEntry rows_s[K::NW][K::MAXT];
-  __shared__ AxisEntry cols_s[K::NW][K::MAXT];
+  constexpr int CWIN = K::MAXT / K::PWB;   // column samples per pooled column held at a time
+  __shared__ RowEntry rows_s[K::NW][K::ROWT];
+  __shared__ ColEntry cols_s[K::NW][K::MAXT];
   __shared__ __attribute__((aligned(16))) T stage_s[K::NW][K::STAGE];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  auto uni_i = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  auto uni_f = [](float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); };
   // Job decode.  Workgroups are dealt to the 8 XCDs round-robin, so blockIdx % 8
   // names the XCD: it takes the channel blocks b with b % 8 == xcd and walks
   // the sorted ROIs; with fewer than 8 blocks the ROIs of a block are split
@@ -187,117 +207,159 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
     slot = part * range + wi;
   }
   if (slot >= R) return;
-  const int roi = __builtin_amdgcn_readfirstlane(order[slot]);
+  const int roi = uni_i(order[slot]);
   const int c0 = cb * K::CB, nch = min(K::CB, C - c0);
   const int grp = lane >> 3, quad = lane & 7;   // pooled column within a step, channel quad
   const bool quad_on = 4 * quad < nch;
   const RoiGeom g = roi_geometry(rois + static_cast<long long>(roi) * 5, scale, PH, PW, S);
   const int bins = PH * PW;
-  const bool image_ok = g.batch >= 0 && g.batch < num_images;
-  const int n_cols = PW * g.grid_w, n_rows = PH * g.grid_h;
-  const bool tables = n_cols <= K::MAXT && n_rows <= K::MAXT;
-  AxisEntry* const rows = rows_s[wave];
-  AxisEntry* const cols = cols_s[wave];
+  const int batch = uni_i(g.batch);
+  const bool image_ok = batch >= 0 && batch < num_images;
+  const int gh = uni_i(g.grid_h), gw = uni_i(g.grid_w);
+  const float count = uni_f(g.count);
+  // count is a power of two for the usual sampling ratios: multiply by its exact reciprocal
+  const bool pow2 = (gh & (gh - 1)) == 0 && (gw & (gw - 1)) == 0;
+  const float inv_count = 1.0f / count;
+  RowEntry* const rows = rows_s[wave];
+  ColEntry* const cols = cols_s[wave];
   T* const stage = stage_s[wave];
   const int px_bytes = K::CB * static_cast<int>(sizeof(T)), row_bytes = W * px_bytes;
-
-  auto col_entry = [&](int pw, int ix) {
-    const AxisSample a = axis_sample(sample_coord(g.start_w, pw, g.bin_w, ix, g.grid_w), W);
-    return AxisEntry{a.valid ? a.low * px_bytes : -1, a.l};
-  };
-  auto row_entry = [&](int ph, int iy) {
-    const AxisSample a = axis_sample(sample_coord(g.start_h, ph, g.bin_h, iy, g.grid_h), H);
-    return AxisEntry{a.valid ? a.low * row_bytes : -1, a.l};
-  };
-  // low or high corner of a sample along one axis
-  auto corner = [](AxisEntry e, int hi, int stride, int last) {
-    Corner c;
-    c.valid = e.off >= 0;
-    c.off = hi ? e.off + (e.off < last ? stride : 0) : e.off;
-    c.w = hi ? e.l : 1.0f - e.l;
-    return c;
-  };
-  const int last_col = (W - 1) * px_bytes, last_row = (H - 1) * row_bytes;
-  if (image_ok && tables) {
-    for (int s = lane; s < n_cols; s += 64) cols[s] = col_entry(s / g.grid_w, s % g.grid_w);
-    for (int s = lane; s < n_rows; s += 64) rows[s] = row_entry(s / g.grid_h, s % g.grid_h);
-  }
-
-  const char* const base = reinterpret_cast<const char*>(xt) +
-      (static_cast<size_t>(image_ok ? g.batch : 0) * cblk + cb) * H * row_bytes;
   const int lane_off = quad * 4 * static_cast<int>(sizeof(T));
-  auto uni_i = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
-  auto uni_f = [](float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); };
-  const int gh = uni_i(g.grid_h), gw = uni_i(g.grid_w);
+  constexpr int kDead = static_cast<int>(0x80000000u);
+
+  // The (image, channel block) plane as a raw buffer: a load whose lane offset
+  // is kDead falls outside it and returns zero.
+  const char* const plane_ptr = reinterpret_cast<const char*>(xt) +
+      (static_cast<size_t>(image_ok ? batch : 0) * cblk + cb) * H * row_bytes;
+  const __amdgpu_buffer_rsrc_t plane =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(plane_ptr), 0, H * row_bytes, 0x00020000);
+
+  // LDS holds a window of the row samples (flat index ph * gh + iy) and, for the
+  // current block of 8 pooled columns, a window of CWIN column samples each.
+  // Both are refilled by the whole wavefront when a step leaves the window;
+  // with the usual grids one fill per ROI covers everything.
+  int row_s0 = 0, row_s1 = 0;
+  auto need_rows = [&](int s, int n) {
+    if (s < row_s0 || s + n > row_s1) {
+      row_s0 = s;
+      row_s1 = min(s + K::ROWT, PH * gh);
+      for (int i = lane; i < row_s1 - row_s0; i += 64) {
+        const int f = row_s0 + i, ph = f / gh, iy = f - ph * gh;
+        const AxisSample a = axis_sample(sample_coord(g.start_h, ph, g.bin_h, iy, gh), H);
+        rows[i] = RowEntry{a.valid ? a.low * row_bytes : -1, a.high * row_bytes, a.h, a.l};
+      }
+    }
+  };
+  int col_pwb = -1, col_x0 = 0, col_x1 = 0;
+  auto need_cols = [&](int pwb, int ix, int n) {
+    if (pwb != col_pwb || ix < col_x0 || ix + n > col_x1) {
+      col_pwb = pwb; col_x0 = ix; col_x1 = min(ix + CWIN, gw);
+      for (int i = lane; i < K::MAXT; i += 64) {
+        const int pw = pwb + i / CWIN, x = col_x0 + i % CWIN;
+        if (pw < PW && x < col_x1) {
+          const AxisSample a = axis_sample(sample_coord(g.start_w, pw, g.bin_w, x, gw), W);
+          cols[i] = ColEntry{a.valid ? a.low * px_bytes : -1, a.high * px_bytes, a.h, a.l};
+        }
+      }
+    }
+  };
 
   for (int ph0 = 0; ph0 < PH; ph0 += rows_per_pass) {
     const int rp = min(rows_per_pass, PH - ph0), seg = rp * PW;
-    for (int ph = ph0; ph < ph0 + rp; ++ph) {
-      for (int pwb = 0; pwb < PW; pwb += K::PWB) {
-        const int pw = pwb + grp;
-        const bool bin_on = pw < PW && quad_on;
-        const int pwc = min(pw, PW - 1);
+    for (int pwb = 0; pwb < PW; pwb += K::PWB) {
+      const int pw = pwb + grp;
+      const bool bin_on = pw < PW && quad_on;
+#pragma nounroll
+      for (int ph = ph0; ph < ph0 + rp; ++ph) {
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        // two row samples x two column samples = sixteen corners at a time
-        auto gather = [&](auto tables_tag) {
-          constexpr bool TAB = decltype(tables_tag)::value;
+        if (image_ok) {
+#pragma nounroll
           for (int iy0 = 0; iy0 < gh; iy0 += 2) {
-            Corner rc[4];
+            // Row corners of samples iy0, iy0 + 1: the same for every lane, so they
+            // sit in scalar registers and steer uniform branches.
+            const int ny = min(2, gh - iy0);
+            need_rows(ph * gh + iy0, ny);
+            int roff[4];
+            float rw[4];
+            bool rlive[4];
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
-              const int iy = min(iy0 + a, gh - 1);
-              const AxisEntry e = TAB ? rows[ph * gh + iy] : row_entry(ph, iy);
-              const AxisEntry eu = AxisEntry{uni_i(e.off), uni_f(e.l)};
-#pragma unroll
-              for (int hi = 0; hi < 2; ++hi) {
-                rc[2 * a + hi] = corner(eu, hi, row_bytes, last_row);
-                rc[2 * a + hi].valid = rc[2 * a + hi].valid && iy0 + a < gh;
+              const RowEntry e = rows[ph * gh + iy0 + min(a, ny - 1) - row_s0];
+              roff[2 * a] = uni_i(e.lo); roff[2 * a + 1] = uni_i(e.hi);
+              rw[2 * a] = uni_f(e.wl); rw[2 * a + 1] = uni_f(e.wh);
+              rlive[2 * a] = rlive[2 * a + 1] = roff[2 * a] >= 0 && a < ny;
+            }
+            // samples less than a pixel apart share rows: fetch a shared row once
+            if (rlive[0] && rlive[2]) {
+              if (roff[2] == roff[0]) {
+                rw[0] += rw[2]; rw[1] += rw[3];
+                rlive[2] = rlive[3] = false;
+              } else if (roff[2] == roff[1]) {
+                rw[1] += rw[2];
+                rlive[2] = false;
               }
             }
+#pragma nounroll
             for (int ix0 = 0; ix0 < gw; ix0 += 2) {
-              Corner cc[4];
+              // Column corners of samples ix0, ix0 + 1 of this lane's pooled column.
+              // A corner that does not exist (outside the map, past the grid, no
+              // bin for this lane) or that repeats an earlier one is not loaded.
+              const int nx = min(2, gw - ix0);
+              need_cols(pwb, ix0, nx);
+              int coff[4];
+              float cw[4];
 #pragma unroll
               for (int a = 0; a < 2; ++a) {
-                const int ix = min(ix0 + a, gw - 1);
-                const AxisEntry e = TAB ? cols[pwc * gw + ix] : col_entry(pwc, ix);
-#pragma unroll
-                for (int hi = 0; hi < 2; ++hi) {
-                  cc[2 * a + hi] = corner(e, hi, px_bytes, last_col);
-                  cc[2 * a + hi].valid = cc[2 * a + hi].valid && ix0 + a < gw && bin_on;
-                  cc[2 * a + hi].off += lane_off;
-                }
+                const ColEntry e = cols[grp * CWIN + ix0 + min(a, nx - 1) - col_x0];
+                const bool ok = e.lo >= 0 && a < nx && bin_on;
+                coff[2 * a] = ok ? e.lo + lane_off : kDead;
+                coff[2 * a + 1] = ok ? e.hi + lane_off : kDead;
+                cw[2 * a] = ok ? e.wl : 0.0f;
+                cw[2 * a + 1] = ok ? e.wh : 0.0f;
               }
-              V4 v[4][4];
-#pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                const char* const row_base = base + static_cast<unsigned>(rc[r].off);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-#pragma unroll
-                  for (int i = 0; i < 4; ++i) v[r][c].v[i] = from_float<T>(0.0f);
-                  if (rc[r].valid && cc[c].valid)
-                    v[r][c] = *reinterpret_cast<const V4*>(row_base + static_cast<unsigned>(cc[c].off));
-                }
+              {
+                const bool both = coff[0] != kDead && coff[2] != kDead;
+                const bool same = both && coff[2] == coff[0];
+                const bool next = both && !same && coff[2] == coff[1];
+                cw[0] += same ? cw[2] : 0.0f;
+                cw[1] += same ? cw[3] : (next ? cw[2] : 0.0f);
+                if (same || next) { coff[2] = kDead; cw[2] = 0.0f; }
+                if (same) { coff[3] = kDead; cw[3] = 0.0f; }
               }
+              // sixteen corners: four rows (scalar) x four columns (per lane)
+              T v[4][4][4];
 #pragma unroll
               for (int r = 0; r < 4; ++r)
+                if (rlive[r]) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                  const float w = (rc[r].valid && cc[c].valid) ? rc[r].w * cc[c].w : 0.0f;
+                  for (int c = 0; c < 4; ++c) buffer_load4(plane, coff[c], roff[r], v[r][c]);
+                }
 #pragma unroll
-                  for (int i = 0; i < 4; ++i) acc[i] = fmaf(w, to_float(v[r][c].v[i]), acc[i]);
+              for (int r = 0; r < 4; ++r)
+                if (rlive[r]) {
+#pragma unroll
+                  for (int i = 0; i < 4; ++i) {
+                    float t = cw[0] * to_float(v[r][0][i]);
+#pragma unroll
+                    for (int c = 1; c < 4; ++c) t = fmaf(cw[c], to_float(v[r][c][i]), t);
+                    acc[i] = fmaf(rw[r], t, acc[i]);
+                  }
                 }
             }
           }
-        };
-        if (image_ok) {
-          if (tables) gather(std::true_type{});
-          else gather(std::false_type{});
+        }
+        if (pow2) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] *= inv_count;
+        } else {
+          asm volatile("" ::: "memory");   // keeps the division out of the common path
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] /= count;
         }
         if (bin_on) {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            stage[(4 * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i] / g.count);
+            stage[(4 * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i]);
         }
       }
     }
