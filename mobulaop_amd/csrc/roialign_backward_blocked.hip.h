@@ -1,0 +1,226 @@
+// Backward ROIAlign: tile owners accumulate in LDS, 16 bytes per lane.
+//
+// dx is cut into tiles of 16 rows x 56 columns x 32 channels.  One workgroup
+// owns one tile, keeps it in LDS as acc[row][column][channel] and is the only
+// writer of that piece of dx: no atomics anywhere and a summation order fixed
+// by the ROI order.  Wavefront w owns tile row w, so the sixteen wavefronts
+// never touch the same cell and need no barrier.  The 64 lanes of a wavefront
+// are 8 pooled columns x 8 channel quads: a lane folds the row taps of a ROI
+// into four gradients (its pooled column, its four channels) and adds them to
+// the two cells of each of its column samples with 16-byte LDS accesses.
+// Pooled columns whose cells may coincide are taken in separate turns (the
+// pre-pass stores the spacing at which they cannot).
+//
+// dy is read from a channel-blocked copy dyb[R][C/32][PH][PWp][32] (PWp = PW
+// rounded up to 8): one 16-byte load per lane fetches a pooled row (1 KB).
+#pragma once
+#include "roialign_taps.hip.h"
+
+namespace roialign {
+
+struct BwdBlocked {
+  static constexpr int TH = kTileRows;   // tile rows = wavefronts
+  static constexpr int TW = 56;          // tile columns
+  static constexpr int CB = 32;          // channels per workgroup
+  static constexpr int NW = TH;
+  static constexpr int NT = NW * 64;
+  static constexpr int CS = 36;          // floats per cell: 32 channels + 4 of padding (bank spread)
+  static constexpr int RS = TW + 2;      // cells per row: one dummy on either side
+  static constexpr int G = 4;            // work entries per pipeline stage
+  static constexpr int PWB = 8;          // pooled columns per turn (one per group of 8 lanes)
+};
+
+inline bool backward_blocked_supports(int PH, int PW, int S) { return lists_supported(PH, PW, S); }
+
+// dy[r][c][ph][pw] -> dyb[r][cb][ph][PWp][32], zero where pw >= PW or the channel
+// does not exist.  One workgroup per (ROI, channel block): the 32*PH*PW input
+// words are contiguous and so are the PH*PWp*32 output words.
+__global__ void __launch_bounds__(256)
+transpose_dy_blocked_kernel(const float* __restrict__ dy, float* __restrict__ dyb, int C, int PH,
+                            int PW, int PWp, int cblk) {
+  constexpr int CB = BwdBlocked::CB;
+  extern __shared__ float tbuf[];   // [32][PH*PW + 1]
+  const int r = blockIdx.x / cblk, cb = blockIdx.x % cblk;
+  const int c0 = cb * CB, nch = min(CB, C - c0);
+  const int bins = PH * PW, pitch = bins + 1;
+  const float* src = dy + (static_cast<size_t>(r) * C + c0) * bins;
+  for (int i = threadIdx.x; i < nch * bins; i += 256) {
+    const int c = i / bins;
+    tbuf[c * pitch + (i - c * bins)] = src[i];
+  }
+  __syncthreads();
+  float* dst = dyb + (static_cast<size_t>(r) * cblk + cb) * PH * PWp * CB;
+  const int quads = PH * PWp * (CB / 4);
+  for (int q = threadIdx.x; q < quads; q += 256) {
+    const int cq = q & 7, cell = q >> 3, pw = cell % PWp, ph = cell / PWp;
+    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (pw < PW) {
+      const float* in = tbuf + ph * PW + pw;
+      const int c = 4 * cq;
+      if (c + 0 < nch) v.x = in[(c + 0) * pitch];
+      if (c + 1 < nch) v.y = in[(c + 1) * pitch];
+      if (c + 2 < nch) v.z = in[(c + 2) * pitch];
+      if (c + 3 < nch) v.w = in[(c + 3) * pitch];
+    }
+    *reinterpret_cast<float4*>(dst + static_cast<size_t>(q) * 4) = v;
+  }
+}
+
+// Number of workgroups for `tiles` tiles and cblk channel blocks (job decode at
+// the top of backward_blocked_kernel).
+inline long long backward_blocked_grid(long long tiles, int cblk) {
+  long long per_xcd;
+  if (cblk >= 8) per_xcd = tiles * ((cblk + 7) / 8);
+  else per_xcd = (tiles + (8 / cblk) - 1) / (8 / cblk);
+  return 8 * per_xcd;
+}
+
+typedef int int16v __attribute__((ext_vector_type(16)));
+
+__global__ void __launch_bounds__(BwdBlocked::NT)
+backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
+                        const WorkRange* __restrict__ ranges, const WorkEntry* __restrict__ entries,
+                        const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll, int C, int H,
+                        int W, int PH, int PW, int S, int cblk, int assign) {
+  using K = BwdBlocked;
+  __shared__ __attribute__((aligned(16))) float acc[K::TH * K::RS * K::CS];
+
+  // Job decode.  Workgroups are dealt to the 8 XCDs round-robin, so blockIdx % 8
+  // names the XCD: it takes the channel blocks b with b % 8 == xcd (their slice
+  // of dyb then stays in that XCD's L2) and walks the tiles in order; with
+  // fewer than 8 blocks the tiles of a block are split into 8 / cblk ranges.
+  const int xcd = blockIdx.x & 7;
+  const long long wi = blockIdx.x >> 3;
+  long long tile;
+  int cb;
+  if (cblk >= 8) {
+    const int nx = (cblk - xcd + 7) >> 3;
+    tile = wi / nx;
+    cb = xcd + 8 * static_cast<int>(wi % nx);
+  } else {
+    const int parts = 8 / cblk;
+    cb = xcd % cblk;
+    const int part = xcd / cblk;
+    const long long range = (tg.total + parts - 1) / parts;
+    if (part >= parts || wi >= range) return;
+    tile = part * range + wi;
+  }
+  if (tile >= tg.total) return;
+  const int n = static_cast<int>(tile / tg.per_image);
+  const int t_in_img = static_cast<int>(tile % tg.per_image);
+  const int ty = t_in_img / tg.tx, tx = t_in_img % tg.tx;
+  const int r0 = ty * K::TH, q0 = tx * K::TW;
+  const int c0 = cb * K::CB, nch = min(K::CB, C - c0);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // = the tile row owned
+  const int rows = min(K::TH, H - r0), cols = min(K::TW, W - q0);
+  if (wave >= rows) return;   // no barrier below: rows are independent
+  const int grp = lane >> 3, quad = lane & 7;   // pooled column within a turn, channel quad
+
+  float* const row = acc + wave * (K::RS * K::CS);
+  for (int i = lane; i < K::RS * K::CS / 4; i += 64)
+    reinterpret_cast<float4*>(row)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+
+  const WorkRange wr = ranges[tile * kTileRows + wave];
+  const int n_entries = wr.count;
+  const int16v* const wl = reinterpret_cast<const int16v*>(entries + wr.begin);
+  const int PWp = ll.col_stride;
+  const size_t dy_ph = static_cast<size_t>(PWp) * K::CB, dy_roi = dy_ph * PH * cblk;
+  float* const cell0 = row + quad * 4;   // this lane's four channels of cell 0 (the left dummy)
+
+  // Each wavefront streams through the work list of its tile row: entries
+  // (ROI, pooled row, weight) in ROI order, four at a time, double buffered:
+  // while the taps of one group are folded and added, the dy rows and column
+  // samples of the next are in flight.
+  for (int pwb = 0; pwb < PW; pwb += K::PWB) {
+    const float* const dy_lane = dyb + static_cast<size_t>(cb) * dy_ph * PH + pwb * K::CB + lane * 4;
+    const AxisUnit* const col_lane = lists + static_cast<long long>(ll.ty) * ll.row_stride +
+                                     static_cast<long long>(tx) * ll.col_stride + pwb + grp;
+    auto issue = [&](const int16v& e, int e0, float4 (&d)[K::G], int4 (&u)[K::G]) {
+#pragma unroll
+      for (int j = 0; j < K::G; ++j) {
+        if (e0 + j < n_entries) {
+          d[j] = *reinterpret_cast<const float4*>(dy_lane + e[4 * j] * dy_roi + e[4 * j + 1] * dy_ph);
+          if ((e[4 * j + 3] & 2) != 0)
+            u[j] = *reinterpret_cast<const int4*>(col_lane + static_cast<long long>(e[4 * j]) * ll.roi_stride);
+        }
+      }
+    };
+    float g[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    // adds g * (weights of the two cells) to the cells pos, pos + 1 of the row
+    auto add_sample = [&](int pos, float wlo, float whi) {
+      float* const a = cell0 + pos * K::CS;
+      float4 lo = *reinterpret_cast<const float4*>(a);
+      float4 hi = *reinterpret_cast<const float4*>(a + K::CS);
+      lo.x = fmaf(g[0], wlo, lo.x); lo.y = fmaf(g[1], wlo, lo.y);
+      lo.z = fmaf(g[2], wlo, lo.z); lo.w = fmaf(g[3], wlo, lo.w);
+      hi.x = fmaf(g[0], whi, hi.x); hi.y = fmaf(g[1], whi, hi.y);
+      hi.z = fmaf(g[2], whi, hi.z); hi.w = fmaf(g[3], whi, hi.w);
+      *reinterpret_cast<float4*>(a) = lo;
+      *reinterpret_cast<float4*>(a + K::CS) = hi;
+    };
+    auto process = [&](const int16v& e, int e0, const float4 (&d)[K::G], const int4 (&u)[K::G]) {
+#pragma unroll
+      for (int j = 0; j < K::G; ++j) {
+        if (e0 + j < n_entries) {
+          const float wy = __int_as_float(e[4 * j + 2]);
+          const int fl = e[4 * j + 3];
+          if ((fl & 1) == 0) {
+            g[0] = d[j].x * wy; g[1] = d[j].y * wy; g[2] = d[j].z * wy; g[3] = d[j].w * wy;
+          } else {
+            g[0] = fmaf(d[j].x, wy, g[0]); g[1] = fmaf(d[j].y, wy, g[1]);
+            g[2] = fmaf(d[j].z, wy, g[2]); g[3] = fmaf(d[j].w, wy, g[3]);
+          }
+          if ((fl & 2) != 0) {
+            // last tap of this ROI on this row: spread g over the column samples
+            const int cf = u[j].y;
+            const int pos0 = u[j].x & 0xffff, pos1 = static_cast<unsigned>(u[j].x) >> 16;
+            const float l0 = __int_as_float(u[j].z), l1 = __int_as_float(u[j].w);
+            const int lg = (__builtin_amdgcn_readfirstlane(cf) >> kColStrideShift) & kColStrideMask;
+            const int turns = min(K::PWB, max(1, (1 << lg) / S));
+            for (int t = 0; t < turns; ++t) {
+              if ((grp & (turns - 1)) == t) {
+                if ((cf & 3) != 0) add_sample(pos0, (cf & 1) ? 1.0f - l0 : 0.0f, (cf & 2) ? l0 : 0.0f);
+                if ((cf & 12) != 0) add_sample(pos1, (cf & 4) ? 1.0f - l1 : 0.0f, (cf & 8) ? l1 : 0.0f);
+              }
+            }
+          }
+        }
+      }
+    };
+
+    if (n_entries > 0) {
+      int16v e_cur = wl[0], e_nx = wl[1], e_n2;
+      float4 d_a[K::G], d_b[K::G];
+      int4 u_a[K::G], u_b[K::G];
+      issue(e_cur, 0, d_a, u_a);
+      for (int e0 = 0; e0 < n_entries; e0 += 2 * K::G) {
+        // group at e0 lives in set a, group at e0 + G in set b
+        e_n2 = wl[(e0 >> 2) + 2];
+        if (e0 + K::G < n_entries) issue(e_nx, e0 + K::G, d_b, u_b);
+        process(e_cur, e0, d_a, u_a);
+        e_cur = e_nx; e_nx = e_n2;
+        if (e0 + K::G < n_entries) {
+          e_n2 = wl[(e0 >> 2) + 3];
+          if (e0 + 2 * K::G < n_entries) issue(e_nx, e0 + 2 * K::G, d_a, u_a);
+          process(e_cur, e0 + K::G, d_b, u_b);
+          e_cur = e_nx; e_nx = e_n2;
+        }
+      }
+    }
+  }
+
+  // The owner writes its row: one channel plane at a time, lanes along x.
+  float* const out = dx + ((static_cast<size_t>(n) * C + c0) * H + r0 + wave) * W + q0;
+  const size_t plane = static_cast<size_t>(H) * W;
+  if (lane < cols) {
+    const float* const src = row + (lane + 1) * K::CS;
+    if (assign) {
+      for (int c = 0; c < nch; ++c) out[c * plane + lane] = src[c];
+    } else {
+      for (int c = 0; c < nch; ++c) out[c * plane + lane] += src[c];
+    }
+  }
+}
+
+}  // namespace roialign

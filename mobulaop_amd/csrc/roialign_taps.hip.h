@@ -19,7 +19,8 @@
 //                           the sample count of the bin: a 16-entry index
 //                           (start | count << 8) followed by the taps, sorted
 //                           by tile row, then by sample order
-//   col list  of (roi, tx): PW*2 units, slot = pw*2 + ix
+//   col list  of (roi, tx): one 16-byte ColPair per pooled column (padded to a
+//                           multiple of 8 columns): its one or two sample columns
 // Only fixed sampling grids with S <= 2 use this path.
 // Sample coordinates come from roialign_geometry.h (reference operation order).
 #pragma once
@@ -30,16 +31,19 @@ namespace roialign {
 // `bin` is the pooled row/column; `pos` the local position of the low corner.
 struct alignas(16) AxisUnit { int bin; int pos; float w0, w1; };
 
-// Bit 16 of `bin` of the first column unit of a pooled column: the cells of
-// its two units overlap.  Bit 17: this pooled column's cells overlap the next
-// pooled column's.
-// Bits 18..20 of `bin` of slot 0 of a column list: log2 of the smallest power
-// of two s such that units k and k+s of the list never share a cell.  Units
-// k, k+s, k+2s, ... can then be processed together (loads before stores).
-constexpr int kPairOverlaps = 1 << 16;
-constexpr int kNextOverlaps = 1 << 17;
-constexpr int kStrideShift = 18;
-constexpr int kStrideMask = 7;
+// The sample columns of one pooled column inside one tile column band.
+//   cells  (pos0 + 1) | (pos1 + 1) << 16: index of the low corner's cell in a tile
+//          row whose cell 0 is a dummy to the left of the tile (so a low corner
+//          one column left of the tile is cell 0, its high corner cell 1)
+//   flags  bit 0/1: low/high corner of sample 0 lies in the tile and has a
+//          non-zero weight; bit 2/3: same for sample 1; bits 8..10: log2 of the
+//          smallest power-of-two distance (in sample columns) at which two
+//          samples of this list never share a cell: pooled columns that far
+//          apart can be added concurrently
+//   l0/l1  weight of the high corner; the low corner weighs 1 - l
+struct alignas(16) ColPair { int cells; int flags; float l0, l1; };
+constexpr int kColStrideShift = 8;
+constexpr int kColStrideMask = 7;
 
 constexpr int kRowSlots = 32;   // PH * S <= 32 sample rows per ROI
 constexpr int kMaxListPW = 16;  // PW <= 16, S <= 2
@@ -56,7 +60,7 @@ constexpr int kRowTableUnits = sizeof(RowTapTable) / 16;   // in 16-byte units
 struct ListLayout {
   int ty, tx;            // tiles per image
   int row_stride;        // 16-byte units per (roi, ty) row-tap table
-  int col_stride;        // units per (roi, tx) column list = 2 * PW
+  int col_stride;        // 16-byte units per (roi, tx) column list: PW rounded up to 8
   long long roi_stride;  // units per ROI: ty*row_stride + tx*col_stride
 };
 
@@ -64,7 +68,7 @@ inline ListLayout make_list_layout(const TileGrid& tg, int PW) {
   ListLayout l;
   l.ty = tg.ty; l.tx = tg.tx;
   l.row_stride = kRowTableUnits;
-  l.col_stride = 2 * PW;
+  l.col_stride = (PW + 7) / 8 * 8;
   l.roi_stride = static_cast<long long>(l.ty) * l.row_stride + static_cast<long long>(l.tx) * l.col_stride;
   return l;
 }
@@ -122,68 +126,39 @@ build_lists_kernel(const RoiRec* __restrict__ recs, int R, int PH, int PW, int S
     }
   }
   {
+    // lane = sample column pw * S + ix
     const int pw = lane / S, ix = lane - pw * S;
     const bool real = lane < PW * S;
     AxisSample a = axis_sample(sample_coord(rec.start_w, pw, rec.bin_w, ix, S), W);
     a.valid = a.valid && real;
-    AxisUnit* const cols = base + static_cast<long long>(ll.ty) * ll.row_stride;
+    ColPair* const cols = reinterpret_cast<ColPair*>(base + static_cast<long long>(ll.ty) * ll.row_stride);
     for (int tx = rec.col_lo / tg.tw; tx <= rec.col_hi / tg.tw; ++tx) {
-      AxisUnit u = clip_unit(pw, a, tx * tg.tw, tg.tw, 1.0f);
-      const bool live = u.w0 != 0.0f || u.w1 != 0.0f;
-      // neighbours: the other unit of this pooled column, the units of the next one
-      const int pos_next = __shfl_down(u.pos, 1), pos_next2 = __shfl_down(u.pos, 2);
-      const bool live_next = __shfl_down(live ? 1 : 0, 1) != 0;
-      const bool live_next2 = __shfl_down(live ? 1 : 0, 2) != 0;
-      auto near = [](int p, int q) { return p - q >= -1 && p - q <= 1; };
-      if (S == 2) {
-        // lane = 2*pw + ix.  Flags live in the ix == 0 unit.
-        const bool pair = live && live_next && near(u.pos, pos_next);
-        // this column's units vs the next column's two units
-        const int pos_next3 = __shfl_down(u.pos, 3);
-        const bool live_next3 = __shfl_down(live ? 1 : 0, 3) != 0;
-        bool next = false;
-        if (ix == 0) {
-          next = (live && live_next2 && near(u.pos, pos_next2)) ||
-                 (live && live_next3 && near(u.pos, pos_next3)) ||
-                 (live_next && live_next2 && near(pos_next, pos_next2)) ||
-                 (live_next && live_next3 && near(pos_next, pos_next3));
-          if (pair) u.bin |= kPairOverlaps;
-          if (next) u.bin |= kNextOverlaps;
-        }
-        {
-          // smallest power-of-two stride at which no two live units share a cell
-          int lg = 0;
+      int pos = a.low - tx * tg.tw;
+      const bool lo_in = a.valid && pos >= 0 && pos < tg.tw && a.h != 0.0f;
+      const bool hi_in = a.valid && a.high != a.low && pos + 1 >= 0 && pos + 1 < tg.tw && a.l != 0.0f;
+      const bool live = lo_in || hi_in;
+      if (!live) pos = -1;
+      // smallest power-of-two distance at which no two live samples share a cell
+      int lg = 0;
 #pragma unroll
-          for (int d = 1; d <= 16; d <<= 1) {
-            const int pos_d = __shfl_down(u.pos, d);
-            const bool live_d = __shfl_down(live ? 1 : 0, d) != 0;
-            const bool clash = live && live_d && lane + d < PW * S && near(u.pos, pos_d);
-            if (__ballot(clash) != 0) lg = (d == 16) ? 5 : __builtin_ctz(d) + 1;
-          }
-          if (lane == 0) u.bin |= lg << kStrideShift;
-        }
-        if (real) cols[tx * ll.col_stride + lane] = u;
-      } else {
-        // S == 1: slot 2*pw holds the unit, slot 2*pw + 1 is dead
-        const bool next = live && live_next && near(u.pos, pos_next);
-        if (next) u.bin |= kNextOverlaps;
-        {
-          int lg = 0;
-#pragma unroll
-          for (int d = 1; d <= 16; d <<= 1) {
-            const int pos_d = __shfl_down(u.pos, d);
-            const bool live_d = __shfl_down(live ? 1 : 0, d) != 0;
-            const bool clash = live && live_d && lane + d < PW && near(u.pos, pos_d);
-            // slots are 2 apart for S == 1
-            if (__ballot(clash) != 0) lg = (d == 16) ? 5 : __builtin_ctz(d) + 2;
-          }
-          if (lane == 0) u.bin |= min(lg, 5) << kStrideShift;
-        }
-        if (real) {
-          cols[tx * ll.col_stride + 2 * lane] = u;
-          cols[tx * ll.col_stride + 2 * lane + 1] = AxisUnit{pw, tg.tw, 0.0f, 0.0f};
-        }
+      for (int d = 1; d <= 16; d <<= 1) {
+        const int pos_d = __shfl_down(pos, d);
+        const bool live_d = __shfl_down(live ? 1 : 0, d) != 0;
+        const bool clash = live && live_d && lane + d < PW * S && pos_d - pos >= -1 && pos_d - pos <= 1;
+        if (__ballot(clash) != 0) lg = (d == 16) ? 5 : __builtin_ctz(d) + 1;
       }
+      const int fl = (lo_in ? 1 : 0) | (hi_in ? 2 : 0);
+      const int pos_n = __shfl_down(pos, 1), fl_n = __shfl_down(fl, 1);
+      const float l_n = __shfl_down(a.l, 1);
+      ColPair cp;
+      cp.cells = (pos + 1) | ((S == 2 ? pos_n + 1 : 0) << 16);
+      cp.flags = fl | ((S == 2 ? fl_n : 0) << 2) | (lg << kColStrideShift);
+      cp.l0 = a.l;
+      cp.l1 = S == 2 ? l_n : 0.0f;
+      if (real && ix == 0) cols[tx * ll.col_stride + pw] = cp;
+      // padding columns: nothing to add, same spacing
+      if (lane < ll.col_stride - PW)
+        cols[tx * ll.col_stride + PW + lane] = ColPair{0, lg << kColStrideShift, 0.0f, 0.0f};
     }
   }
 }

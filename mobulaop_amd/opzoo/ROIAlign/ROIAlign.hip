@@ -11,7 +11,7 @@
 
 #include "runtime.h"
 #include "roialign_naive.hip.h"
-#include "roialign_backward_tiled.hip.h"
+#include "roialign_backward_blocked.hip.h"
 #include "roialign_forward_blocked.hip.h"
 
 namespace {
@@ -147,7 +147,7 @@ struct TilePlan {
   int* tile_rois;
   roialign::ListLayout layout;
   roialign::AxisUnit* lists;   // null unless requested
-  float* dyt;                  // [R][PH][C][8] copy of dy, with the lists
+  float* dyb;                  // channel-blocked copy of dy, with the lists
   int* cursor;                 // bump pointer of the work lists (zeroed with tile_count)
   roialign::WorkRange* ranges; // per (tile, tile row)
   roialign::WorkEntry* entries;
@@ -175,7 +175,8 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   const long long n_units = with_lists ? plan->layout.roi_stride * p.R : 0;
   if (n_units > (1ll << 25)) return false;   // 512 MiB of sample lists: not worth it
   const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256) + 256;  // blocks are read whole
-  const size_t b_dyt = with_lists ? align_up(sizeof(float) * 8 * p.R * p.PH * p.C, 256) : 0;
+  const int cblk = (p.C + 31) / 32;
+  const size_t b_dyt = with_lists ? align_up(sizeof(float) * 32 * plan->layout.col_stride * p.R * p.PH * cblk, 256) : 0;
   // work lists: every tap of every ROI once per tile column it spans
   const long long n_entries =
       with_lists ? static_cast<long long>(p.R) * 2 * p.PH * std::max(p.S, 1) * g.tx : 0;
@@ -193,7 +194,7 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   plan->lists = with_lists ? reinterpret_cast<roialign::AxisUnit*>(base + b_recs + 2 * b_cnt + b_list)
                            : nullptr;
   char* cur = base + b_recs + 2 * b_cnt + b_list + b_units;
-  plan->dyt = with_lists ? reinterpret_cast<float*>(cur) : nullptr;
+  plan->dyb = with_lists ? reinterpret_cast<float*>(cur) : nullptr;
   cur += b_dyt;
   plan->ranges = reinterpret_cast<roialign::WorkRange*>(cur);
   cur += b_ranges;
@@ -226,20 +227,22 @@ bool use_tiled() { return mobula_hip::option("roialign_impl", kAuto) != kNaive; 
 void backward_device(const Problem& p, const float* dy, const float* rois, float* dx, bool assign,
                      hipStream_t stream) {
   if (p.N <= 0) return;
-  using BT = roialign::BwdTile;
+  using BB = roialign::BwdBlocked;
   TilePlan plan;
-  if (use_tiled() && roialign::backward_tiled_supports(p.PH, p.PW, p.S) &&
-      plan_tiles(p, rois, BT::TH, BT::TW, /*with_lists=*/true, stream, &plan)) {
-    const int cblocks = (p.C + BT::CH - 1) / BT::CH;
-    const long long jobs = plan.grid.total * cblocks;
-    const long long grid = (jobs + 7) / 8 * 8;
-    if (grid < (1ll << 31)) {
+  if (use_tiled() && roialign::backward_blocked_supports(p.PH, p.PW, p.S) &&
+      plan_tiles(p, rois, BB::TH, BB::TW, /*with_lists=*/true, stream, &plan)) {
+    const int cblk = (p.C + BB::CB - 1) / BB::CB;
+    const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
+    const long long dy_blocks = static_cast<long long>(p.R) * cblk;
+    if (grid < (1ll << 31) && dy_blocks < (1ll << 31)) {
+      const int pwp = plan.layout.col_stride;
       if (p.R > 0)
-        roialign::transpose_dy_kernel<<<p.R * cblocks, 256, sizeof(float) * 64 * p.PH * p.PW, stream>>>(
-            dy, plan.dyt, p.C, p.PH, p.PW, cblocks);
-      roialign::backward_tiled_kernel<<<static_cast<unsigned>(grid), BT::NT, 0, stream>>>(
-          plan.dyt, dx, plan.tile_offset, plan.ranges, plan.entries, plan.lists, plan.grid,
-          plan.layout, p.C, p.H, p.W, p.PH, p.PW, cblocks, jobs, assign ? 1 : 0);
+        roialign::transpose_dy_blocked_kernel<<<static_cast<unsigned>(dy_blocks), 256,
+                                                sizeof(float) * BB::CB * (p.PH * p.PW + 1), stream>>>(
+            dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk);
+      roialign::backward_blocked_kernel<<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
+          plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
+          p.W, p.PH, p.PW, p.S, cblk, assign ? 1 : 0);
       MOBULA_HIP_TRY(hipGetLastError());
       return;
     }
