@@ -81,7 +81,8 @@ __global__ void __launch_bounds__(BwdBlocked::NT)
 backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
                         const WorkRange* __restrict__ ranges, const WorkEntry* __restrict__ entries,
                         const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll, int C, int H,
-                        int W, int PH, int PW, int S, int cblk, int assign) {
+                        int W, int PH, int PW, int cblk, unsigned dyb_bytes, unsigned list_bytes,
+                        int assign) {
   using K = BwdBlocked;
   __shared__ __attribute__((aligned(16))) float acc[K::TH * K::RS * K::CS];
 
@@ -122,28 +123,39 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
     reinterpret_cast<float4*>(row)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 
   const WorkRange wr = ranges[tile * kTileRows + wave];
-  const int n_entries = wr.count;
+  const int n_entries = wr.count;   // a multiple of 2 * G, and G more entries follow: the lists are padded
   const int16v* const wl = reinterpret_cast<const int16v*>(entries + wr.begin);
   const int PWp = ll.col_stride;
-  const size_t dy_ph = static_cast<size_t>(PWp) * K::CB, dy_roi = dy_ph * PH * cblk;
   float* const cell0 = row + quad * 4;   // this lane's four channels of cell 0 (the left dummy)
+
+  // dyb and the sample lists as raw buffers: a scalar byte offset per entry
+  // plus a fixed lane offset
+  const unsigned dy_ph = static_cast<unsigned>(PWp) * K::CB * sizeof(float);
+  const unsigned dy_roi = dy_ph * PH * cblk;
+  const unsigned list_roi = static_cast<unsigned>(ll.roi_stride) * sizeof(AxisUnit);
+  const __amdgpu_buffer_rsrc_t dy_buf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(dyb), 0, static_cast<int>(dyb_bytes), 0x00020000);
+  const __amdgpu_buffer_rsrc_t list_buf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<AxisUnit*>(lists), 0, static_cast<int>(list_bytes), 0x00020000);
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
   // Each wavefront streams through the work list of its tile row: entries
   // (ROI, pooled row, weight) in ROI order, four at a time, double buffered:
   // while the taps of one group are folded and added, the dy rows and column
-  // samples of the next are in flight.
+  // samples of the next are in flight (always eight loads per group, so the
+  // wait before a group counts exactly the loads of the group after it).
   for (int pwb = 0; pwb < PW; pwb += K::PWB) {
-    const float* const dy_lane = dyb + static_cast<size_t>(cb) * dy_ph * PH + pwb * K::CB + lane * 4;
-    const AxisUnit* const col_lane = lists + static_cast<long long>(ll.ty) * ll.row_stride +
-                                     static_cast<long long>(tx) * ll.col_stride + pwb + grp;
-    auto issue = [&](const int16v& e, int e0, float4 (&d)[K::G], int4 (&u)[K::G]) {
+    const unsigned dy_fixed = cb * dy_ph * PH + pwb * K::CB * sizeof(float);
+    const unsigned list_fixed = static_cast<unsigned>(
+        (static_cast<long long>(ll.ty) * ll.row_stride + static_cast<long long>(tx) * ll.col_stride + pwb) *
+        sizeof(AxisUnit));
+    const int dy_lane = lane * 16, list_lane = grp * 16;
+    auto issue = [&](const int16v& e, u32x4 (&d)[K::G], u32x4 (&u)[K::G]) {
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
-        if (e0 + j < n_entries) {
-          d[j] = *reinterpret_cast<const float4*>(dy_lane + e[4 * j] * dy_roi + e[4 * j + 1] * dy_ph);
-          if ((e[4 * j + 3] & 2) != 0)
-            u[j] = *reinterpret_cast<const int4*>(col_lane + static_cast<long long>(e[4 * j]) * ll.roi_stride);
-        }
+        const unsigned roi = e[4 * j], ph = e[4 * j + 1];
+        d[j] = __builtin_amdgcn_raw_buffer_load_b128(dy_buf, dy_lane, roi * dy_roi + ph * dy_ph + dy_fixed, 0);
+        u[j] = __builtin_amdgcn_raw_buffer_load_b128(list_buf, list_lane, roi * list_roi + list_fixed, 0);
       }
     };
     float g[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -159,31 +171,29 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
       *reinterpret_cast<float4*>(a) = lo;
       *reinterpret_cast<float4*>(a + K::CS) = hi;
     };
-    auto process = [&](const int16v& e, int e0, const float4 (&d)[K::G], const int4 (&u)[K::G]) {
+    auto process = [&](const int16v& e, const u32x4 (&d)[K::G], const u32x4 (&u)[K::G]) {
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
-        if (e0 + j < n_entries) {
-          const float wy = __int_as_float(e[4 * j + 2]);
-          const int fl = e[4 * j + 3];
-          if ((fl & 1) == 0) {
-            g[0] = d[j].x * wy; g[1] = d[j].y * wy; g[2] = d[j].z * wy; g[3] = d[j].w * wy;
+        const float wy = __int_as_float(e[4 * j + 2]);
+        const int fl = e[4 * j + 3];
+        const float keep = (fl & 1) ? 1.0f : 0.0f;   // first tap of a ROI restarts the sum
+#pragma unroll
+        for (int i = 0; i < 4; ++i) g[i] = fmaf(__uint_as_float(d[j][i]), wy, keep * g[i]);
+        if ((fl & 2) != 0) {
+          // last tap of this ROI on this row: spread g over the column samples
+          const int cf = u[j][1];
+          const int pos0 = u[j][0] & 0xffff, pos1 = u[j][0] >> 16;
+          const float l0 = __uint_as_float(u[j][2]), l1 = __uint_as_float(u[j][3]);
+          const int turns = 1 << ((__builtin_amdgcn_readfirstlane(cf) >> kColStrideShift) & kColStrideMask);
+          auto add_both = [&] {
+            if ((cf & 3) != 0) add_sample(pos0, (cf & 1) ? 1.0f - l0 : 0.0f, (cf & 2) ? l0 : 0.0f);
+            if ((cf & 12) != 0) add_sample(pos1, (cf & 4) ? 1.0f - l1 : 0.0f, (cf & 8) ? l1 : 0.0f);
+          };
+          if (turns == 1) {
+            add_both();
           } else {
-            g[0] = fmaf(d[j].x, wy, g[0]); g[1] = fmaf(d[j].y, wy, g[1]);
-            g[2] = fmaf(d[j].z, wy, g[2]); g[3] = fmaf(d[j].w, wy, g[3]);
-          }
-          if ((fl & 2) != 0) {
-            // last tap of this ROI on this row: spread g over the column samples
-            const int cf = u[j].y;
-            const int pos0 = u[j].x & 0xffff, pos1 = static_cast<unsigned>(u[j].x) >> 16;
-            const float l0 = __int_as_float(u[j].z), l1 = __int_as_float(u[j].w);
-            const int lg = (__builtin_amdgcn_readfirstlane(cf) >> kColStrideShift) & kColStrideMask;
-            const int turns = min(K::PWB, max(1, (1 << lg) / S));
-            for (int t = 0; t < turns; ++t) {
-              if ((grp & (turns - 1)) == t) {
-                if ((cf & 3) != 0) add_sample(pos0, (cf & 1) ? 1.0f - l0 : 0.0f, (cf & 2) ? l0 : 0.0f);
-                if ((cf & 12) != 0) add_sample(pos1, (cf & 4) ? 1.0f - l1 : 0.0f, (cf & 8) ? l1 : 0.0f);
-              }
-            }
+            for (int t = 0; t < turns; ++t)
+              if ((grp & (turns - 1)) == t) add_both();
           }
         }
       }
@@ -191,21 +201,18 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
 
     if (n_entries > 0) {
       int16v e_cur = wl[0], e_nx = wl[1], e_n2;
-      float4 d_a[K::G], d_b[K::G];
-      int4 u_a[K::G], u_b[K::G];
-      issue(e_cur, 0, d_a, u_a);
+      u32x4 d_a[K::G], d_b[K::G], u_a[K::G], u_b[K::G];
+      issue(e_cur, d_a, u_a);
       for (int e0 = 0; e0 < n_entries; e0 += 2 * K::G) {
         // group at e0 lives in set a, group at e0 + G in set b
         e_n2 = wl[(e0 >> 2) + 2];
-        if (e0 + K::G < n_entries) issue(e_nx, e0 + K::G, d_b, u_b);
-        process(e_cur, e0, d_a, u_a);
+        issue(e_nx, d_b, u_b);
+        process(e_cur, d_a, u_a);
         e_cur = e_nx; e_nx = e_n2;
-        if (e0 + K::G < n_entries) {
-          e_n2 = wl[(e0 >> 2) + 3];
-          if (e0 + 2 * K::G < n_entries) issue(e_nx, e0 + 2 * K::G, d_a, u_a);
-          process(e_cur, e0 + K::G, d_b, u_b);
-          e_cur = e_nx; e_nx = e_n2;
-        }
+        e_n2 = wl[(e0 >> 2) + 3];
+        issue(e_nx, d_a, u_a);   // past the end this is the padding: loaded, never used
+        process(e_cur, d_b, u_b);
+        e_cur = e_nx; e_nx = e_n2;
       }
     }
   }

@@ -37,9 +37,9 @@ struct alignas(16) AxisUnit { int bin; int pos; float w0, w1; };
 //          one column left of the tile is cell 0, its high corner cell 1)
 //   flags  bit 0/1: low/high corner of sample 0 lies in the tile and has a
 //          non-zero weight; bit 2/3: same for sample 1; bits 8..10: log2 of the
-//          smallest power-of-two distance (in sample columns) at which two
-//          samples of this list never share a cell: pooled columns that far
-//          apart can be added concurrently
+//          smallest power-of-two distance (in pooled columns, at most 8) at
+//          which the first (and likewise the second) samples of two pooled
+//          columns never share a cell: columns that far apart are added concurrently
 //   l0/l1  weight of the high corner; the low corner weighs 1 - l
 struct alignas(16) ColPair { int cells; int flags; float l0, l1; };
 constexpr int kColStrideShift = 8;
@@ -152,13 +152,16 @@ build_lists_kernel(const RoiRec* __restrict__ recs, int R, int PH, int PW, int S
       const float l_n = __shfl_down(a.l, 1);
       ColPair cp;
       cp.cells = (pos + 1) | ((S == 2 ? pos_n + 1 : 0) << 16);
-      cp.flags = fl | ((S == 2 ? fl_n : 0) << 2) | (lg << kColStrideShift);
+      // Lanes take the first samples of their pooled columns together, then the
+      // second ones: columns t apart are S * t samples apart.
+      const int turns_log = max(0, min(3, lg - (S == 2 ? 1 : 0)));
+      cp.flags = fl | ((S == 2 ? fl_n : 0) << 2) | (turns_log << kColStrideShift);
       cp.l0 = a.l;
       cp.l1 = S == 2 ? l_n : 0.0f;
       if (real && ix == 0) cols[tx * ll.col_stride + pw] = cp;
       // padding columns: nothing to add, same spacing
       if (lane < ll.col_stride - PW)
-        cols[tx * ll.col_stride + PW + lane] = ColPair{0, lg << kColStrideShift, 0.0f, 0.0f};
+        cols[tx * ll.col_stride + PW + lane] = ColPair{0, turns_log << kColStrideShift, 0.0f, 0.0f};
     }
   }
 }
@@ -177,7 +180,7 @@ struct WorkRange { int begin; int count; };
 
 // One workgroup per tile, one wavefront per tile row: lane j looks at ROI j of
 // the tile's list, takes its taps for this row from the row-tap table, and all
-// lanes append theirs in list order.  Space for the tile's sixteen lists comes
+// lanes append theirs in list order.  WorkRange::count includes the padding.  Space for the tile's sixteen lists comes
 // from one bump-pointer allocation per tile (*cursor).
 __global__ void __launch_bounds__(kTileRows * 64)
 build_worklists_kernel(const int* __restrict__ tile_offset, const int* __restrict__ tile_rois,
@@ -201,7 +204,11 @@ build_worklists_kernel(const int* __restrict__ tile_offset, const int* __restric
     for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
     total += c;
   }
-  if (lane == 0) row_total[row] = total;
+  // Lists are padded to a multiple of eight entries (one turn of the consumer's
+  // double-buffered pipeline) plus four more that it prefetches but never uses.
+  const int padded = (total + 7) & ~7;
+  const int reserved = total > 0 ? padded + 4 : 0;
+  if (lane == 0) row_total[row] = reserved;
   __syncthreads();
   if (threadIdx.x == 0) {
     int sum = 0;
@@ -211,7 +218,7 @@ build_worklists_kernel(const int* __restrict__ tile_offset, const int* __restric
   __syncthreads();
   int out = tile_base;
   for (int r = 0; r < row; ++r) out += row_total[r];
-  if (lane == 0) ranges[tile * kTileRows + row] = WorkRange{out, total};
+  if (lane == 0) ranges[tile * kTileRows + row] = WorkRange{out, padded};
   for (int base = begin; base < end; base += 64) {
     int c = 0, roi = 0;
     const RowTap* taps = nullptr;
@@ -232,6 +239,8 @@ build_worklists_kernel(const int* __restrict__ tile_offset, const int* __restric
       dst[q] = WorkEntry{roi, taps[q].ph, taps[q].wy, (q > 0 ? 1 : 0) | (q == c - 1 ? 2 : 0)};
     out += __shfl(incl, 63);
   }
+  // padding: taps of weight zero that continue the last ROI and never end it
+  if (lane < reserved - total) entries[out + lane] = WorkEntry{tile_rois[end - 1], 0, 0.0f, 1};
 }
 
 }  // namespace roialign

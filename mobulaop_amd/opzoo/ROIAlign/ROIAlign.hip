@@ -148,6 +148,7 @@ struct TilePlan {
   roialign::ListLayout layout;
   roialign::AxisUnit* lists;   // null unless requested
   float* dyb;                  // channel-blocked copy of dy, with the lists
+  size_t dyb_bytes, list_bytes;
   int* cursor;                 // bump pointer of the work lists (zeroed with tile_count)
   roialign::WorkRange* ranges; // per (tile, tile row)
   roialign::WorkEntry* entries;
@@ -179,8 +180,12 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   const size_t b_dyt = with_lists ? align_up(sizeof(float) * 32 * plan->layout.col_stride * p.R * p.PH * cblk, 256) : 0;
   // work lists: every tap of every ROI once per tile column it spans
   const long long n_entries =
-      with_lists ? static_cast<long long>(p.R) * 2 * p.PH * std::max(p.S, 1) * g.tx : 0;
+      with_lists ? static_cast<long long>(p.R) * 2 * p.PH * std::max(p.S, 1) * g.tx +
+                       11 * roialign::kTileRows * g.total : 0;
   if (n_entries > (1ll << 27)) return false;
+  // the consumer addresses both with 32-bit byte offsets
+  if (b_dyt >= (1ull << 31) || b_units >= (1ull << 31)) return false;
+  plan->dyb_bytes = b_dyt; plan->list_bytes = b_units;
   const size_t b_ranges = with_lists ? align_up(sizeof(roialign::WorkRange) * g.total * roialign::kTileRows, 256) : 0;
   const size_t b_entries = with_lists ? align_up(sizeof(roialign::WorkEntry) * n_entries, 256) + 512 : 0;
   char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list + b_units + b_dyt +
@@ -242,7 +247,8 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
             dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk);
       roialign::backward_blocked_kernel<<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
           plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
-          p.W, p.PH, p.PW, p.S, cblk, assign ? 1 : 0);
+          p.W, p.PH, p.PW, cblk, static_cast<unsigned>(plan.dyb_bytes),
+          static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
       MOBULA_HIP_TRY(hipGetLastError());
       return;
     }
