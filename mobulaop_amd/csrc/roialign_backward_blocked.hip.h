@@ -33,34 +33,43 @@ struct BwdBlocked {
 inline bool backward_blocked_supports(int PH, int PW, int S) { return lists_supported(PH, PW, S); }
 
 // dy[r][c][ph][pw] -> dyb[r][cb][ph][PWp][32], zero where pw >= PW or the channel
-// does not exist.  One workgroup per (ROI, channel block): the 32*PH*PW input
-// words are contiguous and so are the PH*PWp*32 output words.
+// does not exist.  One workgroup per (ROI, group of `per` channel blocks):
+// the input words of the group are contiguous and so are its output words.
+// LDS holds the input as it is; the transposition happens in the reads.
 __global__ void __launch_bounds__(256)
 transpose_dy_blocked_kernel(const float* __restrict__ dy, float* __restrict__ dyb, int C, int PH,
-                            int PW, int PWp, int cblk) {
+                            int PW, int PWp, int cblk, int per) {
   constexpr int CB = BwdBlocked::CB;
-  extern __shared__ float tbuf[];   // [32][PH*PW + 1]
-  const int r = blockIdx.x / cblk, cb = blockIdx.x % cblk;
-  const int c0 = cb * CB, nch = min(CB, C - c0);
-  const int bins = PH * PW, pitch = bins + 1;
+  extern __shared__ __attribute__((aligned(16))) float tbuf[];   // [per * 32][PH * PW]
+  const int groups = (cblk + per - 1) / per;
+  const int r = blockIdx.x / groups, grp = blockIdx.x % groups;
+  const int cb0 = grp * per, nblk = min(per, cblk - cb0);
+  const int c0 = cb0 * CB, nch = min(nblk * CB, C - c0);
+  const int bins = PH * PW;
   const float* src = dy + (static_cast<size_t>(r) * C + c0) * bins;
-  for (int i = threadIdx.x; i < nch * bins; i += 256) {
-    const int c = i / bins;
-    tbuf[c * pitch + (i - c * bins)] = src[i];
+  const int n_in = nch * bins;
+  if ((reinterpret_cast<size_t>(src) & 15) == 0) {
+    const int nvec = n_in >> 2;
+    for (int i = threadIdx.x; i < nvec; i += 256)
+      reinterpret_cast<float4*>(tbuf)[i] = reinterpret_cast<const float4*>(src)[i];
+    for (int i = 4 * nvec + threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
+  } else {
+    for (int i = threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
   }
   __syncthreads();
-  float* dst = dyb + (static_cast<size_t>(r) * cblk + cb) * PH * PWp * CB;
-  const int quads = PH * PWp * (CB / 4);
-  for (int q = threadIdx.x; q < quads; q += 256) {
-    const int cq = q & 7, cell = q >> 3, pw = cell % PWp, ph = cell / PWp;
+  float* dst = dyb + (static_cast<size_t>(r) * cblk + cb0) * PH * PWp * CB;
+  const int per_blk = PH * PWp * (CB / 4);   // 16-byte pieces of one channel block
+  for (int q = threadIdx.x; q < nblk * per_blk; q += 256) {
+    const int blk = q / per_blk, p = q - blk * per_blk;
+    const int cq = p & 7, cell = p >> 3, pw = cell % PWp, ph = cell / PWp;
     float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     if (pw < PW) {
-      const float* in = tbuf + ph * PW + pw;
-      const int c = 4 * cq;
-      if (c + 0 < nch) v.x = in[(c + 0) * pitch];
-      if (c + 1 < nch) v.y = in[(c + 1) * pitch];
-      if (c + 2 < nch) v.z = in[(c + 2) * pitch];
-      if (c + 3 < nch) v.w = in[(c + 3) * pitch];
+      const int c = blk * CB + 4 * cq;
+      const float* in = tbuf + c * bins + ph * PW + pw;
+      if (c + 0 < nch) v.x = in[0];
+      if (c + 1 < nch) v.y = in[bins];
+      if (c + 2 < nch) v.z = in[2 * bins];
+      if (c + 3 < nch) v.w = in[3 * bins];
     }
     *reinterpret_cast<float4*>(dst + static_cast<size_t>(q) * 4) = v;
   }

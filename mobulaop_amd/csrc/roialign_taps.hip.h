@@ -93,20 +93,50 @@ __device__ __forceinline__ AxisUnit clip_unit(int bin, const AxisSample& a, int 
 
 // One wavefront per ROI: lane s < PH*S evaluates sample row s once and clips it
 // against every tile row of the ROI's box; likewise for sample columns.
+// The wavefront also finds the ROI's box (the pixels any valid sample touches),
+// stores it as tile ranges for tile_fill_kernel and counts the ROI in every
+// tile of the box.
 __global__ void __launch_bounds__(256)
-build_lists_kernel(const RoiRec* __restrict__ recs, int R, int PH, int PW, int S, int H, int W,
-                   TileGrid tg, ListLayout ll, AxisUnit* __restrict__ lists) {
+build_lists_kernel(const float* __restrict__ rois, int R, float scale, int PH, int PW, int S, int H,
+                   int W, long long num_images, TileGrid tg, ListLayout ll,
+                   TileBox* __restrict__ boxes, int* __restrict__ tile_count,
+                   AxisUnit* __restrict__ lists) {
   const int roi = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
   if (roi >= R) return;
   const int lane = threadIdx.x & 63;
-  const RoiRec rec = recs[roi];
-  if (rec.row_lo > rec.row_hi) return;
+  const RoiGeom g = roi_geometry(rois + static_cast<long long>(roi) * 5, scale, PH, PW, S);
+  // one row sample and one column sample per lane
+  AxisSample ay = axis_sample(sample_coord(g.start_h, lane / S, g.bin_h, lane % S, S), H);
+  ay.valid = ay.valid && lane < PH * S;
+  AxisSample ax = axis_sample(sample_coord(g.start_w, lane / S, g.bin_w, lane % S, S), W);
+  ax.valid = ax.valid && lane < PW * S;
+  struct { int row_lo, row_hi, col_lo, col_hi; float start_h, start_w, bin_h, bin_w, count; } rec;
+  rec.start_h = g.start_h; rec.start_w = g.start_w; rec.bin_h = g.bin_h; rec.bin_w = g.bin_w;
+  rec.count = g.count;
+  {
+    int rlo = ay.valid ? ay.low : H, rhi = ay.valid ? ay.high : -1;
+    int clo = ax.valid ? ax.low : W, chi = ax.valid ? ax.high : -1;
+    for (int off = 32; off > 0; off >>= 1) {
+      rlo = min(rlo, __shfl_xor(rlo, off)); rhi = max(rhi, __shfl_xor(rhi, off));
+      clo = min(clo, __shfl_xor(clo, off)); chi = max(chi, __shfl_xor(chi, off));
+    }
+    const bool image_ok = g.batch >= 0 && g.batch < num_images;
+    const bool any = image_ok && rlo <= rhi && clo <= chi;
+    rec.row_lo = any ? rlo : 0; rec.row_hi = any ? rhi : -1;
+    rec.col_lo = any ? clo : 0; rec.col_hi = any ? chi : -1;
+    const int ty0 = rec.row_lo / tg.th, ty1 = any ? rec.row_hi / tg.th : -1;
+    const int tx0 = rec.col_lo / tg.tw, tx1 = any ? rec.col_hi / tg.tw : -1;
+    if (lane == 0) boxes[roi] = TileBox{any ? g.batch : -1, ty0 | (ty1 << 16), tx0 | (tx1 << 16), 0};
+    if (!any) return;
+    int* const counts = tile_count + static_cast<long long>(g.batch) * tg.per_image;
+    const int nx = tx1 - tx0 + 1, nt = (ty1 - ty0 + 1) * nx;
+    for (int t = lane; t < nt; t += 64) atomicAdd(counts + (ty0 + t / nx) * tg.tx + tx0 + t % nx, 1);
+  }
   AxisUnit* const base = lists + static_cast<long long>(roi) * ll.roi_stride;
   const float inv_count = 1.0f / rec.count;
   {
-    const int ph = lane / S, iy = lane - ph * S;
-    AxisSample a = axis_sample(sample_coord(rec.start_h, ph, rec.bin_h, iy, S), H);
-    a.valid = a.valid && lane < PH * S;
+    const int ph = lane / S;
+    const AxisSample a = ay;
     for (int ty = rec.row_lo / tg.th; ty <= rec.row_hi / tg.th; ++ty) {
       const AxisUnit u = clip_unit(ph, a, ty * tg.th, tg.th, inv_count);
       RowTapTable* const table = reinterpret_cast<RowTapTable*>(base + ty * ll.row_stride);
@@ -129,8 +159,7 @@ build_lists_kernel(const RoiRec* __restrict__ recs, int R, int PH, int PW, int S
     // lane = sample column pw * S + ix
     const int pw = lane / S, ix = lane - pw * S;
     const bool real = lane < PW * S;
-    AxisSample a = axis_sample(sample_coord(rec.start_w, pw, rec.bin_w, ix, S), W);
-    a.valid = a.valid && real;
+    const AxisSample a = ax;
     ColPair* const cols = reinterpret_cast<ColPair*>(base + static_cast<long long>(ll.ty) * ll.row_stride);
     for (int tx = rec.col_lo / tg.tw; tx <= rec.col_hi / tg.tw; ++tx) {
       int pos = a.low - tx * tg.tw;

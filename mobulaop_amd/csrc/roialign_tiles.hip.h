@@ -10,16 +10,6 @@
 
 namespace roialign {
 
-struct RoiRec {
-  float start_h, start_w, bin_h, bin_w;
-  int grid_h, grid_w;
-  float count;
-  int batch;
-  // Inclusive pixel box of every corner pixel of every valid sample;
-  // row_lo > row_hi means the ROI touches nothing.
-  int row_lo, row_hi, col_lo, col_hi;
-};
-
 struct TileGrid {
   int th, tw;        // tile size in pixels
   int ty, tx;        // tiles per image along y and x
@@ -27,50 +17,9 @@ struct TileGrid {
   long long total;   // per_image * num_images
 };
 
-// Samples per axis above which the exact scan of sample positions is replaced
-// by "may touch anything" (the owners still test every sample exactly).
-constexpr int kMaxScan = 4096;
-
-__device__ __forceinline__ void axis_extent(float start, float bin, int pooled, int grid, int size,
-                                            int* lo, int* hi) {
-  const long long total = static_cast<long long>(pooled) * grid;
-  if (total > kMaxScan) { *lo = 0; *hi = size - 1; return; }
-  int mn = size, mx = -1;
-  for (int p = 0; p < pooled; ++p)
-    for (int i = 0; i < grid; ++i) {
-      const AxisSample s = axis_sample(sample_coord(start, p, bin, i, grid), size);
-      if (s.valid) { mn = min(mn, s.low); mx = max(mx, s.high); }
-    }
-  *lo = mn; *hi = mx;
-}
-
-// One thread per ROI: geometry record + per-tile counters.
-__global__ void __launch_bounds__(256)
-roi_prepare_kernel(const float* __restrict__ rois, int R, float scale, int PH, int PW, int S, int H,
-                   int W, long long num_images, TileGrid tg, RoiRec* __restrict__ recs,
-                   int* __restrict__ tile_count) {
-  const int r = blockIdx.x * blockDim.x + threadIdx.x;
-  if (r >= R) return;
-  const RoiGeom g = roi_geometry(rois + static_cast<long long>(r) * 5, scale, PH, PW, S);
-  RoiRec rec;
-  rec.start_h = g.start_h; rec.start_w = g.start_w; rec.bin_h = g.bin_h; rec.bin_w = g.bin_w;
-  rec.grid_h = g.grid_h; rec.grid_w = g.grid_w; rec.count = g.count; rec.batch = g.batch;
-  rec.row_lo = rec.col_lo = 0; rec.row_hi = rec.col_hi = -1;
-  if (g.batch >= 0 && g.batch < num_images) {
-    axis_extent(g.start_h, g.bin_h, PH, g.grid_h, H, &rec.row_lo, &rec.row_hi);
-    axis_extent(g.start_w, g.bin_w, PW, g.grid_w, W, &rec.col_lo, &rec.col_hi);
-    if (rec.row_lo > rec.row_hi || rec.col_lo > rec.col_hi) {
-      rec.row_lo = rec.col_lo = 0; rec.row_hi = rec.col_hi = -1;
-    }
-  }
-  recs[r] = rec;
-  if (rec.row_lo <= rec.row_hi) {
-    int* base = tile_count + static_cast<long long>(g.batch) * tg.per_image;
-    for (int ty = rec.row_lo / tg.th; ty <= rec.row_hi / tg.th; ++ty)
-      for (int tx = rec.col_lo / tg.tw; tx <= rec.col_hi / tg.tw; ++tx)
-        atomicAdd(base + ty * tg.tx + tx, 1);
-  }
-}
+// The tiles a ROI touches: image (-1: none), first | last << 16 tile row, first |
+// last << 16 tile column.
+struct alignas(16) TileBox { int batch; int ty; int tx; int pad; };
 
 // Exclusive prefix sum of tile_count[0..n) into tile_offset[0..n]; one block.
 __global__ void __launch_bounds__(1024)
@@ -100,30 +49,40 @@ tile_scan_kernel(const int* __restrict__ tile_count, long long n, int* __restric
   if (threadIdx.x == 0) tile_offset[n] = carry;
 }
 
-// One wavefront per tile: writes the tile's ROI list in increasing ROI index.
+// One workgroup of four wavefronts per tile: writes the tile's ROI list in
+// increasing ROI index.  Each wavefront takes a quarter of the ROIs, counts its
+// hits, and after one exchange writes them behind those of the quarters before.
 __global__ void __launch_bounds__(256)
-tile_fill_kernel(const RoiRec* __restrict__ recs, int R, TileGrid tg,
+tile_fill_kernel(const TileBox* __restrict__ boxes, int R, TileGrid tg,
                  const int* __restrict__ tile_offset, int* __restrict__ tile_rois) {
-  const long long tile = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
-  if (tile >= tg.total) return;
-  const int lane = threadIdx.x & 63;
+  __shared__ int hits[4];
+  const long long tile = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = static_cast<int>(tile / tg.per_image);
   const int t = static_cast<int>(tile % tg.per_image);
-  const int r0 = (t / tg.tx) * tg.th, c0 = (t % tg.tx) * tg.tw;
+  const int ty = t / tg.tx, tx = t % tg.tx;
   const int begin = tile_offset[tile], want = tile_offset[tile + 1] - begin;
   if (want == 0) return;
-  int written = 0;
-  for (int base = 0; base < R && written < want; base += 64) {
-    const int r = base + lane;
-    bool hit = false;
-    if (r < R) {
-      const RoiRec rec = recs[r];
-      hit = rec.batch == n && rec.row_lo <= rec.row_hi && rec.row_hi >= r0 &&
-            rec.row_lo < r0 + tg.th && rec.col_hi >= c0 && rec.col_lo < c0 + tg.tw;
-    }
+  const int quarter = ((R + 255) / 256) * 64;
+  const int r_begin = wave * quarter, r_end = min(R, r_begin + quarter);
+  auto hit_of = [&](int r) {
+    if (r >= r_end) return false;
+    const TileBox b = boxes[r];
+    return b.batch == n && ty >= (b.ty & 0xffff) && ty <= (b.ty >> 16) && tx >= (b.tx & 0xffff) &&
+           tx <= (b.tx >> 16);
+  };
+  int mine = 0;
+  for (int base = r_begin; base < r_end; base += 64) mine += __popcll(__ballot(hit_of(base + lane)));
+  if (lane == 0) hits[wave] = mine;
+  __syncthreads();
+  int written = begin;
+  for (int w = 0; w < wave; ++w) written += hits[w];
+  for (int base = r_begin; base < r_end && mine > 0; base += 64) {
+    const bool hit = hit_of(base + lane);
     const unsigned long long mask = __ballot(hit);
-    if (hit) tile_rois[begin + written + __popcll(mask & ((1ull << lane) - 1ull))] = r;
+    if (hit) tile_rois[written + __popcll(mask & ((1ull << lane) - 1ull))] = base + lane;
     written += __popcll(mask);
+    mine -= __popcll(mask);
   }
 }
 

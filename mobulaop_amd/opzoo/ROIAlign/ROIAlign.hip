@@ -141,7 +141,7 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
 // Scratch layout of the tile pre-pass, carved out of the device workspace.
 struct TilePlan {
   roialign::TileGrid grid;
-  roialign::RoiRec* recs;
+  roialign::TileBox* boxes;
   int* tile_count;
   int* tile_offset;
   int* tile_rois;
@@ -169,7 +169,7 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   g.total = static_cast<long long>(g.per_image) * p.N;
   const long long list_cap = static_cast<long long>(p.R) * g.per_image;  // every ROI in every tile
   if (g.total <= 0 || g.total > (1ll << 24) || list_cap > (1ll << 27)) return false;
-  const size_t b_recs = align_up(sizeof(roialign::RoiRec) * std::max(p.R, 1), 256);
+  const size_t b_recs = align_up(sizeof(roialign::TileBox) * std::max(p.R, 1), 256);
   const size_t b_cnt = align_up(sizeof(int) * (g.total + 1), 256);
   const size_t b_list = align_up(sizeof(int) * std::max<long long>(list_cap, 1), 256);
   plan->layout = roialign::make_list_layout(g, p.PW);
@@ -191,7 +191,7 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list + b_units + b_dyt +
                                                         b_ranges + b_entries + 256));
   if (failed()) return false;
-  plan->recs = reinterpret_cast<roialign::RoiRec*>(base);
+  plan->boxes = reinterpret_cast<roialign::TileBox*>(base);
   plan->tile_count = reinterpret_cast<int*>(base + b_recs);
   plan->tile_offset = reinterpret_cast<int*>(base + b_recs + b_cnt);
   plan->tile_rois = reinterpret_cast<int*>(base + b_recs + 2 * b_cnt);
@@ -206,23 +206,17 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   plan->entries = reinterpret_cast<roialign::WorkEntry*>(cur);
   cur += b_entries;
   MOBULA_HIP_TRY(hipMemsetAsync(plan->tile_count, 0, sizeof(int) * (g.total + 1), stream));
-  if (p.R > 0) {
-    roialign::roi_prepare_kernel<<<(p.R + 255) / 256, 256, 0, stream>>>(
-        rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->recs, plan->tile_count);
-  }
+  if (p.R > 0)
+    roialign::build_lists_kernel<<<(p.R * 64 + 255) / 256, 256, 0, stream>>>(
+        rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->layout, plan->boxes,
+        plan->tile_count, plan->lists);
   roialign::tile_scan_kernel<<<1, 1024, 0, stream>>>(plan->tile_count, g.total, plan->tile_offset);
-  if (p.R > 0) {
-    const long long threads = g.total * 64;
-    roialign::tile_fill_kernel<<<static_cast<int>((threads + 255) / 256), 256, 0, stream>>>(
-        plan->recs, p.R, g, plan->tile_offset, plan->tile_rois);
-    if (with_lists)
-      roialign::build_lists_kernel<<<(p.R * 64 + 255) / 256, 256, 0, stream>>>(
-          plan->recs, p.R, p.PH, p.PW, p.S, p.H, p.W, g, plan->layout, plan->lists);
-  }
-  if (with_lists)
-    roialign::build_worklists_kernel<<<static_cast<unsigned>(g.total), roialign::kTileRows * 64, 0, stream>>>(
-        plan->tile_offset, plan->tile_rois, plan->lists, g, plan->layout, plan->cursor,
-        plan->ranges, plan->entries);
+  if (p.R > 0)
+    roialign::tile_fill_kernel<<<static_cast<unsigned>(g.total), 256, 0, stream>>>(
+        plan->boxes, p.R, g, plan->tile_offset, plan->tile_rois);
+  roialign::build_worklists_kernel<<<static_cast<unsigned>(g.total), roialign::kTileRows * 64, 0, stream>>>(
+      plan->tile_offset, plan->tile_rois, plan->lists, g, plan->layout, plan->cursor, plan->ranges,
+      plan->entries);
   MOBULA_HIP_TRY(hipGetLastError());
   return !failed();
 }
@@ -238,13 +232,16 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
       plan_tiles(p, rois, BB::TH, BB::TW, /*with_lists=*/true, stream, &plan)) {
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
-    const long long dy_blocks = static_cast<long long>(p.R) * cblk;
-    if (grid < (1ll << 31) && dy_blocks < (1ll << 31)) {
+    // channel blocks per workgroup of the dy transposition: what 64 KB of LDS hold, at most 4
+    const size_t dy_blk_bytes = sizeof(float) * BB::CB * p.PH * p.PW;
+    const int dy_per = static_cast<int>(std::min<size_t>(4, (64 * 1024) / dy_blk_bytes));
+    const long long dy_blocks = dy_per > 0 ? static_cast<long long>(p.R) * ((cblk + dy_per - 1) / dy_per) : 0;
+    if (grid < (1ll << 31) && dy_blocks < (1ll << 31) && dy_per > 0) {
       const int pwp = plan.layout.col_stride;
       if (p.R > 0)
         roialign::transpose_dy_blocked_kernel<<<static_cast<unsigned>(dy_blocks), 256,
-                                                sizeof(float) * BB::CB * (p.PH * p.PW + 1), stream>>>(
-            dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk);
+                                                dy_per * dy_blk_bytes, stream>>>(
+            dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dy_per);
       roialign::backward_blocked_kernel<<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
           plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
           p.W, p.PH, p.PW, cblk, static_cast<unsigned>(plan.dyb_bytes),
