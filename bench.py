@@ -24,6 +24,12 @@ sys.path.insert(0, os.path.join(ROOT, 'tests'))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch of a kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc
+# WRITE_SIZE runs of this script (summaries under profiles/), each scaled by what
+# the same counter reads for a copy of known size.  Keyed by (workload, kernel);
+# absent entries are reported as null.
+MEASURED_TRAFFIC = {}
+
 
 def cpu_baseline(w, budget_s=25.0):
     """Reference kernels on the host cores: forward+backward ROIs/s on a
@@ -112,6 +118,31 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
+    # Per-kernel time of the dominant kernel of each pass: the library brackets it
+    # with HIP events on the launch stream (option "kernel_timing"); measured in
+    # a loop of its own after the throughput loop, same inputs, same stream.
+    from mobulaop_amd import native
+    lib = native.library()
+    lib.mobula_hip_last_kernel_ms.restype = ctypes.c_double
+    lib.mobula_hip_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_char_p)]
+    native.set_option('kernel_timing', 1)
+    kernel_ms = {}
+
+    def note_kernel():
+        name = ctypes.c_char_p()
+        ms = lib.mobula_hip_last_kernel_ms(ctypes.byref(name))
+        if ms >= 0 and name.value:
+            kernel_ms.setdefault(name.value.decode(), []).append(ms)
+
+    for _ in range(args.steps):
+        abi.forward(x, rois, pooled, scale, S, stream=stream)
+        note_kernel()
+        if has_bwd:
+            abi.backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream)
+            note_kernel()
+    native.set_option('kernel_timing', 0)
+    kernel_ms = {k: sum(v) / len(v) for k, v in kernel_ms.items()}
+
     fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
     bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps if has_bwd else 0.0
     ms_per_step = wall * 1e3 / args.steps
@@ -120,8 +151,17 @@ def main():
     def gbs(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
 
-    dominant = 'backward' if bwd_ms > fwd_ms else 'forward'
-    dom_bytes, dom_ms = (b_bwd, bwd_ms) if dominant == 'backward' else (b_fwd, fwd_ms)
+    # The dominant kernel: the longest of the bracketed ones.  Its algorithmic
+    # bytes are those of its pass (each tensor of the pass once): the helper
+    # kernels around it exist only to feed it.
+    pass_of = {'forward_blocked_kernel': ('forward', b_fwd), 'backward_blocked_kernel': ('backward', b_bwd)}
+    if kernel_ms:
+        dom_kernel = max(kernel_ms, key=kernel_ms.get)
+        dom_ms = kernel_ms[dom_kernel]
+        dom_bytes = pass_of.get(dom_kernel, ('forward', b_fwd))[1]
+    else:  # the straightforward kernels carry no bracket: fall back to the slower pass
+        dom_kernel = ('backward' if bwd_ms > fwd_ms else 'forward') + ' pass'
+        dom_bytes, dom_ms = (b_bwd, bwd_ms) if bwd_ms > fwd_ms else (b_fwd, fwd_ms)
     passes = {'forward': {'ms': fwd_ms, 'GB/s': gbs(b_fwd, fwd_ms), 'frac': gbs(b_fwd, fwd_ms) / HBM_PEAK_GBS,
                           'rois_per_s': R / (fwd_ms * 1e-3)}}
     total_bytes = b_fwd
@@ -143,9 +183,11 @@ def main():
         'config': {'workload': '{}: data {} rois {} pooled {} scale {} sampling_ratio {}'.format(
             w['name'], 'x'.join(map(str, w['data'].shape)), R, 'x'.join(map(str, pooled)), scale, S),
             'impl': args.impl, 'step': 'forward + backward(assign)' if has_bwd else 'forward'},
-        'roofline': {'bound': 'hbm', 'kernel': dominant + ' pass', 'achieved': gbs(dom_bytes, dom_ms),
+        'roofline': {'bound': 'hbm', 'kernel': dom_kernel, 'achieved': gbs(dom_bytes, dom_ms),
                      'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': gbs(dom_bytes, dom_ms) / HBM_PEAK_GBS,
-                     'traffic': None, 'algorithmic_bytes': dom_bytes, 'avg_ms': dom_ms},
+                     'traffic': MEASURED_TRAFFIC.get((w['name'], dom_kernel)),
+                     'algorithmic_bytes': dom_bytes, 'avg_ms': dom_ms},
+        'kernels_ms': kernel_ms,
         'passes': passes,
     }
     if not args.no_cpu_baseline:

@@ -92,10 +92,17 @@ const char* mobula_hip_last_error(void);
 void mobula_hip_clear_error(void);
 
 /* Named integer switches ("roialign_impl": 0 auto, 1 tiled, 2 naive;
- * "host_staging_device").  set returns 0, or -1 for an unknown name; get
+ * "host_staging_device"; "kernel_timing": 0 off, 1 on).  set returns 0, or -1 for an unknown name; get
  * returns -1 for a name never set. */
 int mobula_hip_set_option(const char* name, long long value);
 long long mobula_hip_get_option(const char* name);
+
+/* With the option "kernel_timing" set to 1 the library brackets the dominant
+ * kernel of every operator call (the gather of the forward pass, the tile
+ * owners of the backward pass) with HIP events on the launch stream.  Returns
+ * the elapsed milliseconds of the calling thread's last bracket after waiting
+ * for it, -1 if there is none; *name (if not NULL) receives the kernel's name. */
+double mobula_hip_last_kernel_ms(const char** name);
 
 int mobula_hip_device_count(void);
 

@@ -71,6 +71,19 @@ class HostStaging {
 // Synchronises if the call is synchronous and clears the per-call extents.
 void finish_call();
 
+// With the option "kernel_timing" set, brackets the launches issued during its
+// lifetime with HIP events on `stream`; mobula_hip_last_kernel_ms() then
+// reports the elapsed time of the calling thread's last bracket.
+class KernelTimer {
+ public:
+  KernelTimer(const char* name, hipStream_t stream);
+  ~KernelTimer();
+
+ private:
+  hipStream_t stream_;
+  bool on_;
+};
+
 }  // namespace mobula_hip
 
 #define MOBULA_HIP_TRY(expr)                                                        \

@@ -105,6 +105,40 @@ bool HostStaging::flush(hipStream_t stream) {
   return !failed();
 }
 
+namespace {
+struct TimerState {
+  hipEvent_t start = nullptr, stop = nullptr;
+  const char* name = "";
+  bool pending = false;
+};
+TimerState& timer_state() {
+  static thread_local TimerState t;
+  return t;
+}
+}  // namespace
+
+KernelTimer::KernelTimer(const char* name, hipStream_t stream)
+    : stream_(stream), on_(option("kernel_timing", 0) != 0) {
+  if (!on_) return;
+  TimerState& t = timer_state();
+  if (t.start == nullptr) {
+    if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) {
+      t.start = t.stop = nullptr;
+      on_ = false;
+      return;
+    }
+  }
+  t.name = name;
+  t.pending = false;
+  if (hipEventRecord(t.start, stream_) != hipSuccess) on_ = false;
+}
+
+KernelTimer::~KernelTimer() {
+  if (!on_) return;
+  TimerState& t = timer_state();
+  t.pending = hipEventRecord(t.stop, stream_) == hipSuccess;
+}
+
 void finish_call() {
   CallState& st = call_state();
   if (st.synchronous && !failed()) MOBULA_HIP_TRY(hipStreamSynchronize(st.stream));
@@ -136,8 +170,7 @@ const char* mobula_hip_last_error(void) {
 void mobula_hip_clear_error(void) { call_state().error.clear(); }
 
 int mobula_hip_set_option(const char* name, long long value) {
-  static const char* known[] = {"roialign_impl", "host_staging_device", "roialign_fwd_variant",
-                                "roialign_bwd_variant", nullptr};
+  static const char* known[] = {"roialign_impl", "host_staging_device", "kernel_timing", nullptr};
   for (int i = 0; known[i] != nullptr; ++i) {
     if (std::strcmp(known[i], name) == 0) {
       std::lock_guard<std::mutex> lock(mobula_hip::g_mutex);
@@ -149,6 +182,16 @@ int mobula_hip_set_option(const char* name, long long value) {
 }
 
 long long mobula_hip_get_option(const char* name) { return mobula_hip::option(name, -1); }
+
+double mobula_hip_last_kernel_ms(const char** name) {
+  mobula_hip::TimerState& t = mobula_hip::timer_state();
+  if (name != nullptr) *name = t.name;
+  if (!t.pending) return -1.0;
+  float ms = 0.0f;
+  if (hipEventSynchronize(t.stop) != hipSuccess || hipEventElapsedTime(&ms, t.start, t.stop) != hipSuccess)
+    return -1.0;
+  return ms;
+}
 
 int mobula_hip_device_count(void) {
   int n = 0;

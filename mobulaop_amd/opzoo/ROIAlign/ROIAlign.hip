@@ -128,8 +128,11 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
       roialign::transpose_to_blocked_kernel<T, false><<<tgrid, 256, 0, stream>>>(
           x, xt, p.C, static_cast<int>(pixels));
     roialign::roi_order_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
-    roialign::forward_blocked_kernel<T><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
-        xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
+    {
+      mobula_hip::KernelTimer timer("forward_blocked_kernel", stream);
+      roialign::forward_blocked_kernel<T><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+          xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
+    }
     MOBULA_HIP_TRY(hipGetLastError());
     return;
   }
@@ -242,10 +245,13 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
         roialign::transpose_dy_blocked_kernel<<<static_cast<unsigned>(dy_blocks), 256,
                                                 dy_per * dy_blk_bytes, stream>>>(
             dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dy_per);
-      roialign::backward_blocked_kernel<<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
-          plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
-          p.W, p.PH, p.PW, cblk, static_cast<unsigned>(plan.dyb_bytes),
-          static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
+      {
+        mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
+        roialign::backward_blocked_kernel<<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
+            plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
+            p.W, p.PH, p.PW, cblk, static_cast<unsigned>(plan.dyb_bytes),
+            static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
+      }
       MOBULA_HIP_TRY(hipGetLastError());
       return;
     }
