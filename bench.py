@@ -28,7 +28,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # WRITE_SIZE runs of this script (summaries under profiles/), each scaled by what
 # the same counter reads for a copy of known size.  Keyed by (workload, kernel);
 # absent entries are reported as null.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    ('cfg2', 'forward_blocked_kernel'): 473.4e6,    # 272.7 MB read + 200.7 MB written
+    ('cfg2', 'backward_blocked_kernel'): 596.0e6,   # 301.0 MB read + 295.0 MB written
+}
 
 
 def cpu_baseline(w, budget_s=25.0):
