@@ -92,7 +92,9 @@ const char* mobula_hip_last_error(void);
 void mobula_hip_clear_error(void);
 
 /* Named integer switches ("roialign_impl": 0 auto, 1 tiled, 2 naive;
- * "host_staging_device"; "kernel_timing": 0 off, 1 on).  set returns 0, or -1 for an unknown name; get
+ * "host_staging_device"; "kernel_timing": 0 off, 1 on; "side_stream": 1 (default)
+ * lets helper kernels of a call run on a second stream of the device, 0 keeps
+ * everything on the caller's stream).  set returns 0, or -1 for an unknown name; get
  * returns -1 for a name never set. */
 int mobula_hip_set_option(const char* name, long long value);
 long long mobula_hip_get_option(const char* name);

@@ -88,4 +88,12 @@ __global__ void max_batch_kernel(const float* __restrict__ rois, int R, int* __r
   if ((threadIdx.x & 63) == 0) atomicMax(out, m);
 }
 
+// Clears n 32-bit words.  Used instead of a memset so that a caller may capture
+// the launches of a call into a graph and replay them.
+__global__ void __launch_bounds__(256)
+zero_words_kernel(unsigned* __restrict__ p, long long n) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0u;
+}
+
 }  // namespace roialign

@@ -71,6 +71,24 @@ class HostStaging {
 // Synchronises if the call is synchronous and clears the per-call extents.
 void finish_call();
 
+// A second stream of the current device on which independent helper kernels of
+// a call run beside the work on the caller's stream:
+//   SideStream side(stream);   work launched on side.get() starts after what
+//                              `stream` holds so far
+//   side.join();               `stream` waits for what the side stream holds
+// Both streams have the default priority.  With the option "side_stream" set to
+// 0 (or if the stream cannot be created) get() is the caller's stream itself.
+class SideStream {
+ public:
+  explicit SideStream(hipStream_t main);
+  hipStream_t get() const { return side_; }
+  void join();
+
+ private:
+  hipStream_t main_, side_;
+  hipEvent_t joined_ = nullptr;
+};
+
 // With the option "kernel_timing" set, brackets the launches issued during its
 // lifetime with HIP events on `stream`; mobula_hip_last_kernel_ms() then
 // reports the elapsed time of the calling thread's last bracket.

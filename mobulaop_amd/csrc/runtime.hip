@@ -106,6 +106,44 @@ bool HostStaging::flush(hipStream_t stream) {
 }
 
 namespace {
+struct SideState { hipStream_t stream = nullptr; hipEvent_t fork = nullptr, join = nullptr; bool tried = false; };
+SideState& side_state(int device) {
+  static thread_local std::map<int, SideState> states;
+  return states[device];
+}
+}  // namespace
+
+SideStream::SideStream(hipStream_t main) : main_(main), side_(main) {
+  if (option("side_stream", 1) == 0) return;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return;
+  SideState& st = side_state(device);
+  if (!st.tried) {
+    st.tried = true;
+    if (hipStreamCreateWithFlags(&st.stream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&st.fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&st.join, hipEventDisableTiming) != hipSuccess) {
+      st.stream = nullptr;
+      (void)hipGetLastError();
+    }
+  }
+  if (st.stream == nullptr) return;
+  if (hipEventRecord(st.fork, main_) != hipSuccess || hipStreamWaitEvent(st.stream, st.fork, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return;
+  }
+  side_ = st.stream;
+  joined_ = st.join;
+}
+
+void SideStream::join() {
+  if (side_ == main_) return;
+  MOBULA_HIP_TRY(hipEventRecord(joined_, side_));
+  MOBULA_HIP_TRY(hipStreamWaitEvent(main_, joined_, 0));
+  side_ = main_;
+}
+
+namespace {
 struct TimerState {
   hipEvent_t start = nullptr, stop = nullptr;
   const char* name = "";
@@ -170,7 +208,8 @@ const char* mobula_hip_last_error(void) {
 void mobula_hip_clear_error(void) { call_state().error.clear(); }
 
 int mobula_hip_set_option(const char* name, long long value) {
-  static const char* known[] = {"roialign_impl", "host_staging_device", "kernel_timing", nullptr};
+  static const char* known[] = {"roialign_impl", "host_staging_device", "kernel_timing", "side_stream",
+                                nullptr};
   for (int i = 0; known[i] != nullptr; ++i) {
     if (std::strcmp(known[i], name) == 0) {
       std::lock_guard<std::mutex> lock(mobula_hip::g_mutex);

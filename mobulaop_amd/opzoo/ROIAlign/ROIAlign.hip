@@ -89,7 +89,7 @@ long long images_from_rois(const float* d_rois, int R, hipStream_t stream) {
   if (R == 0) return 0;
   int* d_max = static_cast<int*>(mobula_hip::workspace(256));
   if (failed()) return 0;
-  MOBULA_HIP_TRY(hipMemsetAsync(d_max, 0, sizeof(int), stream));
+  roialign::zero_words_kernel<<<1, 64, 0, stream>>>(reinterpret_cast<unsigned*>(d_max), 1);
   roialign::max_batch_kernel<<<std::min(64, (R + 255) / 256), 256, 0, stream>>>(d_rois, R, d_max);
   int h = 0;
   MOBULA_HIP_TRY(hipMemcpyAsync(&h, d_max, sizeof(int), hipMemcpyDeviceToHost, stream));
@@ -118,6 +118,9 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
     if (failed()) return;
     T* const xt = reinterpret_cast<T*>(ws);
     int* const order = reinterpret_cast<int*>(ws + xt_bytes);
+    // the ROI ordering (one small workgroup) runs beside the transposition
+    mobula_hip::SideStream side(stream);
+    roialign::roi_order_kernel<<<1, 1024, 0, side.get()>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
     const dim3 tgrid(static_cast<unsigned>((pixels + 63) / 64), static_cast<unsigned>(cblk),
                      static_cast<unsigned>(p.N));
     const bool vec = pixels % 4 == 0 && reinterpret_cast<size_t>(x) % (4 * sizeof(T)) == 0;
@@ -127,7 +130,7 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
     else
       roialign::transpose_to_blocked_kernel<T, false><<<tgrid, 256, 0, stream>>>(
           x, xt, p.C, static_cast<int>(pixels));
-    roialign::roi_order_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
+    side.join();
     {
       mobula_hip::KernelTimer timer("forward_blocked_kernel", stream);
       roialign::forward_blocked_kernel<T><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
@@ -208,7 +211,8 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   cur += b_ranges;
   plan->entries = reinterpret_cast<roialign::WorkEntry*>(cur);
   cur += b_entries;
-  MOBULA_HIP_TRY(hipMemsetAsync(plan->tile_count, 0, sizeof(int) * (g.total + 1), stream));
+  roialign::zero_words_kernel<<<grid_for(g.total + 1, 256), 256, 0, stream>>>(
+      reinterpret_cast<unsigned*>(plan->tile_count), g.total + 1);
   if (p.R > 0)
     roialign::build_lists_kernel<<<(p.R * 64 + 255) / 256, 256, 0, stream>>>(
         rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->layout, plan->boxes,
@@ -231,8 +235,10 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
   if (p.N <= 0) return;
   using BB = roialign::BwdBlocked;
   TilePlan plan;
+  // the pre-pass (small, latency-bound kernels) runs beside the dy transposition
+  mobula_hip::SideStream side(stream);
   if (use_tiled() && roialign::backward_blocked_supports(p.PH, p.PW, p.S) &&
-      plan_tiles(p, rois, BB::TH, BB::TW, /*with_lists=*/true, stream, &plan)) {
+      plan_tiles(p, rois, BB::TH, BB::TW, /*with_lists=*/true, side.get(), &plan)) {
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
     // channel blocks per workgroup of the dy transposition: what 64 KB of LDS hold, at most 4
@@ -245,6 +251,7 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
         roialign::transpose_dy_blocked_kernel<<<static_cast<unsigned>(dy_blocks), 256,
                                                 dy_per * dy_blk_bytes, stream>>>(
             dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dy_per);
+      side.join();
       {
         mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
         roialign::backward_blocked_kernel<<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
@@ -256,9 +263,11 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
       return;
     }
   }
+  side.join();
   if (failed()) return;
   if (assign)
-    MOBULA_HIP_TRY(hipMemsetAsync(dx, 0, sizeof(float) * p.N * p.C * p.H * p.W, stream));
+    roialign::zero_words_kernel<<<grid_for(static_cast<long long>(p.N) * p.C * p.H * p.W, 256), 256, 0, stream>>>(
+        reinterpret_cast<unsigned*>(dx), static_cast<long long>(p.N) * p.C * p.H * p.W);
   if (p.n_out == 0) return;
   roialign::backward_naive_kernel<<<grid_for(p.n_out, 256), 256, 0, stream>>>(
       p.n_out, dy, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, dx, rois, p.N);
