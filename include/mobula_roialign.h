@@ -77,6 +77,55 @@ void roi_align_forward_e874c59a(const int device_id, const int nthreads,
                                 const int sampling_ratio, const float* bottom_rois,
                                 unsigned short* top_data);
 
+/* ---- Convolution -------------------------------------------------------- */
+
+/* One image: data_col[c, kh, kw, oh, ow] = data_im[c, ih, iw], zero in the
+ * padding; n = element count of data_col.
+ * Replaces: im2col_kernel<float>, opzoo/Convolution/Convolution.cpp:13-45. */
+void im2col_341af5d3(const int device_id, const int n, const float* data_im, const int height,
+                     const int width, const int kernel_h, const int kernel_w, const int pad_h,
+                     const int pad_w, const int stride_h, const int stride_w, const int dilation_h,
+                     const int dilation_w, const int height_col, const int width_col, float* data_col);
+
+/* One image: data_im[c, h, w] = sum of the column entries unfolded from it;
+ * n = element count of data_im.
+ * Replaces: col2im_kernel<float>, opzoo/Convolution/Convolution.cpp:47-90. */
+void col2im_341af5d3(const int device_id, const int n, const float* data_col, const int height,
+                     const int width, const int kernel_h, const int kernel_w, const int pad_h,
+                     const int pad_w, const int stride_h, const int stride_w, const int dilation_h,
+                     const int dilation_w, const int height_col, const int width_col, float* data_im);
+
+/* Extensions: the products the reference operator assembles per image from
+ * im2col / col2im and the framework's matrix product
+ * (opzoo/Convolution/Convolution.py:17-57), as one call each on the matrix
+ * cores.  x [batch, channels, height, width], weight [filters, channels,
+ * kernel_h, kernel_w], y / dy [batch, filters, OH, OW]; device memory only.
+ * n is the element count of the output tensor; accumulate != 0 adds to it. */
+void conv2d_forward_c6a7aa85(const int device_id, const int n, const float* x, const float* weight,
+                             const float* bias, const int has_bias, const int batch,
+                             const int channels, const int height, const int width, const int filters,
+                             const int kernel_h, const int kernel_w, const int pad_h, const int pad_w,
+                             const int stride_h, const int stride_w, const int dilation_h,
+                             const int dilation_w, float* y);
+void conv2d_backward_data_ecf81c91(const int device_id, const int n, const float* dy,
+                                   const float* weight, const int accumulate, const int batch,
+                                   const int channels, const int height, const int width,
+                                   const int filters, const int kernel_h, const int kernel_w,
+                                   const int pad_h, const int pad_w, const int stride_h,
+                                   const int stride_w, const int dilation_h, const int dilation_w,
+                                   float* dx);
+void conv2d_backward_weight_ecf81c91(const int device_id, const int n, const float* dy, const float* x,
+                                     const int accumulate, const int batch, const int channels,
+                                     const int height, const int width, const int filters,
+                                     const int kernel_h, const int kernel_w, const int pad_h,
+                                     const int pad_w, const int stride_h, const int stride_w,
+                                     const int dilation_h, const int dilation_w, float* dw);
+/* db[filters] (+)= sum of dy over images and pixels; n = filters. */
+void conv2d_backward_bias_cd239a08(const int device_id, const int n, const float* dy,
+                                   const int accumulate, const int batch, const int pixels, float* db);
+
+/* ---- Library control ---------------------------------------------------- */
+
 /* Per-thread launch stream (a hipStream_t) for subsequent calls; synchronous
  * != 0 makes each call wait for its result before returning. */
 void mobula_hip_set_stream(void* stream, int synchronous);

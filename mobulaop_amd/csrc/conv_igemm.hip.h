@@ -1,0 +1,324 @@
+// 2-D convolution as implicit GEMM on the fp32 matrix cores of gfx950.
+//
+// The reference (opzoo/Convolution/Convolution.py:17-57) unfolds every image
+// into a [C*KH*KW, OH*OW] column buffer with im2col and multiplies it with the
+// reshaped weights, one image at a time; the backward pass does the transposed
+// product plus col2im for dx and a second im2col for dW.  Here the column
+// buffer never exists: the three products
+//   y [D, N*OH*OW]  = W [D, C*KH*KW]      x col(x) [C*KH*KW, N*OH*OW]
+//   dx[C, N*H*W]    = W'[C, D*KH*KW]      x col'(dy)[D*KH*KW, N*H*W]
+//   dW[D, C*KH*KW]  = dy[D, N*OH*OW]      x col(x)'[N*OH*OW, C*KH*KW]
+// are tiled GEMMs whose operand elements are fetched from the tensors where
+// they lie (an operand functor maps a (row, k) or (k, column) index to an
+// address or to zero in the padding) and staged through LDS.
+//
+// Tiling: a workgroup of four wavefronts owns a 128x128 tile of the result and
+// walks K in steps of 16; each wavefront holds a 64x64 quarter as 2x2
+// accumulators of v_mfma_f32_32x32x2_f32 (64 registers per lane).  The next K
+// step is fetched into registers while the current one is multiplied out of
+// LDS (two LDS buffers, one barrier per step).
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace conv {
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+struct Geometry {
+  int N, C, H, W;        // input
+  int D, KH, KW;         // filters
+  int OH, OW;            // output
+  int pad_h, pad_w, stride_h, stride_w, dil_h, dil_w;
+};
+
+struct Tile {
+  static constexpr int BM = 128, BN = 128, BK = 16;
+  static constexpr int PITCH = BM + 32;   // consecutive k rows of a tile land 32 banks apart
+  static constexpr int NT = 256;
+};
+
+// Table entry for one value of the filter-tap index: element offset into the
+// tensor the taps walk over, and the dilated tap position.
+struct Tap { int off; short dh, dw; };
+
+// taps[k] for k = (c, kh, kw) over x (forward, dW) or k = (d, kh, kw) over dy (dx).
+__global__ void __launch_bounds__(256)
+build_taps_kernel(Tap* __restrict__ taps, int count, int KH, int KW, int plane, int dil_h, int dil_w) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= count) return;
+  const int kw = k % KW, kh = (k / KW) % KH, ch = k / (KW * KH);
+  taps[k] = Tap{ch * plane, static_cast<short>(kh * dil_h), static_cast<short>(kw * dil_w)};
+}
+
+// ---- operand functors -------------------------------------------------------
+// a(m, k): element of the left operand; BCtx b_ctx(n) + b(ctx, k): element of
+// the right operand for a fixed column n; store(m, n, v).
+
+struct ForwardOps {
+  const float* x; const float* w; const float* bias; float* y; const Tap* taps;
+  Geometry g; int M, Ncols, K;
+  struct BCtx { int base; int ih0, iw0; bool ok; };
+  __device__ float a(int m, int k) const { return (m < M && k < K) ? w[static_cast<size_t>(m) * K + k] : 0.0f; }
+  __device__ BCtx b_ctx(int n) const {
+    BCtx c;
+    c.ok = n < Ncols;
+    const int ohw = g.OH * g.OW, img = n / ohw, r = n - img * ohw, oh = r / g.OW, ow = r - oh * g.OW;
+    c.ih0 = oh * g.stride_h - g.pad_h;
+    c.iw0 = ow * g.stride_w - g.pad_w;
+    c.base = img * g.C * g.H * g.W + c.ih0 * g.W + c.iw0;
+    return c;
+  }
+  __device__ float b(const BCtx& c, int k) const {
+    if (!c.ok || k >= K) return 0.0f;
+    const Tap t = taps[k];
+    const int ih = c.ih0 + t.dh, iw = c.iw0 + t.dw;
+    if (static_cast<unsigned>(ih) >= static_cast<unsigned>(g.H) ||
+        static_cast<unsigned>(iw) >= static_cast<unsigned>(g.W))
+      return 0.0f;
+    return x[c.base + t.off + t.dh * g.W + t.dw];
+  }
+  __device__ void store(int m, int n, float v) const {
+    if (m >= M || n >= Ncols) return;
+    const int ohw = g.OH * g.OW, img = n / ohw, r = n - img * ohw;
+    y[(static_cast<size_t>(img) * g.D + m) * ohw + r] = bias != nullptr ? v + bias[m] : v;
+  }
+};
+
+// dx[img, c, ih, iw] = sum over (d, kh, kw) of W[d, c, kh, kw] * dy[img, d, oh, ow]
+// with oh * stride = ih + pad - kh * dil (and likewise for columns).
+struct BackwardDataOps {
+  const float* dy; const float* w; float* dx; const Tap* taps;   // taps over dy: off = d * OH*OW
+  Geometry g; int M, Ncols, K; int accumulate;
+  struct BCtx { int base; int ihp, iwp; bool ok; };
+  __device__ float a(int m, int k) const {
+    if (m >= M || k >= K) return 0.0f;
+    const int khw = g.KH * g.KW, d = k / khw, r = k - d * khw;
+    return w[(static_cast<size_t>(d) * g.C + m) * khw + r];
+  }
+  __device__ BCtx b_ctx(int n) const {
+    BCtx c;
+    c.ok = n < Ncols;
+    const int hw = g.H * g.W, img = n / hw, r = n - img * hw, ih = r / g.W, iw = r - ih * g.W;
+    c.ihp = ih + g.pad_h; c.iwp = iw + g.pad_w;
+    c.base = img * g.D * g.OH * g.OW;
+    return c;
+  }
+  __device__ float b(const BCtx& c, int k) const {
+    if (!c.ok || k >= K) return 0.0f;
+    const Tap t = taps[k];
+    const int th = c.ihp - t.dh, tw = c.iwp - t.dw;
+    if (th < 0 || tw < 0) return 0.0f;
+    const int oh = th / g.stride_h, ow = tw / g.stride_w;
+    if (oh * g.stride_h != th || ow * g.stride_w != tw || oh >= g.OH || ow >= g.OW) return 0.0f;
+    return dy[c.base + t.off + oh * g.OW + ow];
+  }
+  __device__ void store(int m, int n, float v) const {
+    if (m >= M || n >= Ncols) return;
+    const int hw = g.H * g.W, img = n / hw, r = n - img * hw;
+    float* p = dx + (static_cast<size_t>(img) * g.C + m) * hw + r;
+    *p = accumulate ? *p + v : v;
+  }
+};
+
+// partial[z][d, (c, kh, kw)] = sum over the images of slice z and (oh, ow) of
+// dy[img, d, oh, ow] * x[img, c, ih, iw].
+struct BackwardWeightOps {
+  const float* dy; const float* x; float* partial; const Tap* taps;   // taps over x
+  Geometry g; int M, Ncols, K;   // K = images_per_slice * OH*OW
+  int img0, images;              // the images of this slice
+  struct BCtx { int off; int dh, dw; bool ok; };
+  __device__ float a(int m, int k) const {
+    const int ohw = g.OH * g.OW, i = k / ohw, r = k - i * ohw;
+    if (m >= M || i >= images) return 0.0f;
+    return dy[(static_cast<size_t>(img0 + i) * g.D + m) * ohw + r];
+  }
+  __device__ BCtx b_ctx(int n) const {
+    BCtx c;
+    c.ok = n < Ncols;
+    const Tap t = taps[c.ok ? n : 0];
+    c.off = t.off; c.dh = t.dh; c.dw = t.dw;
+    return c;
+  }
+  __device__ float b(const BCtx& c, int k) const {
+    const int ohw = g.OH * g.OW, i = k / ohw, r = k - i * ohw;
+    if (!c.ok || i >= images) return 0.0f;
+    const int oh = r / g.OW, ow = r - oh * g.OW;
+    const int ih = oh * g.stride_h - g.pad_h + c.dh, iw = ow * g.stride_w - g.pad_w + c.dw;
+    if (static_cast<unsigned>(ih) >= static_cast<unsigned>(g.H) ||
+        static_cast<unsigned>(iw) >= static_cast<unsigned>(g.W))
+      return 0.0f;
+    return x[static_cast<size_t>(img0 + i) * g.C * g.H * g.W + c.off + ih * g.W + iw];
+  }
+  __device__ void store(int m, int n, float v) const {
+    if (m >= M || n >= Ncols) return;
+    partial[static_cast<size_t>(m) * Ncols + n] = v;
+  }
+};
+
+// C[M, Ncols] = A[M, K] x B[K, Ncols], one 128x128 tile per workgroup.
+template <typename Ops>
+__device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
+  using T = Tile;
+  __shared__ float As[2][T::BK][T::PITCH];
+  __shared__ float Bs[2][T::BK][T::PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+
+  // staging roles: A: row a_m, eight consecutive k starting at a_k; B: column
+  // b_n, the eight k of one parity
+  const int a_m = tid >> 1, a_k = (tid & 1) * 8;
+  const int b_n = tid & 127, b_k = tid >> 7;
+  const typename Ops::BCtx bctx = ops.b_ctx(n0 + b_n);
+
+  float16v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  float ra[8], rb[8];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ra[j] = ops.a(m0 + a_m, k0 + a_k + j);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) rb[j] = ops.b(bctx, k0 + b_k + 2 * j);
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) As[buf][a_k + j][a_m] = ra[j];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) Bs[buf][b_k + 2 * j][b_n] = rb[j];
+  };
+
+  const int steps = (ops.K + T::BK - 1) / T::BK;
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  for (int s = 0; s < steps; ++s) {
+    const int buf = s & 1;
+    if (s + 1 < steps) fetch((s + 1) * T::BK);
+    const int half = lane >> 5, col = lane & 31;
+#pragma unroll
+    for (int kk = 0; kk < T::BK; kk += 2) {
+      float a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = As[buf][kk + half][wm + i * 32 + col];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) b[j] = Bs[buf][kk + half][wn + j * 32 + col];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (s + 1 < steps) stage(buf ^ 1);
+    __syncthreads();
+  }
+
+  // accumulator register v of a lane: row 8 * (v / 4) + 4 * (lane / 32) + v % 4, column lane % 32
+  const int half = lane >> 5, col = lane & 31;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = 8 * (v >> 2) + 4 * half + (v & 3);
+        ops.store(m0 + wm + i * 32 + row, n0 + wn + j * 32 + col, acc[i][j][v]);
+      }
+}
+
+template <typename Ops>
+__global__ void __launch_bounds__(Tile::NT)
+igemm_kernel(Ops ops) {
+  igemm_tile(ops, blockIdx.y * Tile::BM, blockIdx.x * Tile::BN);
+}
+
+// One slice of images per blockIdx.z; every slice writes its own partial.
+__global__ void __launch_bounds__(Tile::NT)
+igemm_weight_kernel(BackwardWeightOps ops, int images_per_slice, int total_images) {
+  ops.img0 = blockIdx.z * images_per_slice;
+  ops.images = min(images_per_slice, total_images - ops.img0);
+  ops.K = ops.images * ops.g.OH * ops.g.OW;
+  ops.partial += static_cast<size_t>(blockIdx.z) * ops.M * ops.Ncols;
+  igemm_tile(ops, blockIdx.y * Tile::BM, blockIdx.x * Tile::BN);
+}
+
+// out[i] (+)= sum over slices of partial[s][i]
+__global__ void __launch_bounds__(256)
+reduce_slices_kernel(const float* __restrict__ partial, float* __restrict__ out, long long count,
+                     int slices, int accumulate) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float s = 0.0f;
+  for (int z = 0; z < slices; ++z) s += partial[static_cast<long long>(z) * count + i];
+  out[i] = accumulate ? out[i] + s : s;
+}
+
+// db[d] (+)= sum over images and pixels of dy[img, d, :, :]; one workgroup per filter.
+__global__ void __launch_bounds__(256)
+bias_grad_kernel(const float* __restrict__ dy, float* __restrict__ db, int N, int D, int ohw, int accumulate) {
+  __shared__ float part[256];
+  const int d = blockIdx.x;
+  float s = 0.0f;
+  for (int img = 0; img < N; ++img) {
+    const float* p = dy + (static_cast<size_t>(img) * D + d) * ohw;
+    for (int i = threadIdx.x; i < ohw; i += 256) s += p[i];
+  }
+  part[threadIdx.x] = s;
+  __syncthreads();
+  for (int off = 128; off > 0; off >>= 1) {
+    if (threadIdx.x < off) part[threadIdx.x] += part[threadIdx.x + off];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) db[d] = accumulate ? db[d] + part[0] : part[0];
+}
+
+// The reference's unfold and fold (opzoo/Convolution/Convolution.cpp:13-90), one
+// image per launch: kept for callers that use mobula.func.im2col / col2im directly.
+__global__ void __launch_bounds__(256)
+im2col_kernel(long long n, const float* __restrict__ im, int H, int W, int KH, int KW, int pad_h,
+              int pad_w, int stride_h, int stride_w, int dil_h, int dil_w, int OH, int OW,
+              float* __restrict__ col) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; idx < n; idx += stride) {
+    long long t = idx;
+    const int ow = t % OW; t /= OW;
+    const int oh = t % OH; t /= OH;
+    const int kw = t % KW; t /= KW;
+    const int kh = t % KH; t /= KH;
+    const int c = static_cast<int>(t);
+    const int ih = -pad_h + kh * dil_h + stride_h * oh, iw = -pad_w + kw * dil_w + stride_w * ow;
+    const bool in = static_cast<unsigned>(ih) < static_cast<unsigned>(H) &&
+                    static_cast<unsigned>(iw) < static_cast<unsigned>(W);
+    col[idx] = in ? im[(static_cast<long long>(c) * H + ih) * W + iw] : 0.0f;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+col2im_kernel(long long n, const float* __restrict__ col, int H, int W, int KH, int KW, int pad_h,
+              int pad_w, int stride_h, int stride_w, int dil_h, int dil_w, int OH, int OW,
+              float* __restrict__ im) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  const int ext_w = (KW - 1) * dil_w + 1, ext_h = (KH - 1) * dil_h + 1;
+  for (long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; idx < n; idx += stride) {
+    const int w_im = idx % W + pad_w, h_im = (idx / W) % H + pad_h;
+    const int c = static_cast<int>(idx / (static_cast<long long>(W) * H));
+    const int w0 = w_im < ext_w ? 0 : (w_im - ext_w) / stride_w + 1, w1 = min(w_im / stride_w + 1, OW);
+    const int h0 = h_im < ext_h ? 0 : (h_im - ext_h) / stride_h + 1, h1 = min(h_im / stride_h + 1, OH);
+    float v = 0.0f;
+    for (int oh = h0; oh < h1; ++oh)
+      for (int ow = w0; ow < w1; ++ow) {
+        int hk = h_im - oh * stride_h, wk = w_im - ow * stride_w;
+        if (hk % dil_h == 0 && wk % dil_w == 0) {
+          hk /= dil_h; wk /= dil_w;
+          v += col[((static_cast<long long>(c) * KH + hk) * KW + wk) * OH * OW + static_cast<long long>(oh) * OW + ow];
+        }
+      }
+    im[idx] = v;
+  }
+}
+
+}  // namespace conv

@@ -89,6 +89,12 @@ class SideStream {
   hipEvent_t joined_ = nullptr;
 };
 
+// Every operator source adds the names of its entry points to the list that
+// mobula_hip_exports() returns:  static ExportRegistrar r("name_a name_b");
+struct ExportRegistrar {
+  explicit ExportRegistrar(const char* names);
+};
+
 // With the option "kernel_timing" set, brackets the launches issued during its
 // lifetime with HIP events on `stream`; mobula_hip_last_kernel_ms() then
 // reports the elapsed time of the calling thread's last bracket.

@@ -113,6 +113,18 @@ SideState& side_state(int device) {
 }
 }  // namespace
 
+namespace {
+std::string& export_list() {
+  static std::string names = "set_device";
+  return names;
+}
+}  // namespace
+
+ExportRegistrar::ExportRegistrar(const char* names) {
+  export_list() += " ";
+  export_list() += names;
+}
+
 SideStream::SideStream(hipStream_t main) : main_(main), side_(main) {
   if (option("side_stream", 1) == 0) return;
   int device = 0;
@@ -221,6 +233,8 @@ int mobula_hip_set_option(const char* name, long long value) {
 }
 
 long long mobula_hip_get_option(const char* name) { return mobula_hip::option(name, -1); }
+
+const char* mobula_hip_exports(void) { return mobula_hip::export_list().c_str(); }
 
 double mobula_hip_last_kernel_ms(const char** name) {
   mobula_hip::TimerState& t = mobula_hip::timer_state();

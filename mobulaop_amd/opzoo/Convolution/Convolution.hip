@@ -1,0 +1,321 @@
+// Convolution launchers for gfx950 and their C-ABI entry points.
+//
+// im2col / col2im have the argument lists of the reference kernels
+// (opzoo/Convolution/Convolution.cpp:13-90) and are what
+// `mobula.func.im2col / col2im` bind to.  The conv2d_* launchers have no
+// counterpart in the reference: they are the whole products the reference's
+// operator assembles from im2col/col2im and the framework's matrix product
+// (opzoo/Convolution/Convolution.py:17-57), computed on the matrix cores
+// without a column buffer.
+#include <algorithm>
+
+#include "runtime.h"
+#include "conv_igemm.hip.h"
+
+namespace {
+
+using mobula_hip::arg_extent;
+using mobula_hip::call_state;
+using mobula_hip::failed;
+using mobula_hip::set_error;
+
+int blocks_for(long long n) { return static_cast<int>(std::min<long long>((n + 255) / 256, 256ll * 32)); }
+
+bool fits(const char* what, int arg, long long need) {
+  const long long have = arg_extent(arg);
+  if (have >= 0 && have < need) {
+    set_error("%s: argument %d holds %lld elements, the shape needs %lld", what, arg, have, need);
+    return false;
+  }
+  return true;
+}
+
+// Fills g from the scalar arguments; false (with the error text set) if they
+// do not describe a convolution.
+bool describe(conv::Geometry* g, const char* what, int N, int C, int H, int W, int D, int KH, int KW,
+              int pad_h, int pad_w, int stride_h, int stride_w, int dil_h, int dil_w) {
+  if (N < 0 || C <= 0 || H <= 0 || W <= 0 || D <= 0 || KH <= 0 || KW <= 0 || pad_h < 0 || pad_w < 0 ||
+      stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0) {
+    set_error("%s: invalid shape N=%d C=%d H=%d W=%d D=%d K=%dx%d pad=%d,%d stride=%d,%d dilation=%d,%d",
+              what, N, C, H, W, D, KH, KW, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w);
+    return false;
+  }
+  const int eh = (KH - 1) * dil_h + 1, ew = (KW - 1) * dil_w + 1;
+  if (H + 2 * pad_h < eh || W + 2 * pad_w < ew) {
+    set_error("%s: the %dx%d window does not fit the padded %dx%d input", what, eh, ew, H + 2 * pad_h,
+              W + 2 * pad_w);
+    return false;
+  }
+  g->N = N; g->C = C; g->H = H; g->W = W; g->D = D; g->KH = KH; g->KW = KW;
+  g->pad_h = pad_h; g->pad_w = pad_w; g->stride_h = stride_h; g->stride_w = stride_w;
+  g->dil_h = dil_h; g->dil_w = dil_w;
+  g->OH = (H + 2 * pad_h - eh) / stride_h + 1;
+  g->OW = (W + 2 * pad_w - ew) / stride_w + 1;
+  const long long in = static_cast<long long>(N) * C * H * W, out = static_cast<long long>(N) * D * g->OH * g->OW;
+  const long long wt = static_cast<long long>(D) * C * KH * KW;
+  if (in >= (1ll << 31) || out >= (1ll << 31) || wt >= (1ll << 31) || KH * dil_h > 32767 || KW * dil_w > 32767) {
+    set_error("%s: tensors beyond 32-bit indexing are not supported", what);
+    return false;
+  }
+  return true;
+}
+
+conv::Tap* make_taps(int count, int KH, int KW, int plane, int dil_h, int dil_w, size_t extra_bytes,
+                     char** extra, hipStream_t stream) {
+  const size_t tap_bytes = (sizeof(conv::Tap) * count + 255) / 256 * 256;
+  char* ws = static_cast<char*>(mobula_hip::workspace(tap_bytes + extra_bytes));
+  if (failed()) return nullptr;
+  conv::Tap* taps = reinterpret_cast<conv::Tap*>(ws);
+  if (extra != nullptr) *extra = ws + tap_bytes;
+  conv::build_taps_kernel<<<(count + 255) / 256, 256, 0, stream>>>(taps, count, KH, KW, plane, dil_h, dil_w);
+  return taps;
+}
+
+dim3 tiles(long long M, long long Ncols, int z = 1) {
+  return dim3(static_cast<unsigned>((Ncols + conv::Tile::BN - 1) / conv::Tile::BN),
+              static_cast<unsigned>((M + conv::Tile::BM - 1) / conv::Tile::BM), static_cast<unsigned>(z));
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// Launchers (scanned by the Python loader).
+// ---------------------------------------------------------------------------
+
+// One image: data_col[c, kh, kw, oh, ow] = data_im[c, ih, iw] or 0 in the padding.
+template <typename T>
+MOBULA_KERNEL im2col_kernel(const int n, const T* data_im, const int height, const int width,
+                            const int kernel_h, const int kernel_w, const int pad_h, const int pad_w,
+                            const int stride_h, const int stride_w, const int dilation_h,
+                            const int dilation_w, const int height_col, const int width_col,
+                            T* data_col) {
+  if (n <= 0) return;
+  if (!fits("im2col", 14, n)) return;
+  conv::im2col_kernel<<<blocks_for(n), 256, 0, call_state().stream>>>(
+      n, data_im, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h,
+      dilation_w, height_col, width_col, data_col);
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+// One image: data_im[c, h, w] = sum of the column entries that were read from it.
+template <typename T>
+MOBULA_KERNEL col2im_kernel(const int n, const T* data_col, const int height, const int width,
+                            const int kernel_h, const int kernel_w, const int pad_h, const int pad_w,
+                            const int stride_h, const int stride_w, const int dilation_h,
+                            const int dilation_w, const int height_col, const int width_col,
+                            T* data_im) {
+  if (n <= 0) return;
+  if (!fits("col2im", 14, n)) return;
+  conv::col2im_kernel<<<blocks_for(n), 256, 0, call_state().stream>>>(
+      n, data_col, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h,
+      dilation_w, height_col, width_col, data_im);
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+// y[N, D, OH, OW] = conv(x[N, C, H, W], weight[D, C, KH, KW]) (+ bias[D] if has_bias).
+// n is the element count of y.
+template <typename T>
+MOBULA_KERNEL conv2d_forward_kernel(const int n, const T* x, const T* weight, const T* bias,
+                                    const int has_bias, const int batch, const int channels,
+                                    const int height, const int width, const int filters,
+                                    const int kernel_h, const int kernel_w, const int pad_h,
+                                    const int pad_w, const int stride_h, const int stride_w,
+                                    const int dilation_h, const int dilation_w, T* y) {
+  conv::Geometry g;
+  if (!describe(&g, "conv2d_forward", batch, channels, height, width, filters, kernel_h, kernel_w, pad_h,
+                pad_w, stride_h, stride_w, dilation_h, dilation_w))
+    return;
+  const long long out = static_cast<long long>(g.N) * g.D * g.OH * g.OW;
+  if (n != out) { set_error("conv2d_forward: n=%d, the output has %lld elements", n, out); return; }
+  if (!fits("conv2d_forward", 1, static_cast<long long>(g.N) * g.C * g.H * g.W) ||
+      !fits("conv2d_forward", 2, static_cast<long long>(g.D) * g.C * g.KH * g.KW) ||
+      (has_bias && !fits("conv2d_forward", 3, g.D)) || !fits("conv2d_forward", 18, out))
+    return;
+  if (out == 0) return;
+  hipStream_t stream = call_state().stream;
+  conv::ForwardOps ops;
+  ops.x = x; ops.w = weight; ops.bias = has_bias ? bias : nullptr; ops.y = y; ops.g = g;
+  ops.M = g.D; ops.Ncols = g.N * g.OH * g.OW; ops.K = g.C * g.KH * g.KW;
+  ops.taps = make_taps(ops.K, g.KH, g.KW, g.H * g.W, g.dil_h, g.dil_w, 0, nullptr, stream);
+  if (failed()) return;
+  {
+    mobula_hip::KernelTimer timer("conv2d_forward", stream);
+    conv::igemm_kernel<conv::ForwardOps><<<tiles(ops.M, ops.Ncols), conv::Tile::NT, 0, stream>>>(ops);
+  }
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+// dx[N, C, H, W] (+)= the gradient of conv2d_forward with respect to x.  n is the
+// element count of dx.
+template <typename T>
+MOBULA_KERNEL conv2d_backward_data_kernel(const int n, const T* dy, const T* weight, const int accumulate,
+                                          const int batch, const int channels, const int height,
+                                          const int width, const int filters, const int kernel_h,
+                                          const int kernel_w, const int pad_h, const int pad_w,
+                                          const int stride_h, const int stride_w, const int dilation_h,
+                                          const int dilation_w, T* dx) {
+  conv::Geometry g;
+  if (!describe(&g, "conv2d_backward_data", batch, channels, height, width, filters, kernel_h, kernel_w,
+                pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w))
+    return;
+  const long long in = static_cast<long long>(g.N) * g.C * g.H * g.W;
+  if (n != in) { set_error("conv2d_backward_data: n=%d, dx has %lld elements", n, in); return; }
+  if (!fits("conv2d_backward_data", 1, static_cast<long long>(g.N) * g.D * g.OH * g.OW) ||
+      !fits("conv2d_backward_data", 2, static_cast<long long>(g.D) * g.C * g.KH * g.KW) ||
+      !fits("conv2d_backward_data", 17, in))
+    return;
+  if (in == 0) return;
+  hipStream_t stream = call_state().stream;
+  conv::BackwardDataOps ops;
+  ops.dy = dy; ops.w = weight; ops.dx = dx; ops.g = g; ops.accumulate = accumulate;
+  ops.M = g.C; ops.Ncols = g.N * g.H * g.W; ops.K = g.D * g.KH * g.KW;
+  ops.taps = make_taps(ops.K, g.KH, g.KW, g.OH * g.OW, g.dil_h, g.dil_w, 0, nullptr, stream);
+  if (failed()) return;
+  {
+    mobula_hip::KernelTimer timer("conv2d_backward_data", stream);
+    conv::igemm_kernel<conv::BackwardDataOps><<<tiles(ops.M, ops.Ncols), conv::Tile::NT, 0, stream>>>(ops);
+  }
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+// dw[D, C, KH, KW] (+)= the gradient with respect to the weights.  n is the
+// element count of dw.
+template <typename T>
+MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x, const int accumulate,
+                                            const int batch, const int channels, const int height,
+                                            const int width, const int filters, const int kernel_h,
+                                            const int kernel_w, const int pad_h, const int pad_w,
+                                            const int stride_h, const int stride_w, const int dilation_h,
+                                            const int dilation_w, T* dw) {
+  conv::Geometry g;
+  if (!describe(&g, "conv2d_backward_weight", batch, channels, height, width, filters, kernel_h, kernel_w,
+                pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w))
+    return;
+  const long long wt = static_cast<long long>(g.D) * g.C * g.KH * g.KW;
+  if (n != wt) { set_error("conv2d_backward_weight: n=%d, dw has %lld elements", n, wt); return; }
+  if (!fits("conv2d_backward_weight", 1, static_cast<long long>(g.N) * g.D * g.OH * g.OW) ||
+      !fits("conv2d_backward_weight", 2, static_cast<long long>(g.N) * g.C * g.H * g.W) ||
+      !fits("conv2d_backward_weight", 17, wt))
+    return;
+  hipStream_t stream = call_state().stream;
+  conv::BackwardWeightOps ops;
+  ops.dy = dy; ops.x = x; ops.g = g;
+  ops.M = g.D; ops.Ncols = g.C * g.KH * g.KW; ops.K = 0; ops.img0 = 0; ops.images = 0;
+  // K = N*OH*OW is long and the result small: slices of images go to different
+  // workgroups, their partial sums are added in a fixed order afterwards.
+  const dim3 one = tiles(ops.M, ops.Ncols);
+  const long long per_slice_tiles = static_cast<long long>(one.x) * one.y;
+  int slices = static_cast<int>(std::min<long long>(std::max(g.N, 1), std::max<long long>(1, 1024 / per_slice_tiles)));
+  const int images_per_slice = g.N > 0 ? (g.N + slices - 1) / slices : 1;
+  slices = g.N > 0 ? (g.N + images_per_slice - 1) / images_per_slice : 1;
+  char* extra = nullptr;
+  ops.taps = make_taps(ops.Ncols, g.KH, g.KW, g.H * g.W, g.dil_h, g.dil_w,
+                       sizeof(float) * static_cast<size_t>(slices) * wt, &extra, stream);
+  if (failed()) return;
+  ops.partial = reinterpret_cast<float*>(extra);
+  {
+    mobula_hip::KernelTimer timer("conv2d_backward_weight", stream);
+    conv::igemm_weight_kernel<<<tiles(ops.M, ops.Ncols, slices), conv::Tile::NT, 0, stream>>>(
+        ops, images_per_slice, g.N);
+    conv::reduce_slices_kernel<<<blocks_for(wt), 256, 0, stream>>>(ops.partial, dw, wt, slices, accumulate);
+  }
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+// db[D] (+)= sum of dy over images and pixels.  n = D.
+template <typename T>
+MOBULA_KERNEL conv2d_backward_bias_kernel(const int n, const T* dy, const int accumulate, const int batch,
+                                          const int pixels, T* db) {
+  if (n <= 0) return;
+  if (batch < 0 || pixels < 0) { set_error("conv2d_backward_bias: batch=%d pixels=%d", batch, pixels); return; }
+  if (!fits("conv2d_backward_bias", 1, static_cast<long long>(batch) * n * pixels) ||
+      !fits("conv2d_backward_bias", 5, n))
+    return;
+  conv::bias_grad_kernel<<<n, 256, 0, call_state().stream>>>(dy, db, batch, n, pixels, accumulate);
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------
+// Entry points.  Device pointers only: the convolution does not stage host
+// buffers (device id -1 is an error here).
+// ---------------------------------------------------------------------------
+namespace {
+bool on_device(const char* what, int device_id) {
+  if (device_id >= 0) return true;
+  set_error("%s: host buffers are not supported, pass device tensors", what);
+  mobula_hip::finish_call();
+  return false;
+}
+}  // namespace
+
+#define CONV_GEOMETRY_PARAMS                                                                          \
+  const int batch, const int channels, const int height, const int width, const int filters,          \
+      const int kernel_h, const int kernel_w, const int pad_h, const int pad_w, const int stride_h,   \
+      const int stride_w, const int dilation_h, const int dilation_w
+#define CONV_GEOMETRY_ARGS                                                                             \
+  batch, channels, height, width, filters, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,       \
+      dilation_h, dilation_w
+
+extern "C" {
+
+void im2col_341af5d3(const int device_id, const int n, const float* data_im, const int height,
+                     const int width, const int kernel_h, const int kernel_w, const int pad_h,
+                     const int pad_w, const int stride_h, const int stride_w, const int dilation_h,
+                     const int dilation_w, const int height_col, const int width_col, float* data_col) {
+  if (!on_device("im2col", device_id)) return;
+  mobula_hip::DeviceScope scope(device_id);
+  if (scope.ok())
+    im2col_kernel<float>(n, data_im, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
+                         dilation_h, dilation_w, height_col, width_col, data_col);
+  mobula_hip::finish_call();
+}
+
+void col2im_341af5d3(const int device_id, const int n, const float* data_col, const int height,
+                     const int width, const int kernel_h, const int kernel_w, const int pad_h,
+                     const int pad_w, const int stride_h, const int stride_w, const int dilation_h,
+                     const int dilation_w, const int height_col, const int width_col, float* data_im) {
+  if (!on_device("col2im", device_id)) return;
+  mobula_hip::DeviceScope scope(device_id);
+  if (scope.ok())
+    col2im_kernel<float>(n, data_col, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
+                         dilation_h, dilation_w, height_col, width_col, data_im);
+  mobula_hip::finish_call();
+}
+
+void conv2d_forward_c6a7aa85(const int device_id, const int n, const float* x, const float* weight,
+                            const float* bias, const int has_bias, CONV_GEOMETRY_PARAMS, float* y) {
+  if (!on_device("conv2d_forward", device_id)) return;
+  mobula_hip::DeviceScope scope(device_id);
+  if (scope.ok()) conv2d_forward_kernel<float>(n, x, weight, bias, has_bias, CONV_GEOMETRY_ARGS, y);
+  mobula_hip::finish_call();
+}
+
+void conv2d_backward_data_ecf81c91(const int device_id, const int n, const float* dy, const float* weight,
+                                  const int accumulate, CONV_GEOMETRY_PARAMS, float* dx) {
+  if (!on_device("conv2d_backward_data", device_id)) return;
+  mobula_hip::DeviceScope scope(device_id);
+  if (scope.ok()) conv2d_backward_data_kernel<float>(n, dy, weight, accumulate, CONV_GEOMETRY_ARGS, dx);
+  mobula_hip::finish_call();
+}
+
+void conv2d_backward_weight_ecf81c91(const int device_id, const int n, const float* dy, const float* x,
+                                    const int accumulate, CONV_GEOMETRY_PARAMS, float* dw) {
+  if (!on_device("conv2d_backward_weight", device_id)) return;
+  mobula_hip::DeviceScope scope(device_id);
+  if (scope.ok()) conv2d_backward_weight_kernel<float>(n, dy, x, accumulate, CONV_GEOMETRY_ARGS, dw);
+  mobula_hip::finish_call();
+}
+
+void conv2d_backward_bias_cd239a08(const int device_id, const int n, const float* dy, const int accumulate,
+                                   const int batch, const int pixels, float* db) {
+  if (!on_device("conv2d_backward_bias", device_id)) return;
+  mobula_hip::DeviceScope scope(device_id);
+  if (scope.ok()) conv2d_backward_bias_kernel<float>(n, dy, accumulate, batch, pixels, db);
+  mobula_hip::finish_call();
+}
+
+}  // extern "C"
+
+static mobula_hip::ExportRegistrar conv_exports(
+    "im2col_341af5d3 col2im_341af5d3 conv2d_forward_c6a7aa85 conv2d_backward_data_ecf81c91 "
+    "conv2d_backward_weight_ecf81c91 conv2d_backward_bias_cd239a08");

@@ -473,8 +473,8 @@ void roi_align_forward_e874c59a(const int device_id, const int nthreads, const _
                         pooled_height, pooled_width, sampling_ratio, bottom_rois, top_data);
 }
 
-const char* mobula_hip_exports(void) {
-  return "roi_align_forward_ab78de3c roi_align_backward_f318a24e "
-         "roi_align_backward_assign_a8793cbe roi_align_forward_e874c59a set_device";
-}
-}
+}  // extern "C"
+
+static mobula_hip::ExportRegistrar roialign_exports(
+    "roi_align_forward_ab78de3c roi_align_backward_f318a24e roi_align_backward_assign_a8793cbe "
+    "roi_align_forward_e874c59a");
