@@ -51,14 +51,28 @@ build_taps_kernel(Tap* __restrict__ taps, int count, int KH, int KW, int plane, 
 }
 
 // ---- operand functors -------------------------------------------------------
-// a(m, k): element of the left operand; BCtx b_ctx(n) + b(ctx, k): element of
-// the right operand for a fixed column n; store(m, n, v).
+// fetch_a(m, k, out): the eight elements A[m][k .. k+7] of the left operand;
+// BCtx b_ctx(n) + fetch_b(ctx, k, out): the eight elements B[k + 2j][n], j < 8,
+// of the right operand (k is the same for a whole wavefront, so everything
+// that depends only on k is scalar); store(m, n, v).  Elements outside the
+// operands are zero.
 
 struct ForwardOps {
-  const float* x; const float* w; const float* bias; float* y; const Tap* taps;
+  const float* __restrict__ x; const float* __restrict__ w; const float* __restrict__ bias;
+  float* __restrict__ y; const Tap* __restrict__ taps;
   Geometry g; int M, Ncols, K;
   struct BCtx { int base; int ih0, iw0; bool ok; };
-  __device__ float a(int m, int k) const { return (m < M && k < K) ? w[static_cast<size_t>(m) * K + k] : 0.0f; }
+  __device__ void fetch_a(int m, int k, float (&out)[8]) const {
+    const size_t at = static_cast<size_t>(m) * K + k;
+    if (m < M && k + 8 <= K && (at & 3) == 0) {
+      const float4 lo = *reinterpret_cast<const float4*>(w + at), hi = *reinterpret_cast<const float4*>(w + at + 4);
+      out[0] = lo.x; out[1] = lo.y; out[2] = lo.z; out[3] = lo.w;
+      out[4] = hi.x; out[5] = hi.y; out[6] = hi.z; out[7] = hi.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) out[j] = (m < M && k + j < K) ? w[at + j] : 0.0f;
+    }
+  }
   __device__ BCtx b_ctx(int n) const {
     BCtx c;
     c.ok = n < Ncols;
@@ -68,14 +82,16 @@ struct ForwardOps {
     c.base = img * g.C * g.H * g.W + c.ih0 * g.W + c.iw0;
     return c;
   }
-  __device__ float b(const BCtx& c, int k) const {
-    if (!c.ok || k >= K) return 0.0f;
-    const Tap t = taps[k];
-    const int ih = c.ih0 + t.dh, iw = c.iw0 + t.dw;
-    if (static_cast<unsigned>(ih) >= static_cast<unsigned>(g.H) ||
-        static_cast<unsigned>(iw) >= static_cast<unsigned>(g.W))
-      return 0.0f;
-    return x[c.base + t.off + t.dh * g.W + t.dw];
+  __device__ void fetch_b(const BCtx& c, int k, float (&out)[8]) const {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kk = k + 2 * j;
+      const Tap t = taps[min(kk, K - 1)];   // scalar load: kk is uniform
+      const int ih = c.ih0 + t.dh, iw = c.iw0 + t.dw;
+      const bool in = c.ok && kk < K && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
+                      static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
+      out[j] = in ? x[c.base + t.off + t.dh * g.W + t.dw] : 0.0f;
+    }
   }
   __device__ void store(int m, int n, float v) const {
     if (m >= M || n >= Ncols) return;
@@ -87,13 +103,18 @@ struct ForwardOps {
 // dx[img, c, ih, iw] = sum over (d, kh, kw) of W[d, c, kh, kw] * dy[img, d, oh, ow]
 // with oh * stride = ih + pad - kh * dil (and likewise for columns).
 struct BackwardDataOps {
-  const float* dy; const float* w; float* dx; const Tap* taps;   // taps over dy: off = d * OH*OW
+  const float* __restrict__ dy; const float* __restrict__ w; float* __restrict__ dx;
+  const Tap* __restrict__ taps;   // taps over dy: off = d * OH*OW
   Geometry g; int M, Ncols, K; int accumulate;
   struct BCtx { int base; int ihp, iwp; bool ok; };
-  __device__ float a(int m, int k) const {
-    if (m >= M || k >= K) return 0.0f;
-    const int khw = g.KH * g.KW, d = k / khw, r = k - d * khw;
-    return w[(static_cast<size_t>(d) * g.C + m) * khw + r];
+  __device__ void fetch_a(int m, int k, float (&out)[8]) const {
+    const int khw = g.KH * g.KW;
+    int d = k / khw, r = k - d * khw;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      out[j] = (m < M && k + j < K) ? w[(static_cast<size_t>(d) * g.C + m) * khw + r] : 0.0f;
+      if (++r == khw) { r = 0; ++d; }
+    }
   }
   __device__ BCtx b_ctx(int n) const {
     BCtx c;
@@ -103,14 +124,22 @@ struct BackwardDataOps {
     c.base = img * g.D * g.OH * g.OW;
     return c;
   }
-  __device__ float b(const BCtx& c, int k) const {
-    if (!c.ok || k >= K) return 0.0f;
-    const Tap t = taps[k];
-    const int th = c.ihp - t.dh, tw = c.iwp - t.dw;
-    if (th < 0 || tw < 0) return 0.0f;
-    const int oh = th / g.stride_h, ow = tw / g.stride_w;
-    if (oh * g.stride_h != th || ow * g.stride_w != tw || oh >= g.OH || ow >= g.OW) return 0.0f;
-    return dy[c.base + t.off + oh * g.OW + ow];
+  __device__ void fetch_b(const BCtx& c, int k, float (&out)[8]) const {
+    const bool unit = g.stride_h == 1 && g.stride_w == 1;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kk = k + 2 * j;
+      const Tap t = taps[min(kk, K - 1)];
+      const int th = c.ihp - t.dh, tw = c.iwp - t.dw;
+      int oh = th, ow = tw;
+      bool in = c.ok && kk < K && th >= 0 && tw >= 0;
+      if (!unit) {
+        oh = th / g.stride_h; ow = tw / g.stride_w;
+        in = in && oh * g.stride_h == th && ow * g.stride_w == tw;
+      }
+      in = in && oh < g.OH && ow < g.OW;
+      out[j] = in ? dy[c.base + t.off + oh * g.OW + ow] : 0.0f;
+    }
   }
   __device__ void store(int m, int n, float v) const {
     if (m >= M || n >= Ncols) return;
@@ -123,14 +152,19 @@ struct BackwardDataOps {
 // partial[z][d, (c, kh, kw)] = sum over the images of slice z and (oh, ow) of
 // dy[img, d, oh, ow] * x[img, c, ih, iw].
 struct BackwardWeightOps {
-  const float* dy; const float* x; float* partial; const Tap* taps;   // taps over x
+  const float* __restrict__ dy; const float* __restrict__ x; float* __restrict__ partial;
+  const Tap* __restrict__ taps;   // taps over x
   Geometry g; int M, Ncols, K;   // K = images_per_slice * OH*OW
   int img0, images;              // the images of this slice
   struct BCtx { int off; int dh, dw; bool ok; };
-  __device__ float a(int m, int k) const {
-    const int ohw = g.OH * g.OW, i = k / ohw, r = k - i * ohw;
-    if (m >= M || i >= images) return 0.0f;
-    return dy[(static_cast<size_t>(img0 + i) * g.D + m) * ohw + r];
+  __device__ void fetch_a(int m, int k, float (&out)[8]) const {
+    const int ohw = g.OH * g.OW;
+    int i = k / ohw, r = k - i * ohw;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      out[j] = (m < M && i < images) ? dy[(static_cast<size_t>(img0 + i) * g.D + m) * ohw + r] : 0.0f;
+      if (++r == ohw) { r = 0; ++i; }
+    }
   }
   __device__ BCtx b_ctx(int n) const {
     BCtx c;
@@ -139,15 +173,19 @@ struct BackwardWeightOps {
     c.off = t.off; c.dh = t.dh; c.dw = t.dw;
     return c;
   }
-  __device__ float b(const BCtx& c, int k) const {
-    const int ohw = g.OH * g.OW, i = k / ohw, r = k - i * ohw;
-    if (!c.ok || i >= images) return 0.0f;
-    const int oh = r / g.OW, ow = r - oh * g.OW;
-    const int ih = oh * g.stride_h - g.pad_h + c.dh, iw = ow * g.stride_w - g.pad_w + c.dw;
-    if (static_cast<unsigned>(ih) >= static_cast<unsigned>(g.H) ||
-        static_cast<unsigned>(iw) >= static_cast<unsigned>(g.W))
-      return 0.0f;
-    return x[static_cast<size_t>(img0 + i) * g.C * g.H * g.W + c.off + ih * g.W + iw];
+  __device__ void fetch_b(const BCtx& c, int k, float (&out)[8]) const {
+    const int ohw = g.OH * g.OW;
+    int i = k / ohw, r = k - i * ohw;   // scalar: k is uniform
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int oh = r / g.OW, ow = r - oh * g.OW;
+      const int ih = oh * g.stride_h - g.pad_h + c.dh, iw = ow * g.stride_w - g.pad_w + c.dw;
+      const bool in = c.ok && i < images && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
+                      static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
+      out[j] = in ? x[static_cast<size_t>(img0 + i) * g.C * g.H * g.W + c.off + ih * g.W + iw] : 0.0f;
+      r += 2;
+      if (r >= ohw) { r -= ohw; ++i; }
+    }
   }
   __device__ void store(int m, int n, float v) const {
     if (m >= M || n >= Ncols) return;
@@ -167,7 +205,7 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
   // staging roles: A: row a_m, eight consecutive k starting at a_k; B: column
   // b_n, the eight k of one parity
   const int a_m = tid >> 1, a_k = (tid & 1) * 8;
-  const int b_n = tid & 127, b_k = tid >> 7;
+  const int b_n = tid & 127, b_k = __builtin_amdgcn_readfirstlane(tid >> 7);   // the same for a wavefront
   const typename Ops::BCtx bctx = ops.b_ctx(n0 + b_n);
 
   float16v acc[2][2];
@@ -180,10 +218,8 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
 
   float ra[8], rb[8];
   auto fetch = [&](int k0) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) ra[j] = ops.a(m0 + a_m, k0 + a_k + j);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) rb[j] = ops.b(bctx, k0 + b_k + 2 * j);
+    ops.fetch_a(m0 + a_m, k0 + a_k, ra);
+    ops.fetch_b(bctx, k0 + b_k, rb);
   };
   auto stage = [&](int buf) {
 #pragma unroll
