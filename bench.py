@@ -67,18 +67,111 @@ def cpu_baseline(w, budget_s=25.0):
                 n, R, w['name'], 'fwd+bwd' if w['dy'] is not None else 'fwd only', dt)}
 
 
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
+
+
+def bench_conv(args):
+    """cfg5: opzoo Conv2D, N=32, 256 -> 256 channels, 56x56, 3x3, stride 1, pad 1, fp32.
+    One step = forward + data gradient + weight gradient through the C ABI."""
+    import torch
+    from mobulaop_amd import native
+    assert torch.cuda.is_available(), 'bench.py needs a GPU'
+    N, C, H, W, D, K = 32, 256, 56, 56, 256, 3
+    g = torch.Generator().manual_seed(1005)
+    x = torch.randn(N, C, H, W, generator=g).cuda()
+    w = (torch.randn(D, C, K, K, generator=g) * (2.0 / (C * K * K)) ** 0.5).cuda()
+    dy = torch.randn(N, D, H, W, generator=g).cuda()
+    y, dx, dw = torch.empty_like(dy), torch.empty_like(x), torch.empty_like(w)
+    lib = native.library()
+    lib.mobula_hip_last_kernel_ms.restype = ctypes.c_double
+    lib.mobula_hip_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_char_p)]
+    stream = torch.cuda.current_stream().cuda_stream
+    geo = [ctypes.c_int(v) for v in (N, C, H, W, D, K, K, 1, 1, 1, 1, 1, 1)]
+
+    def ptr(t):
+        return ctypes.c_void_p(t.data_ptr())
+
+    def call(fn, *a):
+        native.begin_call(stream, [])
+        fn(ctypes.c_int(0), *a)
+        native.end_call(fn.__name__)
+
+    calls = [
+        lambda: call(lib.conv2d_forward_c6a7aa85, ctypes.c_int(y.numel()), ptr(x), ptr(w), ptr(w),
+                     ctypes.c_int(0), *geo, ptr(y)),
+        lambda: call(lib.conv2d_backward_data_ecf81c91, ctypes.c_int(dx.numel()), ptr(dy), ptr(w),
+                     ctypes.c_int(0), *geo, ptr(dx)),
+        lambda: call(lib.conv2d_backward_weight_ecf81c91, ctypes.c_int(dw.numel()), ptr(dy), ptr(x),
+                     ctypes.c_int(0), *geo, ptr(dw)),
+    ]
+
+    def step():
+        for c in calls:
+            c()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    native.set_option('kernel_timing', 1)
+    kernel_ms = {}
+    for _ in range(args.steps):
+        for c in calls:
+            c()
+            name = ctypes.c_char_p()
+            ms = lib.mobula_hip_last_kernel_ms(ctypes.byref(name))
+            if ms >= 0 and name.value:
+                kernel_ms.setdefault(name.value.decode(), []).append(ms)
+    native.set_option('kernel_timing', 0)
+    kernel_ms = {k: sum(v) / len(v) for k, v in kernel_ms.items()}
+    flops_each = 2.0 * N * D * H * W * C * K * K          # per product; three products per step
+    dom = max(kernel_ms, key=kernel_ms.get)
+    achieved = flops_each / (kernel_ms[dom] * 1e-3) / 1e12
+    out = {
+        'metric': 'conv2d_fwd_bwd_tflops', 'value': 3 * flops_each / (ms_per_step * 1e-3) / 1e12,
+        'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'cfg5: conv2d x 32x256x56x56, 256 filters 3x3 stride 1 pad 1',
+                   'step': 'forward + data gradient + weight gradient'},
+        'roofline': {'bound': 'mfma', 'kernel': dom, 'achieved': achieved, 'peak': MFMA_FP32_PEAK_TFLOPS,
+                     'unit': 'TFLOP/s', 'frac': achieved / MFMA_FP32_PEAK_TFLOPS, 'traffic': None,
+                     'algorithmic_flops': flops_each, 'avg_ms': kernel_ms[dom]},
+        'kernels_ms': kernel_ms,
+    }
+    if not args.no_cpu_baseline:
+        # the C restatement of the reference algorithm (im2col + product per image), one thread,
+        # on the first image of the same tensors
+        from oracle import conv as oracle
+        xs, ws, dys = x[:1].cpu().numpy(), w.cpu().numpy(), dy[:1].cpu().numpy()
+        t0 = time.perf_counter()
+        oracle.conv2d_forward(xs, ws, None, (1, 1), (1, 1), (1, 1))
+        oracle.conv2d_backward(dys, xs, ws, (1, 1), (1, 1), (1, 1), with_bias=False)
+        dt = time.perf_counter() - t0
+        out['cpu_baseline'] = {'value': 3 * flops_each / N / dt / 1e12, 'unit': 'TFLOP/s', 'cores': 1,
+                               'kind': 'port', 'sample': 'first image of 32, one pass, {:.2f} s'.format(dt)}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=30)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workload', default='cfg2', choices=['cfg1', 'cfg2', 'cfg3', 'cfg4'])
+    ap.add_argument('--workload', default='cfg2', choices=['cfg1', 'cfg2', 'cfg3', 'cfg4', 'cfg5'])
     ap.add_argument('--impl', default='auto', choices=['auto', 'tiled', 'naive'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build measures one GPU only (the path shards by image with no '
                  'exchange; see DESIGN.md); run with --gpus 1')
+
+    if args.workload == 'cfg5':
+        return bench_conv(args)
 
     import torch
     from mobulaop_amd import workloads
