@@ -68,11 +68,14 @@ def cpu_baseline(w, budget_s=25.0):
 
 
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 
 
 def bench_conv(args):
-    """cfg5: opzoo Conv2D, N=32, 256 -> 256 channels, 56x56, 3x3, stride 1, pad 1, fp32.
-    One step = forward + data gradient + weight gradient through the C ABI."""
+    """cfg5: opzoo Conv2D, N=32, 256 -> 256 channels, 56x56, 3x3, stride 1, pad 1; fp32 tensors.
+    One step = forward + data gradient + weight gradient through the C ABI.
+    --conv-compute picks how the products are formed: fp32 matrix cores, operands rounded
+    to bf16, or two bf16 per operand (three products, fp32-like results)."""
     import torch
     from mobulaop_amd import native
     assert torch.cuda.is_available(), 'bench.py needs a GPU'
@@ -87,6 +90,11 @@ def bench_conv(args):
     lib.mobula_hip_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_char_p)]
     stream = torch.cuda.current_stream().cuda_stream
     geo = [ctypes.c_int(v) for v in (N, C, H, W, D, K, K, 1, 1, 1, 1, 1, 1)]
+    mode = {'fp32': 0, 'bf16': 1, 'bf16x3': 2}[args.conv_compute]
+    native.set_option('conv_compute', mode)
+    # dense peak of the matrix-core instruction the products run on; the split mode is
+    # priced on the products that count (one per multiply-add of the convolution)
+    peak = MFMA_FP32_PEAK_TFLOPS if mode == 0 else MFMA_BF16_PEAK_TFLOPS
 
     def ptr(t):
         return ctypes.c_void_p(t.data_ptr())
@@ -135,11 +143,11 @@ def bench_conv(args):
         'metric': 'conv2d_fwd_bwd_tflops', 'value': 3 * flops_each / (ms_per_step * 1e-3) / 1e12,
         'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
-        'dtype': 'f32', 'data': 'synthetic',
+        'dtype': {0: 'f32', 1: 'bf16', 2: 'bf16x3'}[mode], 'data': 'synthetic',
         'config': {'workload': 'cfg5: conv2d x 32x256x56x56, 256 filters 3x3 stride 1 pad 1',
-                   'step': 'forward + data gradient + weight gradient'},
-        'roofline': {'bound': 'mfma', 'kernel': dom, 'achieved': achieved, 'peak': MFMA_FP32_PEAK_TFLOPS,
-                     'unit': 'TFLOP/s', 'frac': achieved / MFMA_FP32_PEAK_TFLOPS, 'traffic': None,
+                   'step': 'forward + data gradient + weight gradient', 'compute': args.conv_compute},
+        'roofline': {'bound': 'mfma', 'kernel': dom, 'achieved': achieved, 'peak': peak,
+                     'unit': 'TFLOP/s', 'frac': achieved / peak, 'traffic': None,
                      'algorithmic_flops': flops_each, 'avg_ms': kernel_ms[dom]},
         'kernels_ms': kernel_ms,
     }
@@ -165,6 +173,8 @@ def main():
     ap.add_argument('--workload', default='cfg2', choices=['cfg1', 'cfg2', 'cfg3', 'cfg4', 'cfg5'])
     ap.add_argument('--impl', default='auto', choices=['auto', 'tiled', 'naive'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--conv-compute', default='fp32', choices=['fp32', 'bf16', 'bf16x3'],
+                    help='cfg5 only: how the convolution forms its products')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build measures one GPU only (the path shards by image with no '

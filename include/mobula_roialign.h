@@ -143,7 +143,9 @@ void mobula_hip_clear_error(void);
 /* Named integer switches ("roialign_impl": 0 auto, 1 tiled, 2 naive;
  * "host_staging_device"; "kernel_timing": 0 off, 1 on; "side_stream": 1 (default)
  * lets helper kernels of a call run on a second stream of the device, 0 keeps
- * everything on the caller's stream).  set returns 0, or -1 for an unknown name; get
+ * everything on the caller's stream; "conv_compute": 0 (default) multiplies the
+ * convolution's fp32 operands as they are, 1 rounds them to bf16 and accumulates
+ * in fp32).  set returns 0, or -1 for an unknown name; get
  * returns -1 for a name never set. */
 int mobula_hip_set_option(const char* name, long long value);
 long long mobula_hip_get_option(const char* name);

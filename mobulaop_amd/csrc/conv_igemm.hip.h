@@ -14,9 +14,10 @@
 //
 // Tiling: a workgroup of four wavefronts owns a 128x128 tile of the result and
 // walks K in steps of 16; each wavefront holds a 64x64 quarter as 2x2
-// accumulators of v_mfma_f32_32x32x2_f32 (64 registers per lane).  The next K
-// step is fetched into registers while the current one is multiplied out of
-// LDS (two LDS buffers, one barrier per step).
+// accumulators of v_mfma_f32_32x32x2_f32 (64 registers per lane), or, with
+// operands rounded to bf16, of v_mfma_f32_32x32x16_bf16.  The next K step is
+// fetched into registers while the current one is multiplied out of LDS (two
+// LDS buffers, one barrier per step).
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -52,7 +53,7 @@ build_taps_kernel(Tap* __restrict__ taps, int count, int KH, int KW, int plane, 
 
 // ---- operand functors -------------------------------------------------------
 // fetch_a(m, k, out): the eight elements A[m][k .. k+7] of the left operand;
-// BCtx b_ctx(n) + fetch_b(ctx, k, out): the eight elements B[k + 2j][n], j < 8,
+// BCtx b_ctx(n) + fetch_b(ctx, k, out): the eight elements B[k .. k+7][n]
 // of the right operand (k is the same for a whole wavefront, so everything
 // that depends only on k is scalar); store(m, n, v).  Elements outside the
 // operands are zero.
@@ -85,7 +86,7 @@ struct ForwardOps {
   __device__ void fetch_b(const BCtx& c, int k, float (&out)[8]) const {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int kk = k + 2 * j;
+      const int kk = k + j;
       const Tap t = taps[min(kk, K - 1)];   // scalar load: kk is uniform
       const int ih = c.ih0 + t.dh, iw = c.iw0 + t.dw;
       const bool in = c.ok && kk < K && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
@@ -128,7 +129,7 @@ struct BackwardDataOps {
     const bool unit = g.stride_h == 1 && g.stride_w == 1;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int kk = k + 2 * j;
+      const int kk = k + j;
       const Tap t = taps[min(kk, K - 1)];
       const int th = c.ihp - t.dh, tw = c.iwp - t.dw;
       int oh = th, ow = tw;
@@ -160,6 +161,13 @@ struct BackwardWeightOps {
   __device__ void fetch_a(int m, int k, float (&out)[8]) const {
     const int ohw = g.OH * g.OW;
     int i = k / ohw, r = k - i * ohw;
+    const size_t at = (static_cast<size_t>(img0 + i) * g.D + m) * ohw + r;
+    if (m < M && i < images && r + 8 <= ohw && (at & 3) == 0) {
+      const float4 lo = *reinterpret_cast<const float4*>(dy + at), hi = *reinterpret_cast<const float4*>(dy + at + 4);
+      out[0] = lo.x; out[1] = lo.y; out[2] = lo.z; out[3] = lo.w;
+      out[4] = hi.x; out[5] = hi.y; out[6] = hi.z; out[7] = hi.w;
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       out[j] = (m < M && i < images) ? dy[(static_cast<size_t>(img0 + i) * g.D + m) * ohw + r] : 0.0f;
@@ -183,8 +191,7 @@ struct BackwardWeightOps {
       const bool in = c.ok && i < images && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
                       static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
       out[j] = in ? x[static_cast<size_t>(img0 + i) * g.C * g.H * g.W + c.off + ih * g.W + iw] : 0.0f;
-      r += 2;
-      if (r >= ohw) { r -= ohw; ++i; }
+      if (++r == ohw) { r = 0; ++i; }
     }
   }
   __device__ void store(int m, int n, float v) const {
@@ -193,19 +200,55 @@ struct BackwardWeightOps {
   }
 };
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// fp32 -> bf16, round to nearest even (operands are finite)
+__device__ __forceinline__ unsigned short to_bf16(float f) {
+  const unsigned u = __float_as_uint(f);
+  return static_cast<unsigned short>((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+// How the products are formed.
+//   kFp32:   fp32 operands, v_mfma_f32_32x32x2_f32.
+//   kBf16:   operands rounded to bf16 on their way into LDS, v_mfma_f32_32x32x16_bf16
+//            with fp32 accumulation (relative error of a result about 2e-3).
+//   kBf16x3: every operand split into a bf16 head and a bf16 tail (a = ah + al
+//            to 16 significant bits); ah*bh + ah*bl + al*bh on the bf16 matrix
+//            cores, fp32 accumulation: fp32-like results (about 1e-5) at three
+//            bf16 products, which is still a sixth of the fp32 matrix-core time.
+enum Compute { kFp32 = 0, kBf16 = 1, kBf16x3 = 2 };
+
+// Workgroup id -> tile, for a launch of tile_blocks(count) workgroups.
+// Consecutive workgroup ids go round the eight XCDs, each with an L2 of its
+// own; tile t is handed to XCD t / ceil(count / 8), so that an XCD walks a
+// contiguous range of tiles and the operand rows these share stay in its L2.
+// Returns -1 for the padding workgroups.
+__host__ __device__ inline int tile_blocks(int count) { return (count + 7) / 8 * 8; }
+__device__ __forceinline__ int tile_of_block(int count) {
+  const int per = (count + 7) / 8, t = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  return (blockIdx.x >> 3) < per && t < count ? t : -1;
+}
+
 // C[M, Ncols] = A[M, K] x B[K, Ncols], one 128x128 tile per workgroup.
-template <typename Ops>
+template <typename Ops, int MODE>
 __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
   using T = Tile;
-  __shared__ float As[2][T::BK][T::PITCH];
-  __shared__ float Bs[2][T::BK][T::PITCH];
+  constexpr bool BF16 = MODE != kFp32;
+  constexpr int PARTS = MODE == kBf16x3 ? 2 : 1;   // head, tail
+  // fp32: [k][row] so that the 32 lanes of a half read consecutive words;
+  // bf16: [part][row][k] (pitch 24 halves = 48 bytes) so that a lane reads its eight k as 16 bytes
+  constexpr int PK = 24;
+  constexpr int PART_WORDS = T::BM * PK / 2;
+  constexpr int LDS_WORDS = BF16 ? PARTS * PART_WORDS : T::BK * T::PITCH;
+  __shared__ __attribute__((aligned(16))) float As[2][LDS_WORDS];
+  __shared__ __attribute__((aligned(16))) float Bs[2][LDS_WORDS];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
 
   // staging roles: A: row a_m, eight consecutive k starting at a_k; B: column
-  // b_n, the eight k of one parity
+  // b_n, eight consecutive k starting at b_k (the same for a wavefront)
   const int a_m = tid >> 1, a_k = (tid & 1) * 8;
-  const int b_n = tid & 127, b_k = __builtin_amdgcn_readfirstlane(tid >> 7);   // the same for a wavefront
+  const int b_n = tid & 127, b_k = __builtin_amdgcn_readfirstlane(tid >> 7) * 8;
   const typename Ops::BCtx bctx = ops.b_ctx(n0 + b_n);
 
   float16v acc[2][2];
@@ -222,39 +265,86 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
     ops.fetch_b(bctx, k0 + b_k, rb);
   };
   auto stage = [&](int buf) {
+    if (BF16) {
+      typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int j = 0; j < 8; ++j) As[buf][a_k + j][a_m] = ra[j];
+      for (int part = 0; part < PARTS; ++part) {
+        u32x4 pa, pb;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) Bs[buf][b_k + 2 * j][b_n] = rb[j];
+        for (int j = 0; j < 4; ++j) {
+          pa[j] = to_bf16(ra[2 * j]) | (static_cast<unsigned>(to_bf16(ra[2 * j + 1])) << 16);
+          pb[j] = to_bf16(rb[2 * j]) | (static_cast<unsigned>(to_bf16(rb[2 * j + 1])) << 16);
+        }
+        *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned short*>(As[buf] + part * PART_WORDS) + a_m * PK + a_k) = pa;
+        *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned short*>(Bs[buf] + part * PART_WORDS) + b_n * PK + b_k) = pb;
+        if (part + 1 < PARTS) {
+          // what the heads left over (exact in fp32)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            ra[2 * j] -= __uint_as_float(pa[j] << 16); ra[2 * j + 1] -= __uint_as_float(pa[j] & 0xffff0000u);
+            rb[2 * j] -= __uint_as_float(pb[j] << 16); rb[2 * j + 1] -= __uint_as_float(pb[j] & 0xffff0000u);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) As[buf][(a_k + j) * T::PITCH + a_m] = ra[j];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) Bs[buf][(b_k + j) * T::PITCH + b_n] = rb[j];
+    }
   };
 
   const int steps = (ops.K + T::BK - 1) / T::BK;
+  const int half = lane >> 5, col = lane & 31;
   fetch(0);
   stage(0);
   __syncthreads();
   for (int s = 0; s < steps; ++s) {
     const int buf = s & 1;
     if (s + 1 < steps) fetch((s + 1) * T::BK);
-    const int half = lane >> 5, col = lane & 31;
+    if (BF16) {
+      bf16x8 a[PARTS][2], b[PARTS][2];
 #pragma unroll
-    for (int kk = 0; kk < T::BK; kk += 2) {
-      float a[2], b[2];
+      for (int part = 0; part < PARTS; ++part) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = As[buf][kk + half][wm + i * 32 + col];
+        for (int i = 0; i < 2; ++i)
+          a[part][i] = *reinterpret_cast<const bf16x8*>(
+              reinterpret_cast<const unsigned short*>(As[buf] + part * PART_WORDS) + (wm + i * 32 + col) * PK + half * 8);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) b[j] = Bs[buf][kk + half][wn + j * 32 + col];
+        for (int j = 0; j < 2; ++j)
+          b[part][j] = *reinterpret_cast<const bf16x8*>(
+              reinterpret_cast<const unsigned short*>(Bs[buf] + part * PART_WORDS) + (wn + j * 32 + col) * PK + half * 8);
+      }
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j) {
+          if (PARTS == 2) {   // small terms first
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1][i], b[0][j], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0][i], b[1][j], acc[i][j], 0, 0, 0);
+          }
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0][i], b[0][j], acc[i][j], 0, 0, 0);
+        }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < T::BK; kk += 2) {
+        float a[2], b[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) a[i] = As[buf][(kk + half) * T::PITCH + wm + i * 32 + col];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) b[j] = Bs[buf][(kk + half) * T::PITCH + wn + j * 32 + col];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+      }
     }
     if (s + 1 < steps) stage(buf ^ 1);
     __syncthreads();
   }
 
   // accumulator register v of a lane: row 8 * (v / 4) + 4 * (lane / 32) + v % 4, column lane % 32
-  const int half = lane >> 5, col = lane & 31;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -266,20 +356,29 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
       }
 }
 
-template <typename Ops>
+// Tiles in column-major order: the row tiles of one column tile are neighbours
+// and read the same gathered operand.
+template <typename Ops, int MODE>
 __global__ void __launch_bounds__(Tile::NT)
-igemm_kernel(Ops ops) {
-  igemm_tile(ops, blockIdx.y * Tile::BM, blockIdx.x * Tile::BN);
+igemm_kernel(Ops ops, int row_tiles, int count) {
+  const int t = tile_of_block(count);
+  if (t < 0) return;
+  igemm_tile<Ops, MODE>(ops, (t % row_tiles) * Tile::BM, (t / row_tiles) * Tile::BN);
 }
 
-// One slice of images per blockIdx.z; every slice writes its own partial.
+// Slices of images times tiles, slice-major; every slice writes its own partial.
+template <int MODE>
 __global__ void __launch_bounds__(Tile::NT)
-igemm_weight_kernel(BackwardWeightOps ops, int images_per_slice, int total_images) {
-  ops.img0 = blockIdx.z * images_per_slice;
+igemm_weight_kernel(BackwardWeightOps ops, int images_per_slice, int total_images, int row_tiles,
+                    int tiles_per_slice, int count) {
+  const int t = tile_of_block(count);
+  if (t < 0) return;
+  const int slice = t / tiles_per_slice, tile = t - slice * tiles_per_slice;
+  ops.img0 = slice * images_per_slice;
   ops.images = min(images_per_slice, total_images - ops.img0);
   ops.K = ops.images * ops.g.OH * ops.g.OW;
-  ops.partial += static_cast<size_t>(blockIdx.z) * ops.M * ops.Ncols;
-  igemm_tile(ops, blockIdx.y * Tile::BM, blockIdx.x * Tile::BN);
+  ops.partial += static_cast<size_t>(slice) * ops.M * ops.Ncols;
+  igemm_tile<BackwardWeightOps, MODE>(ops, (tile % row_tiles) * Tile::BM, (tile / row_tiles) * Tile::BN);
 }
 
 // out[i] (+)= sum over slices of partial[s][i]

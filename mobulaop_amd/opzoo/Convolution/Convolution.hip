@@ -19,6 +19,28 @@ using mobula_hip::call_state;
 using mobula_hip::failed;
 using mobula_hip::set_error;
 
+// option "conv_compute": 0 = fp32 operands (default), 1 = operands rounded to
+// bf16, 2 = operands split into two bf16 each (three products); fp32 accumulation throughout
+int compute_mode() {
+  const int mode = mobula_hip::option("conv_compute", 0);
+  return mode == conv::kBf16 || mode == conv::kBf16x3 ? mode : conv::kFp32;
+}
+
+template <typename Ops>
+void launch_igemm(const Ops& ops, hipStream_t stream) {
+  const int row_tiles = (ops.M + conv::Tile::BM - 1) / conv::Tile::BM;
+  const int count = row_tiles * ((ops.Ncols + conv::Tile::BN - 1) / conv::Tile::BN);
+  const dim3 grid(conv::tile_blocks(count));
+  switch (compute_mode()) {
+    case conv::kBf16:
+      conv::igemm_kernel<Ops, conv::kBf16><<<grid, conv::Tile::NT, 0, stream>>>(ops, row_tiles, count); break;
+    case conv::kBf16x3:
+      conv::igemm_kernel<Ops, conv::kBf16x3><<<grid, conv::Tile::NT, 0, stream>>>(ops, row_tiles, count); break;
+    default:
+      conv::igemm_kernel<Ops, conv::kFp32><<<grid, conv::Tile::NT, 0, stream>>>(ops, row_tiles, count);
+  }
+}
+
 int blocks_for(long long n) { return static_cast<int>(std::min<long long>((n + 255) / 256, 256ll * 32)); }
 
 bool fits(const char* what, int arg, long long need) {
@@ -69,11 +91,6 @@ conv::Tap* make_taps(int count, int KH, int KW, int plane, int dil_h, int dil_w,
   if (extra != nullptr) *extra = ws + tap_bytes;
   conv::build_taps_kernel<<<(count + 255) / 256, 256, 0, stream>>>(taps, count, KH, KW, plane, dil_h, dil_w);
   return taps;
-}
-
-dim3 tiles(long long M, long long Ncols, int z = 1) {
-  return dim3(static_cast<unsigned>((Ncols + conv::Tile::BN - 1) / conv::Tile::BN),
-              static_cast<unsigned>((M + conv::Tile::BM - 1) / conv::Tile::BM), static_cast<unsigned>(z));
 }
 
 }  // namespace
@@ -140,7 +157,7 @@ MOBULA_KERNEL conv2d_forward_kernel(const int n, const T* x, const T* weight, co
   if (failed()) return;
   {
     mobula_hip::KernelTimer timer("conv2d_forward", stream);
-    conv::igemm_kernel<conv::ForwardOps><<<tiles(ops.M, ops.Ncols), conv::Tile::NT, 0, stream>>>(ops);
+    launch_igemm(ops, stream);
   }
   MOBULA_HIP_TRY(hipGetLastError());
 }
@@ -173,7 +190,7 @@ MOBULA_KERNEL conv2d_backward_data_kernel(const int n, const T* dy, const T* wei
   if (failed()) return;
   {
     mobula_hip::KernelTimer timer("conv2d_backward_data", stream);
-    conv::igemm_kernel<conv::BackwardDataOps><<<tiles(ops.M, ops.Ncols), conv::Tile::NT, 0, stream>>>(ops);
+    launch_igemm(ops, stream);
   }
   MOBULA_HIP_TRY(hipGetLastError());
 }
@@ -203,8 +220,9 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
   ops.M = g.D; ops.Ncols = g.C * g.KH * g.KW; ops.K = 0; ops.img0 = 0; ops.images = 0;
   // K = N*OH*OW is long and the result small: slices of images go to different
   // workgroups, their partial sums are added in a fixed order afterwards.
-  const dim3 one = tiles(ops.M, ops.Ncols);
-  const long long per_slice_tiles = static_cast<long long>(one.x) * one.y;
+  const int row_tiles = (ops.M + conv::Tile::BM - 1) / conv::Tile::BM;
+  const long long per_slice_tiles = static_cast<long long>(row_tiles) * ((ops.Ncols + conv::Tile::BN - 1) / conv::Tile::BN);
+  if (per_slice_tiles * std::max(g.N, 1) >= (1ll << 30)) { set_error("conv2d_backward_weight: too many tiles"); return; }
   int slices = static_cast<int>(std::min<long long>(std::max(g.N, 1), std::max<long long>(1, 1024 / per_slice_tiles)));
   const int images_per_slice = g.N > 0 ? (g.N + slices - 1) / slices : 1;
   slices = g.N > 0 ? (g.N + images_per_slice - 1) / images_per_slice : 1;
@@ -215,8 +233,19 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
   ops.partial = reinterpret_cast<float*>(extra);
   {
     mobula_hip::KernelTimer timer("conv2d_backward_weight", stream);
-    conv::igemm_weight_kernel<<<tiles(ops.M, ops.Ncols, slices), conv::Tile::NT, 0, stream>>>(
-        ops, images_per_slice, g.N);
+    const int tps = static_cast<int>(per_slice_tiles), count = tps * slices;
+    const dim3 grid(conv::tile_blocks(count));
+    switch (compute_mode()) {
+      case conv::kBf16:
+        conv::igemm_weight_kernel<conv::kBf16><<<grid, conv::Tile::NT, 0, stream>>>(
+            ops, images_per_slice, g.N, row_tiles, tps, count); break;
+      case conv::kBf16x3:
+        conv::igemm_weight_kernel<conv::kBf16x3><<<grid, conv::Tile::NT, 0, stream>>>(
+            ops, images_per_slice, g.N, row_tiles, tps, count); break;
+      default:
+        conv::igemm_weight_kernel<conv::kFp32><<<grid, conv::Tile::NT, 0, stream>>>(
+            ops, images_per_slice, g.N, row_tiles, tps, count);
+    }
     conv::reduce_slices_kernel<<<blocks_for(wt), 256, 0, stream>>>(ops.partial, dw, wt, slices, accumulate);
   }
   MOBULA_HIP_TRY(hipGetLastError());
