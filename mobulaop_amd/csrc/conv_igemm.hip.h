@@ -38,61 +38,102 @@ struct Tile {
   static constexpr int NT = 256;
 };
 
-// Table entry for one value of the filter-tap index: element offset into the
-// tensor the taps walk over, and the dilated tap position.
-struct Tap { int off; short dh, dw; };
+// Offsets that a raw buffer load answers with zero: beyond every record count used here.
+constexpr int kDead = static_cast<int>(0x80000000u);
+constexpr unsigned kRecordLimit = 0x7fffffffu;
 
-// taps[k] for k = (c, kh, kw) over x (forward, dW) or k = (d, kh, kw) over dy (dx).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const float* base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+__device__ __forceinline__ float buffer_load1(__amdgpu_buffer_rsrc_t r, int voffset, int soffset) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voffset, soffset, 0));
+}
+
+// ---- the two gathered products (forward, data gradient) ----------------------
+// K runs tap-major: k = tap * Cpad + c with Cpad = channels rounded up to 16,
+// so that a K step of 16 lies within one filter tap: the position of the tap
+// and whether it falls into the padding is worked out once per step and lane,
+// and the 16 channels are 16 loads from one address with scalar plane offsets.
+// The left operand is a copy of the weights in that order, [Mpad][taps][Cpad],
+// zero where a row or channel is padding (arrange_weights_kernel), so that its
+// loads need no guards; the gathered operand re-reads the last real channel
+// for padding channels (times zero).
+
+// One K step of a gathered product.
+struct GatherStep {
+  int dh, dw;     // dilated tap position
+  int delta;      // byte offset of the tap relative to the lane's anchor pixel
+  int c0;         // first channel of the step
+};
+
+// steps[s] for s = tap * (Cpad / 16) + c0 / 16; sign = +1: taps walk forward over
+// the source (forward pass), -1: backward (data gradient, source = dy).
 __global__ void __launch_bounds__(256)
-build_taps_kernel(Tap* __restrict__ taps, int count, int KH, int KW, int plane, int dil_h, int dil_w) {
-  const int k = blockIdx.x * blockDim.x + threadIdx.x;
-  if (k >= count) return;
-  const int kw = k % KW, kh = (k / KW) % KH, ch = k / (KW * KH);
-  taps[k] = Tap{ch * plane, static_cast<short>(kh * dil_h), static_cast<short>(kw * dil_w)};
+build_gather_steps_kernel(GatherStep* __restrict__ steps, int count, int per_tap, int KW, int dil_h,
+                          int dil_w, int row, int sign) {
+  const int s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= count) return;
+  const int tap = s / per_tap, kh = tap / KW, kw = tap - kh * KW;
+  steps[s] = GatherStep{kh * dil_h, kw * dil_w, sign * (kh * dil_h * row + kw * dil_w) * 4,
+                        (s - tap * per_tap) * 16};
+}
+
+// out[m][tap][c] = w[m * stride_m + c * stride_c + tap] for m < M and c < C, else 0
+// (m < Mpad, c < Cpad).
+__global__ void __launch_bounds__(256)
+arrange_weights_kernel(const float* __restrict__ w, float* __restrict__ out, int M, int Mpad, int C,
+                       int Cpad, int taps, long long stride_m, long long stride_c) {
+  const long long total = static_cast<long long>(Mpad) * taps * Cpad;
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int c = static_cast<int>(i % Cpad), tap = static_cast<int>((i / Cpad) % taps);
+  const int m = static_cast<int>(i / (static_cast<long long>(Cpad) * taps));
+  out[i] = (m < M && c < C) ? w[m * stride_m + c * stride_c + tap] : 0.0f;
 }
 
 // ---- operand functors -------------------------------------------------------
-// fetch_a(m, k, out): the eight elements A[m][k .. k+7] of the left operand;
-// BCtx b_ctx(n) + fetch_b(ctx, k, out): the eight elements B[k .. k+7][n]
-// of the right operand (k is the same for a whole wavefront, so everything
-// that depends only on k is scalar); store(m, n, v).  Elements outside the
-// operands are zero.
+// Step load_step(s): what is the same for all lanes in K step s (scalar);
+// fetch_a(m, step, s, ak, out): A[m][16 s + ak .. + 7]; BCtx b_ctx(n, n0): what
+// column n needs throughout (n0 = first column of the tile);
+// fetch_b(ctx, step, bk, out): B[16 s + bk .. + 7][n], bk the same for a
+// wavefront; store(m, n, v).  Elements outside the operands are zero.
 
 struct ForwardOps {
-  const float* __restrict__ x; const float* __restrict__ w; const float* __restrict__ bias;
-  float* __restrict__ y; const Tap* __restrict__ taps;
-  Geometry g; int M, Ncols, K;
-  struct BCtx { int base; int ih0, iw0; bool ok; };
-  __device__ void fetch_a(int m, int k, float (&out)[8]) const {
-    const size_t at = static_cast<size_t>(m) * K + k;
-    if (m < M && k + 8 <= K && (at & 3) == 0) {
-      const float4 lo = *reinterpret_cast<const float4*>(w + at), hi = *reinterpret_cast<const float4*>(w + at + 4);
-      out[0] = lo.x; out[1] = lo.y; out[2] = lo.z; out[3] = lo.w;
-      out[4] = hi.x; out[5] = hi.y; out[6] = hi.z; out[7] = hi.w;
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) out[j] = (m < M && k + j < K) ? w[at + j] : 0.0f;
-    }
+  const float* __restrict__ x; const float* __restrict__ wp; const float* __restrict__ bias;
+  float* __restrict__ y; const GatherStep* __restrict__ steps;
+  Geometry g; int M, Ncols, K;   // K = taps * Cpad
+  typedef GatherStep Step;
+  struct BCtx { __amdgpu_buffer_rsrc_t src; int anchor; int ih0, iw0; bool ok; };
+  __device__ Step load_step(int s) const { return steps[s]; }
+  __device__ void fetch_a(int m, const Step&, int s, int ak, float (&out)[8]) const {
+    const float4* p = reinterpret_cast<const float4*>(wp + static_cast<size_t>(m) * K + s * Tile::BK + ak);
+    const float4 lo = p[0], hi = p[1];
+    out[0] = lo.x; out[1] = lo.y; out[2] = lo.z; out[3] = lo.w;
+    out[4] = hi.x; out[5] = hi.y; out[6] = hi.z; out[7] = hi.w;
   }
-  __device__ BCtx b_ctx(int n) const {
+  __device__ BCtx b_ctx(int n, int n0) const {
     BCtx c;
     c.ok = n < Ncols;
-    const int ohw = g.OH * g.OW, img = n / ohw, r = n - img * ohw, oh = r / g.OW, ow = r - oh * g.OW;
+    const int ohw = g.OH * g.OW, image = g.C * g.H * g.W;
+    const int first = __builtin_amdgcn_readfirstlane(n0 / ohw);
+    const int img = n / ohw, r = n - img * ohw, oh = r / g.OW, ow = r - oh * g.OW;
+    const size_t skip = static_cast<size_t>(first) * image;
+    const size_t left = (static_cast<size_t>(g.N) * image - skip) * sizeof(float);
+    c.src = buffer_of(x + skip, static_cast<unsigned>(left < kRecordLimit ? left : kRecordLimit));
     c.ih0 = oh * g.stride_h - g.pad_h;
     c.iw0 = ow * g.stride_w - g.pad_w;
-    c.base = img * g.C * g.H * g.W + c.ih0 * g.W + c.iw0;
+    c.anchor = ((img - first) * image + c.ih0 * g.W + c.iw0) * 4;
     return c;
   }
-  __device__ void fetch_b(const BCtx& c, int k, float (&out)[8]) const {
+  __device__ void fetch_b(const BCtx& c, const Step& e, int bk, float (&out)[8]) const {
+    const int ih = c.ih0 + e.dh, iw = c.iw0 + e.dw;
+    const bool in = c.ok && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
+                    static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
+    const int at = in ? c.anchor + e.delta : kDead;
+    const int plane = g.H * g.W * 4;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int kk = k + j;
-      const Tap t = taps[min(kk, K - 1)];   // scalar load: kk is uniform
-      const int ih = c.ih0 + t.dh, iw = c.iw0 + t.dw;
-      const bool in = c.ok && kk < K && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
-                      static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
-      out[j] = in ? x[c.base + t.off + t.dh * g.W + t.dw] : 0.0f;
-    }
+    for (int j = 0; j < 8; ++j)
+      out[j] = buffer_load1(c.src, at, min(e.c0 + bk + j, g.C - 1) * plane);
   }
   __device__ void store(int m, int n, float v) const {
     if (m >= M || n >= Ncols) return;
@@ -104,43 +145,50 @@ struct ForwardOps {
 // dx[img, c, ih, iw] = sum over (d, kh, kw) of W[d, c, kh, kw] * dy[img, d, oh, ow]
 // with oh * stride = ih + pad - kh * dil (and likewise for columns).
 struct BackwardDataOps {
-  const float* __restrict__ dy; const float* __restrict__ w; float* __restrict__ dx;
-  const Tap* __restrict__ taps;   // taps over dy: off = d * OH*OW
+  const float* __restrict__ dy; const float* __restrict__ wp; float* __restrict__ dx;
+  const GatherStep* __restrict__ steps;
   Geometry g; int M, Ncols, K; int accumulate;
-  struct BCtx { int base; int ihp, iwp; bool ok; };
-  __device__ void fetch_a(int m, int k, float (&out)[8]) const {
-    const int khw = g.KH * g.KW;
-    int d = k / khw, r = k - d * khw;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      out[j] = (m < M && k + j < K) ? w[(static_cast<size_t>(d) * g.C + m) * khw + r] : 0.0f;
-      if (++r == khw) { r = 0; ++d; }
-    }
+  typedef GatherStep Step;
+  struct BCtx { __amdgpu_buffer_rsrc_t src; int anchor; int ihp, iwp; bool ok; };
+  __device__ Step load_step(int s) const { return steps[s]; }
+  __device__ void fetch_a(int m, const Step&, int s, int ak, float (&out)[8]) const {
+    const float4* p = reinterpret_cast<const float4*>(wp + static_cast<size_t>(m) * K + s * Tile::BK + ak);
+    const float4 lo = p[0], hi = p[1];
+    out[0] = lo.x; out[1] = lo.y; out[2] = lo.z; out[3] = lo.w;
+    out[4] = hi.x; out[5] = hi.y; out[6] = hi.z; out[7] = hi.w;
   }
-  __device__ BCtx b_ctx(int n) const {
+  __device__ BCtx b_ctx(int n, int n0) const {
     BCtx c;
     c.ok = n < Ncols;
-    const int hw = g.H * g.W, img = n / hw, r = n - img * hw, ih = r / g.W, iw = r - ih * g.W;
+    const int hw = g.H * g.W, image = g.D * g.OH * g.OW;
+    const int first = __builtin_amdgcn_readfirstlane(n0 / hw);
+    const int img = n / hw, r = n - img * hw, ih = r / g.W, iw = r - ih * g.W;
+    const size_t skip = static_cast<size_t>(first) * image;
+    const size_t left = (static_cast<size_t>(g.N) * image - skip) * sizeof(float);
+    c.src = buffer_of(dy + skip, static_cast<unsigned>(left < kRecordLimit ? left : kRecordLimit));
     c.ihp = ih + g.pad_h; c.iwp = iw + g.pad_w;
-    c.base = img * g.D * g.OH * g.OW;
+    // stride 1: byte offset of dy[img, 0, ihp, iwp]; otherwise of dy[img, 0, 0, 0]
+    const bool unit = g.stride_h == 1 && g.stride_w == 1;
+    c.anchor = ((img - first) * image + (unit ? c.ihp * g.OW + c.iwp : 0)) * 4;
     return c;
   }
-  __device__ void fetch_b(const BCtx& c, int k, float (&out)[8]) const {
-    const bool unit = g.stride_h == 1 && g.stride_w == 1;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int kk = k + j;
-      const Tap t = taps[min(kk, K - 1)];
-      const int th = c.ihp - t.dh, tw = c.iwp - t.dw;
-      int oh = th, ow = tw;
-      bool in = c.ok && kk < K && th >= 0 && tw >= 0;
-      if (!unit) {
-        oh = th / g.stride_h; ow = tw / g.stride_w;
-        in = in && oh * g.stride_h == th && ow * g.stride_w == tw;
-      }
-      in = in && oh < g.OH && ow < g.OW;
-      out[j] = in ? dy[c.base + t.off + oh * g.OW + ow] : 0.0f;
+  __device__ void fetch_b(const BCtx& c, const Step& e, int bk, float (&out)[8]) const {
+    const int th = c.ihp - e.dh, tw = c.iwp - e.dw;
+    int at;
+    if (g.stride_h == 1 && g.stride_w == 1) {
+      const bool in = c.ok && static_cast<unsigned>(th) < static_cast<unsigned>(g.OH) &&
+                      static_cast<unsigned>(tw) < static_cast<unsigned>(g.OW);
+      at = in ? c.anchor + e.delta : kDead;
+    } else {
+      const int oh = th / g.stride_h, ow = tw / g.stride_w;
+      const bool in = c.ok && th >= 0 && tw >= 0 && oh * g.stride_h == th && ow * g.stride_w == tw &&
+                      oh < g.OH && ow < g.OW;
+      at = in ? c.anchor + (oh * g.OW + ow) * 4 : kDead;
     }
+    const int plane = g.OH * g.OW * 4;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      out[j] = buffer_load1(c.src, at, min(e.c0 + bk + j, g.D - 1) * plane);
   }
   __device__ void store(int m, int n, float v) const {
     if (m >= M || n >= Ncols) return;
@@ -150,17 +198,35 @@ struct BackwardDataOps {
   }
 };
 
+// Table entry for one column of the weight gradient, n = (c, kh, kw): element
+// offset of the channel plane in x and the dilated tap position.
+struct Tap { int off; short dh, dw; };
+
+__global__ void __launch_bounds__(256)
+build_taps_kernel(Tap* __restrict__ taps, int count, int KH, int KW, int plane, int dil_h, int dil_w) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= count) return;
+  const int kw = k % KW, kh = (k / KW) % KH, ch = k / (KW * KH);
+  taps[k] = Tap{ch * plane, static_cast<short>(kh * dil_h), static_cast<short>(kw * dil_w)};
+}
+
 // partial[z][d, (c, kh, kw)] = sum over the images of slice z and (oh, ow) of
-// dy[img, d, oh, ow] * x[img, c, ih, iw].
+// dy[img, d, oh, ow] * x[img, c, ih, iw]; k = (image of the slice, oh, ow).
 struct BackwardWeightOps {
   const float* __restrict__ dy; const float* __restrict__ x; float* __restrict__ partial;
   const Tap* __restrict__ taps;   // taps over x
   Geometry g; int M, Ncols, K;   // K = images_per_slice * OH*OW
   int img0, images;              // the images of this slice
+  struct Step { int i, r; };     // image within the slice and pixel of the step's first k
   struct BCtx { int off; int dh, dw; bool ok; };
-  __device__ void fetch_a(int m, int k, float (&out)[8]) const {
+  __device__ Step load_step(int s) const {
+    const int ohw = g.OH * g.OW, k = s * Tile::BK, i = k / ohw;
+    return Step{i, k - i * ohw};
+  }
+  __device__ void fetch_a(int m, const Step& e, int, int ak, float (&out)[8]) const {
     const int ohw = g.OH * g.OW;
-    int i = k / ohw, r = k - i * ohw;
+    int i = e.i, r = e.r + ak;
+    if (r >= ohw) { r -= ohw; ++i; }
     const size_t at = (static_cast<size_t>(img0 + i) * g.D + m) * ohw + r;
     if (m < M && i < images && r + 8 <= ohw && (at & 3) == 0) {
       const float4 lo = *reinterpret_cast<const float4*>(dy + at), hi = *reinterpret_cast<const float4*>(dy + at + 4);
@@ -174,23 +240,38 @@ struct BackwardWeightOps {
       if (++r == ohw) { r = 0; ++i; }
     }
   }
-  __device__ BCtx b_ctx(int n) const {
+  __device__ BCtx b_ctx(int n, int) const {
     BCtx c;
     c.ok = n < Ncols;
     const Tap t = taps[c.ok ? n : 0];
     c.off = t.off; c.dh = t.dh; c.dw = t.dw;
     return c;
   }
-  __device__ void fetch_b(const BCtx& c, int k, float (&out)[8]) const {
-    const int ohw = g.OH * g.OW;
-    int i = k / ohw, r = k - i * ohw;   // scalar: k is uniform
+  __device__ void fetch_b(const BCtx& c, const Step& e, int bk, float (&out)[8]) const {
+    const int ohw = g.OH * g.OW, image = g.C * g.H * g.W;
+    int i = e.i, r = e.r + bk;   // scalar: the step and bk are uniform
+    if (r >= ohw) { r -= ohw; ++i; }
+    const int oh0 = r / g.OW, ow0 = r - oh0 * g.OW;
+    if (g.stride_w == 1 && ow0 + 8 <= g.OW && i < images) {
+      // eight pixels of one output row: one row check, loads from one address
+      const __amdgpu_buffer_rsrc_t src = buffer_of(x + static_cast<size_t>(img0 + i) * image, image * 4u);
+      const int ih = oh0 * g.stride_h - g.pad_h + c.dh, iw0 = ow0 - g.pad_w + c.dw;
+      const bool row = c.ok && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H);
+      const int at = (c.off + ih * g.W + iw0) * 4;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const bool in = row && static_cast<unsigned>(iw0 + j) < static_cast<unsigned>(g.W);
+        out[j] = buffer_load1(src, in ? at + 4 * j : kDead, 0);
+      }
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int oh = r / g.OW, ow = r - oh * g.OW;
       const int ih = oh * g.stride_h - g.pad_h + c.dh, iw = ow * g.stride_w - g.pad_w + c.dw;
       const bool in = c.ok && i < images && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
                       static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
-      out[j] = in ? x[static_cast<size_t>(img0 + i) * g.C * g.H * g.W + c.off + ih * g.W + iw] : 0.0f;
+      out[j] = in ? x[static_cast<size_t>(img0 + i) * image + c.off + ih * g.W + iw] : 0.0f;
       if (++r == ohw) { r = 0; ++i; }
     }
   }
@@ -249,7 +330,7 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
   // b_n, eight consecutive k starting at b_k (the same for a wavefront)
   const int a_m = tid >> 1, a_k = (tid & 1) * 8;
   const int b_n = tid & 127, b_k = __builtin_amdgcn_readfirstlane(tid >> 7) * 8;
-  const typename Ops::BCtx bctx = ops.b_ctx(n0 + b_n);
+  const typename Ops::BCtx bctx = ops.b_ctx(n0 + b_n, n0);
 
   float16v acc[2][2];
 #pragma unroll
@@ -260,9 +341,10 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   float ra[8], rb[8];
-  auto fetch = [&](int k0) {
-    ops.fetch_a(m0 + a_m, k0 + a_k, ra);
-    ops.fetch_b(bctx, k0 + b_k, rb);
+  auto fetch = [&](int s) {
+    const typename Ops::Step e = ops.load_step(s);
+    ops.fetch_a(m0 + a_m, e, s, a_k, ra);
+    ops.fetch_b(bctx, e, b_k, rb);
   };
   auto stage = [&](int buf) {
     if (BF16) {
@@ -301,7 +383,7 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
   __syncthreads();
   for (int s = 0; s < steps; ++s) {
     const int buf = s & 1;
-    if (s + 1 < steps) fetch((s + 1) * T::BK);
+    if (s + 1 < steps) fetch(s + 1);
     if (BF16) {
       bf16x8 a[PARTS][2], b[PARTS][2];
 #pragma unroll

@@ -93,6 +93,38 @@ conv::Tap* make_taps(int count, int KH, int KW, int plane, int dil_h, int dil_w,
   return taps;
 }
 
+// Workspace of a gathered product (forward, data gradient): the table of K
+// steps and the weights in [Mpad][taps][Cpad] order.  channels = what K runs
+// over besides the taps, plane_row = row length of the gathered tensor.
+struct GatherPlan { conv::GatherStep* steps; float* weights; int K; };
+
+bool plan_gather(GatherPlan* plan, const char* what, const conv::Geometry& g, const float* w, int M,
+                 int channels, long long image_elems, int columns_per_image, int plane_row, int sign,
+                 long long stride_m, long long stride_c, hipStream_t stream) {
+  // a tile's columns span this many images at most; their byte offsets must stay below 2^31
+  const long long span = (conv::Tile::BN - 1) / std::max(columns_per_image, 1) + 2;
+  if (span * image_elems * 4 >= (1ll << 31)) {
+    set_error("%s: images of %lld elements are too large for the 32-bit offsets of the gather", what, image_elems);
+    return false;
+  }
+  const int taps = g.KH * g.KW, cpad = (channels + 15) / 16 * 16, per_tap = cpad / 16;
+  const int mpad = (M + conv::Tile::BM - 1) / conv::Tile::BM * conv::Tile::BM;
+  const long long k = static_cast<long long>(taps) * cpad, wcount = k * mpad;
+  if (k >= (1ll << 31) || wcount >= (1ll << 31)) { set_error("%s: weights too large", what); return false; }
+  const int count = taps * per_tap;
+  const size_t step_bytes = (sizeof(conv::GatherStep) * count + 255) / 256 * 256;
+  char* ws = static_cast<char*>(mobula_hip::workspace(step_bytes + sizeof(float) * wcount));
+  if (failed()) return false;
+  plan->steps = reinterpret_cast<conv::GatherStep*>(ws);
+  plan->weights = reinterpret_cast<float*>(ws + step_bytes);
+  plan->K = static_cast<int>(k);
+  conv::build_gather_steps_kernel<<<(count + 255) / 256, 256, 0, stream>>>(plan->steps, count, per_tap, g.KW,
+                                                                          g.dil_h, g.dil_w, plane_row, sign);
+  conv::arrange_weights_kernel<<<blocks_for(wcount), 256, 0, stream>>>(w, plan->weights, M, mpad, channels, cpad,
+                                                                       taps, stride_m, stride_c);
+  return true;
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -151,12 +183,16 @@ MOBULA_KERNEL conv2d_forward_kernel(const int n, const T* x, const T* weight, co
   if (out == 0) return;
   hipStream_t stream = call_state().stream;
   conv::ForwardOps ops;
-  ops.x = x; ops.w = weight; ops.bias = has_bias ? bias : nullptr; ops.y = y; ops.g = g;
-  ops.M = g.D; ops.Ncols = g.N * g.OH * g.OW; ops.K = g.C * g.KH * g.KW;
-  ops.taps = make_taps(ops.K, g.KH, g.KW, g.H * g.W, g.dil_h, g.dil_w, 0, nullptr, stream);
-  if (failed()) return;
+  ops.x = x; ops.bias = has_bias ? bias : nullptr; ops.y = y; ops.g = g;
+  ops.M = g.D; ops.Ncols = g.N * g.OH * g.OW;
   {
     mobula_hip::KernelTimer timer("conv2d_forward", stream);
+    GatherPlan plan;
+    const long long taps = g.KH * g.KW;
+    if (!plan_gather(&plan, "conv2d_forward", g, weight, g.D, g.C, static_cast<long long>(g.C) * g.H * g.W,
+                     g.OH * g.OW, g.W, +1, g.C * taps, taps, stream))
+      return;
+    ops.wp = plan.weights; ops.steps = plan.steps; ops.K = plan.K;
     launch_igemm(ops, stream);
   }
   MOBULA_HIP_TRY(hipGetLastError());
@@ -184,12 +220,17 @@ MOBULA_KERNEL conv2d_backward_data_kernel(const int n, const T* dy, const T* wei
   if (in == 0) return;
   hipStream_t stream = call_state().stream;
   conv::BackwardDataOps ops;
-  ops.dy = dy; ops.w = weight; ops.dx = dx; ops.g = g; ops.accumulate = accumulate;
-  ops.M = g.C; ops.Ncols = g.N * g.H * g.W; ops.K = g.D * g.KH * g.KW;
-  ops.taps = make_taps(ops.K, g.KH, g.KW, g.OH * g.OW, g.dil_h, g.dil_w, 0, nullptr, stream);
-  if (failed()) return;
+  ops.dy = dy; ops.dx = dx; ops.g = g; ops.accumulate = accumulate;
+  ops.M = g.C; ops.Ncols = g.N * g.H * g.W;
   {
     mobula_hip::KernelTimer timer("conv2d_backward_data", stream);
+    GatherPlan plan;
+    const long long taps = g.KH * g.KW;
+    // row m of the left operand is input channel m: element [m][tap][d] = weight[d][m][tap]
+    if (!plan_gather(&plan, "conv2d_backward_data", g, weight, g.C, g.D,
+                     static_cast<long long>(g.D) * g.OH * g.OW, g.H * g.W, g.OW, -1, taps, g.C * taps, stream))
+      return;
+    ops.wp = plan.weights; ops.steps = plan.steps; ops.K = plan.K;
     launch_igemm(ops, stream);
   }
   MOBULA_HIP_TRY(hipGetLastError());
@@ -214,6 +255,10 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
       !fits("conv2d_backward_weight", 2, static_cast<long long>(g.N) * g.C * g.H * g.W) ||
       !fits("conv2d_backward_weight", 17, wt))
     return;
+  if (static_cast<long long>(g.C) * g.H * g.W * 4 >= (1ll << 31)) {
+    set_error("conv2d_backward_weight: images too large for 32-bit byte offsets");
+    return;
+  }
   hipStream_t stream = call_state().stream;
   conv::BackwardWeightOps ops;
   ops.dy = dy; ops.x = x; ops.g = g;
