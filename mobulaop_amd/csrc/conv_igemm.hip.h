@@ -210,25 +210,25 @@ build_taps_kernel(Tap* __restrict__ taps, int count, int KH, int KW, int plane, 
   taps[k] = Tap{ch * plane, static_cast<short>(kh * dil_h), static_cast<short>(kw * dil_w)};
 }
 
-// partial[z][d, (c, kh, kw)] = sum over the images of slice z and (oh, ow) of
-// dy[img, d, oh, ow] * x[img, c, ih, iw]; k = (image of the slice, oh, ow).
+// partial[z][d, (c, kh, kw)] = sum over the k of slice z of dy[img, d, oh, ow] *
+// x[img, c, ih, iw], k = (img, oh, ow) flattened; a slice is a range of k.
 struct BackwardWeightOps {
   const float* __restrict__ dy; const float* __restrict__ x; float* __restrict__ partial;
   const Tap* __restrict__ taps;   // taps over x
-  Geometry g; int M, Ncols, K;   // K = images_per_slice * OH*OW
-  int img0, images;              // the images of this slice
-  struct Step { int i, r; };     // image within the slice and pixel of the step's first k
+  Geometry g; int M, Ncols, K;   // K = length of this slice
+  int k_begin;                   // first k of this slice
+  struct Step { int img, r, left; };   // image and pixel of the step's first k; k left in the slice
   struct BCtx { int off; int dh, dw; bool ok; };
   __device__ Step load_step(int s) const {
-    const int ohw = g.OH * g.OW, k = s * Tile::BK, i = k / ohw;
-    return Step{i, k - i * ohw};
+    const int ohw = g.OH * g.OW, k = k_begin + s * Tile::BK, img = k / ohw;
+    return Step{img, k - img * ohw, K - s * Tile::BK};
   }
   __device__ void fetch_a(int m, const Step& e, int, int ak, float (&out)[8]) const {
     const int ohw = g.OH * g.OW;
-    int i = e.i, r = e.r + ak;
-    if (r >= ohw) { r -= ohw; ++i; }
-    const size_t at = (static_cast<size_t>(img0 + i) * g.D + m) * ohw + r;
-    if (m < M && i < images && r + 8 <= ohw && (at & 3) == 0) {
+    int img = e.img, r = e.r + ak;
+    if (r >= ohw) { r -= ohw; ++img; }
+    const size_t at = (static_cast<size_t>(img) * g.D + m) * ohw + r;
+    if (m < M && ak + 8 <= e.left && r + 8 <= ohw && (at & 3) == 0) {
       const float4 lo = *reinterpret_cast<const float4*>(dy + at), hi = *reinterpret_cast<const float4*>(dy + at + 4);
       out[0] = lo.x; out[1] = lo.y; out[2] = lo.z; out[3] = lo.w;
       out[4] = hi.x; out[5] = hi.y; out[6] = hi.z; out[7] = hi.w;
@@ -236,8 +236,8 @@ struct BackwardWeightOps {
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      out[j] = (m < M && i < images) ? dy[(static_cast<size_t>(img0 + i) * g.D + m) * ohw + r] : 0.0f;
-      if (++r == ohw) { r = 0; ++i; }
+      out[j] = (m < M && ak + j < e.left) ? dy[(static_cast<size_t>(img) * g.D + m) * ohw + r] : 0.0f;
+      if (++r == ohw) { r = 0; ++img; }
     }
   }
   __device__ BCtx b_ctx(int n, int) const {
@@ -249,12 +249,12 @@ struct BackwardWeightOps {
   }
   __device__ void fetch_b(const BCtx& c, const Step& e, int bk, float (&out)[8]) const {
     const int ohw = g.OH * g.OW, image = g.C * g.H * g.W;
-    int i = e.i, r = e.r + bk;   // scalar: the step and bk are uniform
-    if (r >= ohw) { r -= ohw; ++i; }
+    int img = e.img, r = e.r + bk;   // scalar: the step and bk are uniform
+    if (r >= ohw) { r -= ohw; ++img; }
     const int oh0 = r / g.OW, ow0 = r - oh0 * g.OW;
-    if (g.stride_w == 1 && ow0 + 8 <= g.OW && i < images) {
+    if (g.stride_w == 1 && ow0 + 8 <= g.OW && bk + 8 <= e.left) {
       // eight pixels of one output row: one row check, loads from one address
-      const __amdgpu_buffer_rsrc_t src = buffer_of(x + static_cast<size_t>(img0 + i) * image, image * 4u);
+      const __amdgpu_buffer_rsrc_t src = buffer_of(x + static_cast<size_t>(img) * image, image * 4u);
       const int ih = oh0 * g.stride_h - g.pad_h + c.dh, iw0 = ow0 - g.pad_w + c.dw;
       const bool row = c.ok && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H);
       const int at = (c.off + ih * g.W + iw0) * 4;
@@ -269,10 +269,10 @@ struct BackwardWeightOps {
     for (int j = 0; j < 8; ++j) {
       const int oh = r / g.OW, ow = r - oh * g.OW;
       const int ih = oh * g.stride_h - g.pad_h + c.dh, iw = ow * g.stride_w - g.pad_w + c.dw;
-      const bool in = c.ok && i < images && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
+      const bool in = c.ok && bk + j < e.left && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
                       static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
-      out[j] = in ? x[static_cast<size_t>(img0 + i) * image + c.off + ih * g.W + iw] : 0.0f;
-      if (++r == ohw) { r = 0; ++i; }
+      out[j] = in ? x[static_cast<size_t>(img) * image + c.off + ih * g.W + iw] : 0.0f;
+      if (++r == ohw) { r = 0; ++img; }
     }
   }
   __device__ void store(int m, int n, float v) const {
@@ -283,10 +283,13 @@ struct BackwardWeightOps {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-// fp32 -> bf16, round to nearest even (operands are finite)
-__device__ __forceinline__ unsigned short to_bf16(float f) {
-  const unsigned u = __float_as_uint(f);
-  return static_cast<unsigned short>((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// two fp32 -> two bf16 in one word, round to nearest even (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ unsigned pack_bf16(float lo, float hi) {
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
 }
 
 // How the products are formed.
@@ -354,8 +357,8 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
         u32x4 pa, pb;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          pa[j] = to_bf16(ra[2 * j]) | (static_cast<unsigned>(to_bf16(ra[2 * j + 1])) << 16);
-          pb[j] = to_bf16(rb[2 * j]) | (static_cast<unsigned>(to_bf16(rb[2 * j + 1])) << 16);
+          pa[j] = pack_bf16(ra[2 * j], ra[2 * j + 1]);
+          pb[j] = pack_bf16(rb[2 * j], rb[2 * j + 1]);
         }
         *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned short*>(As[buf] + part * PART_WORDS) + a_m * PK + a_k) = pa;
         *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned short*>(Bs[buf] + part * PART_WORDS) + b_n * PK + b_k) = pb;
@@ -448,17 +451,16 @@ igemm_kernel(Ops ops, int row_tiles, int count) {
   igemm_tile<Ops, MODE>(ops, (t % row_tiles) * Tile::BM, (t / row_tiles) * Tile::BN);
 }
 
-// Slices of images times tiles, slice-major; every slice writes its own partial.
+// Slices of K times tiles, slice-major; every slice writes its own partial.
 template <int MODE>
 __global__ void __launch_bounds__(Tile::NT)
-igemm_weight_kernel(BackwardWeightOps ops, int images_per_slice, int total_images, int row_tiles,
+igemm_weight_kernel(BackwardWeightOps ops, int k_per_slice, int k_total, int row_tiles,
                     int tiles_per_slice, int count) {
   const int t = tile_of_block(count);
   if (t < 0) return;
   const int slice = t / tiles_per_slice, tile = t - slice * tiles_per_slice;
-  ops.img0 = slice * images_per_slice;
-  ops.images = min(images_per_slice, total_images - ops.img0);
-  ops.K = ops.images * ops.g.OH * ops.g.OW;
+  ops.k_begin = slice * k_per_slice;
+  ops.K = min(k_per_slice, k_total - ops.k_begin);
   ops.partial += static_cast<size_t>(slice) * ops.M * ops.Ncols;
   igemm_tile<BackwardWeightOps, MODE>(ops, (tile % row_tiles) * Tile::BM, (tile / row_tiles) * Tile::BN);
 }

@@ -41,6 +41,9 @@ void launch_igemm(const Ops& ops, hipStream_t stream) {
   }
 }
 
+// workgroups the weight gradient aims at: four per CU of a 256-CU device
+constexpr long long kWeightSlots = 1024;
+
 int blocks_for(long long n) { return static_cast<int>(std::min<long long>((n + 255) / 256, 256ll * 32)); }
 
 bool fits(const char* what, int arg, long long need) {
@@ -262,15 +265,18 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
   hipStream_t stream = call_state().stream;
   conv::BackwardWeightOps ops;
   ops.dy = dy; ops.x = x; ops.g = g;
-  ops.M = g.D; ops.Ncols = g.C * g.KH * g.KW; ops.K = 0; ops.img0 = 0; ops.images = 0;
-  // K = N*OH*OW is long and the result small: slices of images go to different
-  // workgroups, their partial sums are added in a fixed order afterwards.
+  ops.M = g.D; ops.Ncols = g.C * g.KH * g.KW; ops.K = 0; ops.k_begin = 0;
+  // K = N*OH*OW is long and the result small: K is cut into slices of whole K
+  // steps, as many as give every CU four workgroups; the partial sums of the
+  // slices are added in a fixed order afterwards.
   const int row_tiles = (ops.M + conv::Tile::BM - 1) / conv::Tile::BM;
   const long long per_slice_tiles = static_cast<long long>(row_tiles) * ((ops.Ncols + conv::Tile::BN - 1) / conv::Tile::BN);
-  if (per_slice_tiles * std::max(g.N, 1) >= (1ll << 30)) { set_error("conv2d_backward_weight: too many tiles"); return; }
-  int slices = static_cast<int>(std::min<long long>(std::max(g.N, 1), std::max<long long>(1, 1024 / per_slice_tiles)));
-  const int images_per_slice = g.N > 0 ? (g.N + slices - 1) / slices : 1;
-  slices = g.N > 0 ? (g.N + images_per_slice - 1) / images_per_slice : 1;
+  const long long k_total = static_cast<long long>(g.N) * g.OH * g.OW;   // < 2^31: checked by describe()
+  if (per_slice_tiles >= (1ll << 20)) { set_error("conv2d_backward_weight: too many tiles"); return; }
+  const long long k_steps = std::max<long long>(1, (k_total + conv::Tile::BK - 1) / conv::Tile::BK);
+  long long slices = std::min<long long>(k_steps, std::max<long long>(1, kWeightSlots / per_slice_tiles));
+  const long long k_per_slice = (k_steps + slices - 1) / slices * conv::Tile::BK;
+  slices = std::max<long long>(1, (k_total + k_per_slice - 1) / k_per_slice);
   char* extra = nullptr;
   ops.taps = make_taps(ops.Ncols, g.KH, g.KW, g.H * g.W, g.dil_h, g.dil_w,
                        sizeof(float) * static_cast<size_t>(slices) * wt, &extra, stream);
@@ -278,20 +284,20 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
   ops.partial = reinterpret_cast<float*>(extra);
   {
     mobula_hip::KernelTimer timer("conv2d_backward_weight", stream);
-    const int tps = static_cast<int>(per_slice_tiles), count = tps * slices;
+    const int tps = static_cast<int>(per_slice_tiles), count = tps * static_cast<int>(slices);
     const dim3 grid(conv::tile_blocks(count));
     switch (compute_mode()) {
       case conv::kBf16:
         conv::igemm_weight_kernel<conv::kBf16><<<grid, conv::Tile::NT, 0, stream>>>(
-            ops, images_per_slice, g.N, row_tiles, tps, count); break;
+            ops, static_cast<int>(k_per_slice), static_cast<int>(k_total), row_tiles, tps, count); break;
       case conv::kBf16x3:
         conv::igemm_weight_kernel<conv::kBf16x3><<<grid, conv::Tile::NT, 0, stream>>>(
-            ops, images_per_slice, g.N, row_tiles, tps, count); break;
+            ops, static_cast<int>(k_per_slice), static_cast<int>(k_total), row_tiles, tps, count); break;
       default:
         conv::igemm_weight_kernel<conv::kFp32><<<grid, conv::Tile::NT, 0, stream>>>(
-            ops, images_per_slice, g.N, row_tiles, tps, count);
+            ops, static_cast<int>(k_per_slice), static_cast<int>(k_total), row_tiles, tps, count);
     }
-    conv::reduce_slices_kernel<<<blocks_for(wt), 256, 0, stream>>>(ops.partial, dw, wt, slices, accumulate);
+    conv::reduce_slices_kernel<<<blocks_for(wt), 256, 0, stream>>>(ops.partial, dw, wt, static_cast<int>(slices), accumulate);
   }
   MOBULA_HIP_TRY(hipGetLastError());
 }
