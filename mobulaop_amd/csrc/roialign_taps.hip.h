@@ -94,13 +94,14 @@ __device__ __forceinline__ AxisUnit clip_unit(int bin, const AxisSample& a, int 
 // One wavefront per ROI: lane s < PH*S evaluates sample row s once and clips it
 // against every tile row of the ROI's box; likewise for sample columns.
 // The wavefront also finds the ROI's box (the pixels any valid sample touches),
-// stores it as tile ranges for tile_fill_kernel and counts the ROI in every
-// tile of the box.
+// and stores it as tile ranges for build_tile_work_kernel.
 __global__ void __launch_bounds__(256)
 build_lists_kernel(const float* __restrict__ rois, int R, float scale, int PH, int PW, int S, int H,
                    int W, long long num_images, TileGrid tg, ListLayout ll,
-                   TileBox* __restrict__ boxes, int* __restrict__ tile_count,
+                   TileBox* __restrict__ boxes, int* __restrict__ cursors,
                    AxisUnit* __restrict__ lists) {
+  // the two bump pointers of build_tile_work_kernel, which runs after this one
+  if (blockIdx.x == 0 && threadIdx.x < 2) cursors[threadIdx.x] = 0;
   const int roi = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
   if (roi >= R) return;
   const int lane = threadIdx.x & 63;
@@ -128,9 +129,6 @@ build_lists_kernel(const float* __restrict__ rois, int R, float scale, int PH, i
     const int tx0 = rec.col_lo / tg.tw, tx1 = any ? rec.col_hi / tg.tw : -1;
     if (lane == 0) boxes[roi] = TileBox{any ? g.batch : -1, ty0 | (ty1 << 16), tx0 | (tx1 << 16), 0};
     if (!any) return;
-    int* const counts = tile_count + static_cast<long long>(g.batch) * tg.per_image;
-    const int nx = tx1 - tx0 + 1, nt = (ty1 - ty0 + 1) * nx;
-    for (int t = lane; t < nt; t += 64) atomicAdd(counts + (ty0 + t / nx) * tg.tx + tx0 + t % nx, 1);
   }
   AxisUnit* const base = lists + static_cast<long long>(roi) * ll.roi_stride;
   const float inv_count = 1.0f / rec.count;
@@ -207,21 +205,65 @@ struct alignas(16) WorkEntry {
 };
 struct WorkRange { int begin; int count; };
 
-// One workgroup per tile, one wavefront per tile row: lane j looks at ROI j of
-// the tile's list, takes its taps for this row from the row-tap table, and all
-// lanes append theirs in list order.  WorkRange::count includes the padding.  Space for the tile's sixteen lists comes
-// from one bump-pointer allocation per tile (*cursor).
+// One workgroup per tile, one wavefront per tile row.
+// First the tile's ROI list: every wavefront takes a sixteenth of the ROIs,
+// counts those whose box covers the tile, and after one exchange writes them,
+// in increasing ROI index, into space taken from cursors[0] with one atomic.
+// Then the work lists: lane j looks at ROI j of the tile's list, takes its taps
+// for this wavefront's row from the row-tap table, and all lanes append theirs
+// in list order.  WorkRange::count includes the padding.  Space for the tile's
+// sixteen lists comes from one bump-pointer allocation per tile (cursors[1]).
+// The order in which tiles take their space varies from run to run; what is
+// written into it does not.
 __global__ void __launch_bounds__(kTileRows * 64)
-build_worklists_kernel(const int* __restrict__ tile_offset, const int* __restrict__ tile_rois,
+build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict__ tile_rois,
                        const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll,
-                       int* __restrict__ cursor, WorkRange* __restrict__ ranges,
+                       int* __restrict__ cursors, WorkRange* __restrict__ ranges,
                        WorkEntry* __restrict__ entries) {
+  __shared__ int hits[kTileRows];
   __shared__ int row_total[kTileRows];
-  __shared__ int tile_base;
+  __shared__ int list_base, tile_base;
   const long long tile = blockIdx.x;
   const int lane = threadIdx.x & 63, row = threadIdx.x >> 6;
-  const int ty = static_cast<int>(tile % tg.per_image) / tg.tx;
-  const int begin = tile_offset[tile], end = tile_offset[tile + 1];
+  const int image = static_cast<int>(tile / tg.per_image);
+  const int t = static_cast<int>(tile % tg.per_image);
+  const int ty = t / tg.tx, tx = t % tg.tx;
+
+  // ---- the tile's ROI list ----
+  const int share = ((R + kTileRows * 64 - 1) / (kTileRows * 64)) * 64;
+  const int r_begin = row * share, r_end = min(R, r_begin + share);
+  auto hit_of = [&](int r) {
+    if (r >= r_end) return false;
+    const TileBox b = boxes[r];
+    return b.batch == image && ty >= (b.ty & 0xffff) && ty <= (b.ty >> 16) && tx >= (b.tx & 0xffff) &&
+           tx <= (b.tx >> 16);
+  };
+  int mine = 0;
+  for (int base = r_begin; base < r_end; base += 64) mine += __popcll(__ballot(hit_of(base + lane)));
+  if (lane == 0) hits[row] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int sum = 0;
+    for (int r = 0; r < kTileRows; ++r) sum += hits[r];
+    list_base = sum > 0 ? atomicAdd(cursors, sum) : 0;
+  }
+  __syncthreads();
+  int written = list_base, count = 0;
+  for (int r = 0; r < kTileRows; ++r) {
+    if (r < row) written += hits[r];
+    count += hits[r];
+  }
+  const int begin = list_base, end = list_base + count;
+  for (int base = r_begin; base < r_end && mine > 0; base += 64) {
+    const bool hit = hit_of(base + lane);
+    const unsigned long long mask = __ballot(hit);
+    if (hit) tile_rois[written + __popcll(mask & ((1ull << lane) - 1ull))] = base + lane;
+    written += __popcll(mask);
+    mine -= __popcll(mask);
+  }
+  __syncthreads();   // the list is complete and visible to the whole workgroup
+
+  // ---- the work lists of the sixteen rows ----
   auto table_of = [&](int roi) {
     return reinterpret_cast<const RowTapTable*>(lists + static_cast<long long>(roi) * ll.roi_stride +
                                                 static_cast<long long>(ty) * ll.row_stride);
@@ -242,7 +284,7 @@ build_worklists_kernel(const int* __restrict__ tile_offset, const int* __restric
   if (threadIdx.x == 0) {
     int sum = 0;
     for (int r = 0; r < kTileRows; ++r) sum += row_total[r];
-    tile_base = sum > 0 ? atomicAdd(cursor, sum) : 0;
+    tile_base = sum > 0 ? atomicAdd(cursors + 1, sum) : 0;
   }
   __syncthreads();
   int out = tile_base;

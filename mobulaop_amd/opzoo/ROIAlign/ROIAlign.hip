@@ -148,21 +148,19 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
 struct TilePlan {
   roialign::TileGrid grid;
   roialign::TileBox* boxes;
-  int* tile_count;
-  int* tile_offset;
+  int* cursors;                // bump pointers: [0] ROI lists, [1] work lists
   int* tile_rois;
   roialign::ListLayout layout;
   roialign::AxisUnit* lists;   // null unless requested
   float* dyb;                  // channel-blocked copy of dy, with the lists
   size_t dyb_bytes, list_bytes;
-  int* cursor;                 // bump pointer of the work lists (zeroed with tile_count)
   roialign::WorkRange* ranges; // per (tile, tile row)
   roialign::WorkEntry* entries;
 };
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// Runs the pre-pass (ROI records, per-tile ROI lists) for tiles of th x tw
+// Runs the pre-pass (ROI boxes and sample tables, per-tile ROI and work lists) for tiles of th x tw
 // pixels.  Returns false if the problem is too large for the list buffers (or
 // on error); the caller then uses the straightforward kernels.
 bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_lists,
@@ -176,7 +174,7 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   const long long list_cap = static_cast<long long>(p.R) * g.per_image;  // every ROI in every tile
   if (g.total <= 0 || g.total > (1ll << 24) || list_cap > (1ll << 27)) return false;
   const size_t b_recs = align_up(sizeof(roialign::TileBox) * std::max(p.R, 1), 256);
-  const size_t b_cnt = align_up(sizeof(int) * (g.total + 1), 256);
+  const size_t b_cnt = 256;   // the two bump pointers
   const size_t b_list = align_up(sizeof(int) * std::max<long long>(list_cap, 1), 256);
   plan->layout = roialign::make_list_layout(g, p.PW);
   const long long n_units = with_lists ? plan->layout.roi_stride * p.R : 0;
@@ -194,35 +192,27 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   plan->dyb_bytes = b_dyt; plan->list_bytes = b_units;
   const size_t b_ranges = with_lists ? align_up(sizeof(roialign::WorkRange) * g.total * roialign::kTileRows, 256) : 0;
   const size_t b_entries = with_lists ? align_up(sizeof(roialign::WorkEntry) * n_entries, 256) + 512 : 0;
-  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + 2 * b_cnt + b_list + b_units + b_dyt +
+  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + b_cnt + b_list + b_units + b_dyt +
                                                         b_ranges + b_entries + 256));
   if (failed()) return false;
   plan->boxes = reinterpret_cast<roialign::TileBox*>(base);
-  plan->tile_count = reinterpret_cast<int*>(base + b_recs);
-  plan->tile_offset = reinterpret_cast<int*>(base + b_recs + b_cnt);
-  plan->tile_rois = reinterpret_cast<int*>(base + b_recs + 2 * b_cnt);
-  plan->cursor = plan->tile_count + g.total;   // spare slot of the zeroed counter array
-  plan->lists = with_lists ? reinterpret_cast<roialign::AxisUnit*>(base + b_recs + 2 * b_cnt + b_list)
+  plan->cursors = reinterpret_cast<int*>(base + b_recs);
+  plan->tile_rois = reinterpret_cast<int*>(base + b_recs + b_cnt);
+  plan->lists = with_lists ? reinterpret_cast<roialign::AxisUnit*>(base + b_recs + b_cnt + b_list)
                            : nullptr;
-  char* cur = base + b_recs + 2 * b_cnt + b_list + b_units;
+  char* cur = base + b_recs + b_cnt + b_list + b_units;
   plan->dyb = with_lists ? reinterpret_cast<float*>(cur) : nullptr;
   cur += b_dyt;
   plan->ranges = reinterpret_cast<roialign::WorkRange*>(cur);
   cur += b_ranges;
   plan->entries = reinterpret_cast<roialign::WorkEntry*>(cur);
   cur += b_entries;
-  roialign::zero_words_kernel<<<grid_for(g.total + 1, 256), 256, 0, stream>>>(
-      reinterpret_cast<unsigned*>(plan->tile_count), g.total + 1);
-  if (p.R > 0)
-    roialign::build_lists_kernel<<<(p.R * 64 + 255) / 256, 256, 0, stream>>>(
-        rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->layout, plan->boxes,
-        plan->tile_count, plan->lists);
-  roialign::tile_scan_kernel<<<1, 1024, 0, stream>>>(plan->tile_count, g.total, plan->tile_offset);
-  if (p.R > 0)
-    roialign::tile_fill_kernel<<<static_cast<unsigned>(g.total), 256, 0, stream>>>(
-        plan->boxes, p.R, g, plan->tile_offset, plan->tile_rois);
-  roialign::build_worklists_kernel<<<static_cast<unsigned>(g.total), roialign::kTileRows * 64, 0, stream>>>(
-      plan->tile_offset, plan->tile_rois, plan->lists, g, plan->layout, plan->cursor, plan->ranges,
+  // two kernels: per-ROI tables (which also resets the bump pointers), then per-tile lists
+  roialign::build_lists_kernel<<<std::max(1, (p.R * 64 + 255) / 256), 256, 0, stream>>>(
+      rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->layout, plan->boxes,
+      plan->cursors, plan->lists);
+  roialign::build_tile_work_kernel<<<static_cast<unsigned>(g.total), roialign::kTileRows * 64, 0, stream>>>(
+      plan->boxes, p.R, plan->tile_rois, plan->lists, g, plan->layout, plan->cursors, plan->ranges,
       plan->entries);
   MOBULA_HIP_TRY(hipGetLastError());
   return !failed();
