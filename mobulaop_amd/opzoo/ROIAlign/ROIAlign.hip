@@ -13,6 +13,7 @@
 #include "roialign_naive.hip.h"
 #include "roialign_backward_blocked.hip.h"
 #include "roialign_forward_blocked.hip.h"
+#include "roialign_forward_merged.hip.h"
 
 namespace {
 
@@ -131,9 +132,14 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
       roialign::transpose_to_blocked_kernel<T, false><<<tgrid, 256, 0, stream>>>(
           x, xt, p.C, static_cast<int>(pixels));
     side.join();
-    {
+    if (p.S == 1 || p.S == 2) {
       mobula_hip::KernelTimer timer("forward_blocked_kernel", stream);
       roialign::forward_blocked_kernel<T><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+          xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
+    } else {
+      // larger (or adaptive) sampling grids: every pixel of a bin is loaded once
+      mobula_hip::KernelTimer timer("forward_merged_kernel", stream);
+      roialign::forward_merged_kernel<T><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
           xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
     }
     MOBULA_HIP_TRY(hipGetLastError());

@@ -96,6 +96,9 @@ def test_fp16_storage_forward(impl):
     (2, 130, 18, 70, 50, (14, 14), 0.125, 2),
     (1, 7, 64, 64, 20, (5, 9), 0.3, 3),     # non-square pooling, S=3
     (2, 4, 40, 40, 25, (7, 7), 1.0, 5),     # dense grid
+    (2, 36, 60, 90, 40, (7, 7), 0.25, 0),   # adaptive grid over the blocked layout, ragged last block
+    (1, 8, 200, 160, 12, (3, 14), 1.0, 0),  # bins of up to 67 x 11 samples: several sample windows
+    (2, 8, 50, 50, 30, (14, 7), 0.5, 4),    # more pooled rows than one set of row lists holds
 ])
 def test_ragged_shapes(impl, shape):
     abi.set_impl(impl)
