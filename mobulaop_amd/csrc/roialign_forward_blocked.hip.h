@@ -1,11 +1,12 @@
 // Forward ROIAlign over a channel-blocked copy of the feature map.
 //
-// The map is first rewritten from NCHW to [N][C/32][H][W][32]: the 32 channels
-// of a block at one pixel are one 128-byte line.  A wavefront then computes
-// one (ROI, channel block): its 64 lanes are 8 pooled columns x 8 channel
-// quads, so a single 16-byte load per lane fetches one bilinear corner of
-// eight bins (1 KB), sixteen such loads are in flight per lane, and every lane
-// sums its own bin: no cross-lane traffic.  Row corners are the same for the
+// The map is first rewritten from NCHW to [N][C/CB][H][W][CB] with CB = 32
+// channels for fp32 and 64 for fp16: the channels of a block at one pixel are
+// one 128-byte line.  A wavefront then computes one (ROI, channel block): its
+// 64 lanes are 8 pooled columns x 8 groups of 16 bytes of channels, so a single
+// 16-byte load per lane fetches one bilinear corner of eight bins (1 KB),
+// sixteen such loads are in flight per lane, and every lane sums its own bin:
+// no cross-lane traffic.  Row corners are the same for the
 // whole wavefront and live in scalar registers.
 // Channel block b is only ever read by XCD b % 8 and ROIs are visited in
 // spatial order, so what one L2 has to hold is a 128-byte-per-pixel slice of
@@ -16,29 +17,37 @@
 namespace roialign {
 
 struct FwdBlocked {
-  static constexpr int CB = 32;        // channels per block of the blocked layout
   static constexpr int NW = 4;         // independent wavefronts per workgroup
   static constexpr int MAXT = 128;     // column samples held in LDS (16 for each of 8 pooled columns)
   static constexpr int ROWT = 96;      // row samples held in LDS
-  static constexpr int STAGE = 1600;   // staged outputs per wavefront
   static constexpr int PWB = 8;        // pooled columns per step (one per group of 8 lanes)
   static constexpr int CELL = 32;      // side of the sorting cells in pixels
   static constexpr int MAXCELLS = 8192;
 };
 
+// Per element type: channels per lane (16 bytes), channels per block of the
+// blocked layout (8 lanes: 128 bytes per pixel), staged outputs per wavefront.
+template <typename T>
+struct BlockOf {
+  static constexpr int CPL = 16 / sizeof(T);
+  static constexpr int CB = 8 * CPL;
+  static constexpr int STAGE = 6400 / sizeof(T);
+};
+
 // Pooled rows staged per pass, 0 if the shape is not taken by this path.
-inline int blocked_rows_per_pass(int C, long long H, long long W, int PH, int PW, size_t elem) {
-  using K = FwdBlocked;
-  if (C % 4 != 0 || PW < 1 || K::CB * PW > K::STAGE) return 0;
-  if (H * W * K::CB * static_cast<long long>(elem) >= (1ll << 31)) return 0;
-  return min(PH, K::STAGE / (K::CB * PW));
+template <typename T>
+inline int blocked_rows_per_pass(int C, long long H, long long W, int PH, int PW) {
+  using B = BlockOf<T>;
+  if (C % B::CPL != 0 || PW < 1 || B::CB * PW > B::STAGE) return 0;
+  if (H * W * 128 >= (1ll << 31)) return 0;
+  return min(PH, B::STAGE / (B::CB * PW));
 }
 
-// out[n][cb][p][32] = in[n][cb*32 + k][p]; channels past C are written as zero.
+// out[n][cb][p][CB] = in[n][cb*CB + k][p]; channels past C are written as zero.
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 transpose_to_blocked_kernel(const T* __restrict__ in, T* __restrict__ out, int C, int P) {
-  constexpr int CB = FwdBlocked::CB;
+  constexpr int CB = BlockOf<T>::CB;
   struct alignas(4 * sizeof(T)) V4 { T v[4]; };
   __shared__ T tile[CB][65];
   const int n = blockIdx.z, cb = blockIdx.y, cblk = gridDim.y;
@@ -48,7 +57,7 @@ transpose_to_blocked_kernel(const T* __restrict__ in, T* __restrict__ out, int C
   if (VEC) {
     const int q = threadIdx.x & 15, r = threadIdx.x >> 4;   // 16 quads of pixels, 16 channels per pass
 #pragma unroll
-    for (int k = 0; k < 2; ++k) {
+    for (int k = 0; k < CB / 16; ++k) {
       const int c = c0 + r + 16 * k, p = p0 + 4 * q;
       V4 v;
 #pragma unroll
@@ -60,16 +69,17 @@ transpose_to_blocked_kernel(const T* __restrict__ in, T* __restrict__ out, int C
   } else {
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    for (int k = 0; k < CB / 4; ++k) {
       const int c = c0 + ty + 4 * k, p = p0 + tx;
       tile[ty + 4 * k][tx] = (c < C && p < P) ? src[static_cast<size_t>(c) * P + p] : from_float<T>(0.0f);
     }
   }
   __syncthreads();
-  const int cq = threadIdx.x & 7, pr = threadIdx.x >> 3;     // 8 channel quads, 32 pixels per pass
+  constexpr int QP = CB / 4, PP = 256 / QP;   // channel quads per pixel, pixels per pass
+  const int cq = threadIdx.x % QP, pr = threadIdx.x / QP;
 #pragma unroll
-  for (int k = 0; k < 2; ++k) {
-    const int pl = pr + 32 * k;
+  for (int k = 0; k < 64 / PP; ++k) {
+    const int pl = pr + PP * k;
     if (p0 + pl < P) {
       V4 v;
 #pragma unroll
@@ -140,23 +150,20 @@ struct alignas(16) RowEntry { int lo, hi; float wl, wh; };
 // A column sample, likewise, with the offsets in bytes along a row.
 struct alignas(16) ColEntry { int lo, hi; float wl, wh; };
 
-// Four consecutive elements (16 or 8 bytes) at byte offset lane_off + row_off of
-// a raw buffer; lane offsets outside the buffer read as zero without an access.
-__device__ __forceinline__ void buffer_load4(__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_off,
-                                             float (&out)[4]) {
+// Sixteen bytes of consecutive channels as they lie in a lane's registers: four
+// fp32 or eight fp16 (kept packed; an element is widened where it is used).
+template <typename T> struct LaneData;
+template <> struct LaneData<float> { typedef float type __attribute__((ext_vector_type(4))); };
+template <> struct LaneData<__half> { typedef _Float16 type __attribute__((ext_vector_type(8))); };
+
+// The sixteen bytes at byte offset lane_off + row_off of a raw buffer; lane
+// offsets outside the buffer read as zero without an access.
+template <typename T>
+__device__ __forceinline__ typename LaneData<T>::type buffer_load_lane(__amdgpu_buffer_rsrc_t rsrc, int lane_off,
+                                                                       int row_off) {
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   const u32x4 raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off, row_off, 0);
-  out[0] = __uint_as_float(raw.x); out[1] = __uint_as_float(raw.y);
-  out[2] = __uint_as_float(raw.z); out[3] = __uint_as_float(raw.w);
-}
-__device__ __forceinline__ void buffer_load4(__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_off,
-                                             __half (&out)[4]) {
-  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-  const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_off, row_off, 0);
-  out[0] = __ushort_as_half(static_cast<unsigned short>(raw.x & 0xffffu));
-  out[1] = __ushort_as_half(static_cast<unsigned short>(raw.x >> 16));
-  out[2] = __ushort_as_half(static_cast<unsigned short>(raw.y & 0xffffu));
-  out[3] = __ushort_as_half(static_cast<unsigned short>(raw.y >> 16));
+  return __builtin_bit_cast(typename LaneData<T>::type, raw);
 }
 
 // Number of workgroups for R ROIs and cblk channel blocks (see the job decode
@@ -176,11 +183,12 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
                        int W, int PH, int PW, int S, long long num_images, int cblk,
                        int rows_per_pass, int R) {
   using K = FwdBlocked;
+  constexpr int CPL = BlockOf<T>::CPL, CB = BlockOf<T>::CB, STAGE = BlockOf<T>::STAGE;
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   constexpr int CWIN = K::MAXT / K::PWB;   // column samples per pooled column held at a time
   __shared__ RowEntry rows_s[K::NW][K::ROWT];
   __shared__ ColEntry cols_s[K::NW][K::MAXT];
-  __shared__ __attribute__((aligned(16))) T stage_s[K::NW][K::STAGE];
+  __shared__ __attribute__((aligned(16))) T stage_s[K::NW][STAGE];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -208,9 +216,9 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   }
   if (slot >= R) return;
   const int roi = uni_i(order[slot]);
-  const int c0 = cb * K::CB, nch = min(K::CB, C - c0);
+  const int c0 = cb * CB, nch = min(CB, C - c0);
   const int grp = lane >> 3, quad = lane & 7;   // pooled column within a step, channel quad
-  const bool quad_on = 4 * quad < nch;
+  const bool quad_on = CPL * quad < nch;
   const RoiGeom g = roi_geometry(rois + static_cast<long long>(roi) * 5, scale, PH, PW, S);
   const int bins = PH * PW;
   const int batch = uni_i(g.batch);
@@ -223,8 +231,8 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   RowEntry* const rows = rows_s[wave];
   ColEntry* const cols = cols_s[wave];
   T* const stage = stage_s[wave];
-  const int px_bytes = K::CB * static_cast<int>(sizeof(T)), row_bytes = W * px_bytes;
-  const int lane_off = quad * 4 * static_cast<int>(sizeof(T));
+  const int px_bytes = CB * static_cast<int>(sizeof(T)), row_bytes = W * px_bytes;
+  const int lane_off = quad * 16;
   constexpr int kDead = static_cast<int>(0x80000000u);
 
   // The (image, channel block) plane as a raw buffer: a load whose lane offset
@@ -271,7 +279,9 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
       const bool bin_on = pw < PW && quad_on;
 #pragma nounroll
       for (int ph = ph0; ph < ph0 + rp; ++ph) {
-        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        float acc[CPL];
+#pragma unroll
+        for (int i = 0; i < CPL; ++i) acc[i] = 0.0f;
         if (image_ok) {
 #pragma nounroll
           for (int iy0 = 0; iy0 < gh; iy0 += 2) {
@@ -327,21 +337,21 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
                 if (same) { coff[3] = kDead; cw[3] = 0.0f; }
               }
               // sixteen corners: four rows (scalar) x four columns (per lane)
-              T v[4][4][4];
+              typename LaneData<T>::type v[4][4];
 #pragma unroll
               for (int r = 0; r < 4; ++r)
                 if (rlive[r]) {
 #pragma unroll
-                  for (int c = 0; c < 4; ++c) buffer_load4(plane, coff[c], roff[r], v[r][c]);
+                  for (int c = 0; c < 4; ++c) v[r][c] = buffer_load_lane<T>(plane, coff[c], roff[r]);
                 }
 #pragma unroll
               for (int r = 0; r < 4; ++r)
                 if (rlive[r]) {
 #pragma unroll
-                  for (int i = 0; i < 4; ++i) {
-                    float t = cw[0] * to_float(v[r][0][i]);
+                  for (int i = 0; i < CPL; ++i) {
+                    float t = cw[0] * static_cast<float>(v[r][0][i]);
 #pragma unroll
-                    for (int c = 1; c < 4; ++c) t = fmaf(cw[c], to_float(v[r][c][i]), t);
+                    for (int c = 1; c < 4; ++c) t = fmaf(cw[c], static_cast<float>(v[r][c][i]), t);
                     acc[i] = fmaf(rw[r], t, acc[i]);
                   }
                 }
@@ -350,16 +360,16 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
         }
         if (pow2) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[i] *= inv_count;
+          for (int i = 0; i < CPL; ++i) acc[i] *= inv_count;
         } else {
           asm volatile("" ::: "memory");   // keeps the division out of the common path
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[i] /= count;
+          for (int i = 0; i < CPL; ++i) acc[i] /= count;
         }
         if (bin_on) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            stage[(4 * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i]);
+          for (int i = 0; i < CPL; ++i)
+            stage[(CPL * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i]);
         }
       }
     }

@@ -75,12 +75,13 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
                       int rows_per_pass, int R) {
   using K = FwdBlocked;
   using M = FwdMerged;
+  constexpr int CPL = BlockOf<T>::CPL, CB = BlockOf<T>::CB, STAGE = BlockOf<T>::STAGE;
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   __shared__ MergedEntry rowm_s[K::NW][M::RPH][M::LCAP];
   __shared__ MergedEntry colm_s[K::NW][K::PWB][M::LCAP];
   __shared__ int rown_s[K::NW][M::RPH];
   __shared__ int coln_s[K::NW][K::PWB];
-  __shared__ __attribute__((aligned(16))) T stage_s[K::NW][K::STAGE];
+  __shared__ __attribute__((aligned(16))) T stage_s[K::NW][STAGE];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -105,9 +106,9 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   }
   if (slot >= R) return;
   const int roi = uni_i(order[slot]);
-  const int c0 = cb * K::CB, nch = min(K::CB, C - c0);
+  const int c0 = cb * CB, nch = min(CB, C - c0);
   const int grp = lane >> 3, quad = lane & 7;
-  const bool quad_on = 4 * quad < nch;
+  const bool quad_on = CPL * quad < nch;
   const RoiGeom g = roi_geometry(rois + static_cast<long long>(roi) * 5, scale, PH, PW, S);
   const int bins = PH * PW;
   const int batch = uni_i(g.batch);
@@ -119,8 +120,8 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   int* const rown = rown_s[wave];
   int* const coln = coln_s[wave];
   T* const stage = stage_s[wave];
-  const int px_bytes = K::CB * static_cast<int>(sizeof(T)), row_bytes = W * px_bytes;
-  const int lane_off = quad * 4 * static_cast<int>(sizeof(T));
+  const int px_bytes = CB * static_cast<int>(sizeof(T)), row_bytes = W * px_bytes;
+  const int lane_off = quad * 16;
   constexpr int kDead = static_cast<int>(0x80000000u);
 
   const char* const plane_ptr = reinterpret_cast<const char*>(xt) +
@@ -166,7 +167,9 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
       const bool bin_on = pw < PW && quad_on;
 #pragma nounroll
       for (int ph = ph0; ph < ph0 + rp; ++ph) {
-        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        float acc[CPL];
+#pragma unroll
+        for (int i = 0; i < CPL; ++i) acc[i] = 0.0f;
         if (image_ok) {
 #pragma nounroll
           for (int iyw = 0; iyw < gh; iyw += M::WS) {
@@ -200,21 +203,21 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
                     coff[k] = ok ? e.off + lane_off : kDead;
                     cw[k] = ok ? e.w : 0.0f;
                   }
-                  T v[4][4][4];
+                  typename LaneData<T>::type v[4][4];
 #pragma unroll
                   for (int r = 0; r < 4; ++r)
                     if (rlive[r]) {
 #pragma unroll
-                      for (int c = 0; c < 4; ++c) buffer_load4(plane, coff[c], roff[r], v[r][c]);
+                      for (int c = 0; c < 4; ++c) v[r][c] = buffer_load_lane<T>(plane, coff[c], roff[r]);
                     }
 #pragma unroll
                   for (int r = 0; r < 4; ++r)
                     if (rlive[r]) {
 #pragma unroll
-                      for (int i = 0; i < 4; ++i) {
-                        float t = cw[0] * to_float(v[r][0][i]);
+                      for (int i = 0; i < CPL; ++i) {
+                        float t = cw[0] * static_cast<float>(v[r][0][i]);
 #pragma unroll
-                        for (int c = 1; c < 4; ++c) t = fmaf(cw[c], to_float(v[r][c][i]), t);
+                        for (int c = 1; c < 4; ++c) t = fmaf(cw[c], static_cast<float>(v[r][c][i]), t);
                         acc[i] = fmaf(rw[r], t, acc[i]);
                       }
                     }
@@ -224,11 +227,11 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
           }
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] /= count;
+        for (int i = 0; i < CPL; ++i) acc[i] /= count;
         if (bin_on) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            stage[(4 * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i]);
+          for (int i = 0; i < CPL; ++i)
+            stage[(CPL * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i]);
         }
       }
     }

@@ -109,12 +109,13 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
   if (p.n_out == 0) return;
   using FB = roialign::FwdBlocked;
   const long long pixels = static_cast<long long>(p.H) * p.W;
-  const int cblk = (p.C + FB::CB - 1) / FB::CB;
-  const int rpp = roialign::blocked_rows_per_pass(p.C, p.H, p.W, p.PH, p.PW, sizeof(T));
+  constexpr int CB = roialign::BlockOf<T>::CB;
+  const int cblk = (p.C + CB - 1) / CB;
+  const int rpp = roialign::blocked_rows_per_pass<T>(p.C, p.H, p.W, p.PH, p.PW);
   const long long grid = roialign::blocked_grid(p.R, cblk);
   if (use_tiled() && rpp > 0 && p.N > 0 && p.N < 65536 && cblk < 65536 && grid < (1ll << 31)) {
     // channel-blocked copy of the map, spatial ROI order, then the gather
-    const size_t xt_bytes = (sizeof(T) * p.N * cblk * FB::CB * pixels + 255) / 256 * 256;
+    const size_t xt_bytes = (sizeof(T) * p.N * cblk * CB * pixels + 255) / 256 * 256;
     char* const ws = static_cast<char*>(mobula_hip::workspace(xt_bytes + sizeof(int) * p.R));
     if (failed()) return;
     T* const xt = reinterpret_cast<T*>(ws);

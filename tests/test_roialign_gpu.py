@@ -87,6 +87,24 @@ def test_fp16_storage_forward(impl):
     assert_parity(y.astype(np.float32), want.astype(np.float16).astype(np.float32), FP16_TOL, 'fp16')
 
 
+@pytest.mark.parametrize('S', [2, 0, 3])
+@pytest.mark.parametrize('C', [72, 64, 20])
+def test_fp16_channel_blocks(C, S):
+    # fp16 maps are blocked by 64 channels, eight per lane: a ragged last block (72), exact
+    # blocks (64), and a count that is no multiple of eight (20: straightforward kernel)
+    abi.set_impl('auto')
+    rng = np.random.default_rng(100 * C + S)
+    N, H, W, R, pooled, scale = 2, 30, 44, 60, (7, 7), 0.25
+    x16 = rng.standard_normal((N, C, H, W)).astype(np.float16)
+    c = np.stack([rng.uniform(0, W / scale, R), rng.uniform(0, H / scale, R)], 1)
+    wh = np.stack([rng.uniform(2, W / scale, R), rng.uniform(2, H / scale, R)], 1)
+    rois = np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+    y = abi.forward(abi.to_dev(x16), abi.to_dev(rois), pooled, scale, S).cpu().numpy()
+    assert y.dtype == np.float16
+    want = oracle.forward(x16.astype(np.float32), rois, pooled, scale, S)
+    assert_parity(y.astype(np.float32), want.astype(np.float16).astype(np.float32), FP16_TOL, 'fp16')
+
+
 @pytest.mark.parametrize('impl', IMPLS)
 @pytest.mark.parametrize('shape', [
     # N, C, H, W, R, pooled, scale, S
