@@ -18,9 +18,20 @@ OP_MODULE_GLOBALS = None  # set to mobula.op's namespace when that package is im
 backend = None            # set by glue/__init__.py
 
 
+@functools.lru_cache(maxsize=None)
+def _argspec_of_function(func):
+    return inspect.getfullargspec(func)
+
+
+def _argspec(func):
+    """Signature of a method, looked up once per underlying function (the calls
+    below sit on the per-invocation path of every operator)."""
+    return _argspec_of_function(getattr(func, '__func__', func))
+
+
 def get_varnames(func):
     """Positional parameter names of a method, without `self`."""
-    return inspect.getfullargspec(func).args[1:]
+    return _argspec(func).args[1:]
 
 
 def get_in_data(*args, **kwargs):
@@ -29,7 +40,7 @@ def get_in_data(*args, **kwargs):
 
     Returns (inputs, [ctor_args, ctor_kwargs])  (reference: common.py:68-105)."""
     op = kwargs.pop('op')
-    spec = inspect.getfullargspec(op.forward)
+    spec = _argspec(op.forward)
     names = spec.args[1:]
     n_in = len(names)
     n_opt = len(spec.defaults) if spec.defaults else 0

@@ -85,7 +85,11 @@ def _make_function(op, op_name):
             ret = ret if isinstance(ret, (list, tuple)) else [ret]
             for i in range(len(get_varnames(mod._forward))):
                 mod.assign(mod.in_grad[i], mod.req[i], ret[i])
-        return (None,) + tuple(mod.in_grad)
+        # the operator object lets go of the gradients: a tensor that autograd alone
+        # holds is adopted as .grad, one that is still referenced here is copied first
+        grads = tuple(mod.in_grad)
+        mod.in_grad = mod.out_grad = None
+        return (None,) + grads
 
     return type('_%s_TORCH_FUNC' % op_name, (op, torch.autograd.Function),
                 dict(forward=staticmethod(forward), backward=staticmethod(backward)))
