@@ -173,6 +173,9 @@ def main():
     ap.add_argument('--workload', default='cfg2', choices=['cfg1', 'cfg2', 'cfg3', 'cfg4', 'cfg5'])
     ap.add_argument('--impl', default='auto', choices=['auto', 'tiled', 'naive'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--layout', default='nchw', choices=['nchw', 'nhwc'],
+                    help='nhwc: channels-last tensors through the channels-last entry points (an extension; '
+                         'the reference interface, and the default here, is nchw)')
     ap.add_argument('--conv-compute', default='fp32', choices=['fp32', 'bf16', 'bf16x3'],
                     help='cfg5 only: how the convolution forms its products')
     args = ap.parse_args()
@@ -190,24 +193,27 @@ def main():
 
     w = workloads.make_workload(args.workload)
     pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
-    x = abi.to_dev(w['data'])
+    nhwc = args.layout == 'nhwc'
+    x = abi.to_dev(w['data'].transpose(0, 2, 3, 1) if nhwc else w['data'])
     rois = abi.to_dev(w['rois'])
     has_bwd = w['dy'] is not None
-    dy = abi.to_dev(w['dy']) if has_bwd else None
+    dy = abi.to_dev(w['dy'].transpose(0, 2, 3, 1) if nhwc else w['dy']) if has_bwd else None
     R = rois.shape[0]
     abi.set_impl(args.impl)
     stream = torch.cuda.current_stream().cuda_stream  # launches and events share this stream
 
     dx = torch.empty_like(x) if has_bwd else None
+    run_forward = abi.forward_nhwc if nhwc else abi.forward
+    run_backward = abi.backward_nhwc if nhwc else abi.backward
 
     def step(events=None):
         if events is not None:
             events[0].record()
-        y = abi.forward(x, rois, pooled, scale, S, stream=stream)
+        y = run_forward(x, rois, pooled, scale, S, stream=stream)
         if events is not None:
             events[1].record()
         if has_bwd:
-            abi.backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream)
+            run_backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream)
         if events is not None:
             events[2].record()
         return y
@@ -241,10 +247,10 @@ def main():
             kernel_ms.setdefault(name.value.decode(), []).append(ms)
 
     for _ in range(args.steps):
-        abi.forward(x, rois, pooled, scale, S, stream=stream)
+        run_forward(x, rois, pooled, scale, S, stream=stream)
         note_kernel()
         if has_bwd:
-            abi.backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream)
+            run_backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream)
             note_kernel()
     native.set_option('kernel_timing', 0)
     kernel_ms = {k: sum(v) / len(v) for k, v in kernel_ms.items()}
@@ -260,7 +266,8 @@ def main():
     # The dominant kernel: the longest of the bracketed ones.  Its algorithmic
     # bytes are those of its pass (each tensor of the pass once): the helper
     # kernels around it exist only to feed it.
-    pass_of = {'forward_blocked_kernel': ('forward', b_fwd), 'backward_blocked_kernel': ('backward', b_bwd)}
+    pass_of = {'forward_blocked_kernel': ('forward', b_fwd), 'forward_merged_kernel': ('forward', b_fwd),
+               'backward_blocked_kernel': ('backward', b_bwd)}
     if kernel_ms:
         dom_kernel = max(kernel_ms, key=kernel_ms.get)
         dom_ms = kernel_ms[dom_kernel]
@@ -288,10 +295,11 @@ def main():
         'data': 'synthetic',
         'config': {'workload': '{}: data {} rois {} pooled {} scale {} sampling_ratio {}'.format(
             w['name'], 'x'.join(map(str, w['data'].shape)), R, 'x'.join(map(str, pooled)), scale, S),
-            'impl': args.impl, 'step': 'forward + backward(assign)' if has_bwd else 'forward'},
+            'impl': args.impl, 'layout': args.layout,
+            'step': 'forward + backward(assign)' if has_bwd else 'forward'},
         'roofline': {'bound': 'hbm', 'kernel': dom_kernel, 'achieved': gbs(dom_bytes, dom_ms),
                      'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': gbs(dom_bytes, dom_ms) / HBM_PEAK_GBS,
-                     'traffic': MEASURED_TRAFFIC.get((w['name'], dom_kernel)),
+                     'traffic': None if nhwc else MEASURED_TRAFFIC.get((w['name'], dom_kernel)),
                      'algorithmic_bytes': dom_bytes, 'avg_ms': dom_ms},
         'kernels_ms': kernel_ms,
         'passes': passes,

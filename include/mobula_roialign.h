@@ -77,6 +77,44 @@ void roi_align_forward_e874c59a(const int device_id, const int nthreads,
                                 const int sampling_ratio, const float* bottom_rois,
                                 unsigned short* top_data);
 
+/* The three operations on channels-last tensors: the map as [N,H,W,C], the pooled
+ * tensor as [R,PH,PW,C] (what a torch tensor in torch.channels_last format holds);
+ * scalar arguments as above (channels, height, width name C, H, W).  No
+ * counterpart in the reference, whose binding makes tensors NCHW-contiguous
+ * before the call (mobula/func.py:79-92): with these entry points neither that
+ * copy nor the library's own re-layout of the map and of top_diff is made.
+ * Device pointers only, 16-byte aligned.  A shape the fast kernels do not take is
+ * an error (mobula_hip_last_error), not a slow path: ask
+ * mobula_hip_roialign_nhwc_supported first and convert to NCHW otherwise.  Takes:
+ * forward: channels a multiple of 4 (fp32) or 8 (fp16), pooled_width <= 50, one
+ * image below 2 GiB; backward: fp32, channels a multiple of 4, sampling_ratio 1
+ * or 2, pooled_width <= 16, pooled_height * sampling_ratio <= 32, top_diff below
+ * 2 GiB. */
+void roi_align_forward_nhwc_ab78de3c(const int device_id, const int nthreads, const float* bottom_data,
+                                     const float spatial_scale, const int channels, const int height,
+                                     const int width, const int pooled_height, const int pooled_width,
+                                     const int sampling_ratio, const float* bottom_rois, float* top_data);
+void roi_align_forward_nhwc_e874c59a(const int device_id, const int nthreads,
+                                     const unsigned short* bottom_data, const float spatial_scale,
+                                     const int channels, const int height, const int width,
+                                     const int pooled_height, const int pooled_width,
+                                     const int sampling_ratio, const float* bottom_rois,
+                                     unsigned short* top_data);
+void roi_align_backward_nhwc_f318a24e(const int device_id, const int nthreads, const float* top_diff,
+                                      const float spatial_scale, const int channels, const int height,
+                                      const int width, const int pooled_height, const int pooled_width,
+                                      const int sampling_ratio, float* bottom_diff, const float* bottom_rois);
+void roi_align_backward_nhwc_assign_a8793cbe(const int device_id, const int nthreads, const float* top_diff,
+                                             const float spatial_scale, const int channels, const int height,
+                                             const int width, const int pooled_height, const int pooled_width,
+                                             const int sampling_ratio, const int num_images, float* bottom_diff,
+                                             const float* bottom_rois);
+/* 1 if the channels-last entry points take the shape, else 0.  backward != 0 asks
+ * about the two backward entry points; elem_bytes is 4 (fp32) or 2 (fp16). */
+int mobula_hip_roialign_nhwc_supported(int backward, int elem_bytes, int channels, int height, int width,
+                                       int pooled_height, int pooled_width, int sampling_ratio,
+                                       long long num_rois);
+
 /* ---- Convolution -------------------------------------------------------- */
 
 /* One image: data_col[c, kh, kw, oh, ow] = data_im[c, ih, iw], zero in the

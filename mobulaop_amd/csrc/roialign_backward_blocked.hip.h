@@ -86,6 +86,7 @@ inline long long backward_blocked_grid(long long tiles, int cblk) {
 
 typedef int int16v __attribute__((ext_vector_type(16)));
 
+template <bool NHWC>
 __global__ void __launch_bounds__(BwdBlocked::NT)
 backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
                         const WorkRange* __restrict__ ranges, const WorkEntry* __restrict__ entries,
@@ -139,8 +140,10 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
 
   // dyb and the sample lists as raw buffers: a scalar byte offset per entry
   // plus a fixed lane offset
-  const unsigned dy_ph = static_cast<unsigned>(PWp) * K::CB * sizeof(float);
-  const unsigned dy_roi = dy_ph * PH * cblk;
+  // (NHWC: dyb is the caller's dy[R][PH][PW][C] itself)
+  const unsigned dy_pw = (NHWC ? C : K::CB) * sizeof(float);
+  const unsigned dy_ph = static_cast<unsigned>(NHWC ? PW : PWp) * dy_pw;
+  const unsigned dy_roi = NHWC ? dy_ph * PH : dy_ph * PH * cblk;
   const unsigned list_roi = static_cast<unsigned>(ll.roi_stride) * sizeof(AxisUnit);
   const __amdgpu_buffer_rsrc_t dy_buf = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<float*>(dyb), 0, static_cast<int>(dyb_bytes), 0x00020000);
@@ -154,11 +157,14 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
   // samples of the next are in flight (always eight loads per group, so the
   // wait before a group counts exactly the loads of the group after it).
   for (int pwb = 0; pwb < PW; pwb += K::PWB) {
-    const unsigned dy_fixed = cb * dy_ph * PH + pwb * K::CB * sizeof(float);
+    const unsigned dy_fixed = (NHWC ? cb * K::CB * sizeof(float) : cb * dy_ph * PH) + pwb * dy_pw;
     const unsigned list_fixed = static_cast<unsigned>(
         (static_cast<long long>(ll.ty) * ll.row_stride + static_cast<long long>(tx) * ll.col_stride + pwb) *
         sizeof(AxisUnit));
-    const int dy_lane = lane * 16, list_lane = grp * 16;
+    // a lane whose pooled column or channels do not exist loads from outside the buffer (zero, no access)
+    const int dy_lane = pwb + grp < PW && quad * 4 < nch ? static_cast<int>(grp * dy_pw) + quad * 16
+                                                         : static_cast<int>(0x80000000u);
+    const int list_lane = grp * 16;
     auto issue = [&](const int16v& e, u32x4 (&d)[K::G], u32x4 (&u)[K::G]) {
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
@@ -226,6 +232,25 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
     }
   }
 
+  if (NHWC) {
+    // dx[n][row][col][C]: a pixel's channels of this block are 128 contiguous bytes;
+    // eight pixels per step, a lane moves its four channels
+    float* const px0 = dx + ((static_cast<size_t>(n) * H + r0 + wave) * W + q0) * C + c0 + quad * 4;
+    if (quad * 4 < nch) {
+      for (int col = grp; col < cols; col += 8) {
+        const float4 v = *reinterpret_cast<const float4*>(row + (col + 1) * K::CS + quad * 4);
+        float4* const dst = reinterpret_cast<float4*>(px0 + static_cast<size_t>(col) * C);
+        if (assign) {
+          *dst = v;
+        } else {
+          float4 o = *dst;
+          o.x += v.x; o.y += v.y; o.z += v.z; o.w += v.w;
+          *dst = o;
+        }
+      }
+    }
+    return;
+  }
   // The owner writes its row: one channel plane at a time, lanes along x.
   float* const out = dx + ((static_cast<size_t>(n) * C + c0) * H + r0 + wave) * W + q0;
   const size_t plane = static_cast<size_t>(H) * W;

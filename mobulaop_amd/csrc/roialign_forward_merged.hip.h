@@ -67,7 +67,7 @@ __device__ __forceinline__ int merge_axis_samples(MergedEntry* out, float start,
   return count;
 }
 
-template <typename T>
+template <typename T, bool NHWC>
 __global__ void __launch_bounds__(FwdBlocked::NW * 64, 4)
 forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
                       const int* __restrict__ order, T* __restrict__ y, float scale, int C, int H,
@@ -120,14 +120,16 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   int* const rown = rown_s[wave];
   int* const coln = coln_s[wave];
   T* const stage = stage_s[wave];
-  const int px_bytes = CB * static_cast<int>(sizeof(T)), row_bytes = W * px_bytes;
+  // NHWC: the caller's [N][H][W][C] map is read where it lies, a pixel's channels C * sizeof(T) apart
+  const int px_bytes = (NHWC ? C : CB) * static_cast<int>(sizeof(T)), row_bytes = W * px_bytes;
   const int lane_off = quad * 16;
   constexpr int kDead = static_cast<int>(0x80000000u);
 
+  const size_t image_no = static_cast<size_t>(image_ok ? batch : 0);
   const char* const plane_ptr = reinterpret_cast<const char*>(xt) +
-      (static_cast<size_t>(image_ok ? batch : 0) * cblk + cb) * H * row_bytes;
-  const __amdgpu_buffer_rsrc_t plane =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(plane_ptr), 0, H * row_bytes, 0x00020000);
+      (NHWC ? image_no * H * row_bytes + static_cast<size_t>(cb) * 128 : (image_no * cblk + cb) * H * row_bytes);
+  const __amdgpu_buffer_rsrc_t plane = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(plane_ptr), 0, H * row_bytes - (NHWC ? cb * 128 : 0), 0x00020000);
 
   // Lists held in LDS: rows of pooled rows row_p0 .. row_p0 + RPH - 1 for the
   // sample window starting at row_i0 (lane l builds the list of pooled row
@@ -228,13 +230,23 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
         }
 #pragma unroll
         for (int i = 0; i < CPL; ++i) acc[i] /= count;
-        if (bin_on) {
+        if (NHWC) {
+          // y[roi][ph][pw][C]: the lane's channels of its bin are 16 contiguous bytes
+          if (bin_on) {
+            T out[CPL];
+#pragma unroll
+            for (int i = 0; i < CPL; ++i) out[i] = from_float<T>(acc[i]);
+            T* const dst = y + ((static_cast<size_t>(roi) * PH + ph) * PW + pw) * C + c0 + CPL * quad;
+            *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(out);
+          }
+        } else if (bin_on) {
 #pragma unroll
           for (int i = 0; i < CPL; ++i)
             stage[(CPL * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i]);
         }
       }
     }
+    if (NHWC) continue;
     // the wavefront's outputs of this pass leave LDS in the order of y
     const int total = nch * seg;
     if (rp == PH) {

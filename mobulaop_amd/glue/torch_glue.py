@@ -65,7 +65,13 @@ def _make_function(op, op_name):
         out_shapes = mod.infer_shape(get_in_shape(inputs))[1]
         dtype = inputs[0].dtype if inputs else torch.float32
         device = inputs[0].device if inputs else torch.device('cpu')
-        mod.out_data = [torch.empty(tuple(int(v) for v in s), dtype=dtype, device=device)
+        # an operator that says so gets 4-D outputs in the memory format of a channels-last first input
+        fmt = torch.contiguous_format
+        if (getattr(mod, 'follows_channels_last', False) and inputs and inputs[0].dim() == 4 and
+                not inputs[0].is_contiguous() and inputs[0].is_contiguous(memory_format=torch.channels_last)):
+            fmt = torch.channels_last
+        mod.out_data = [torch.empty(tuple(int(v) for v in s), dtype=dtype, device=device,
+                                    memory_format=fmt if len(s) == 4 else torch.contiguous_format)
                         for s in out_shapes]
         ret = mod._forward(*inputs)
         if ret is not None:

@@ -85,6 +85,18 @@ def exported_names():
     return lib.mobula_hip_exports().decode().split()
 
 
+def roialign_channels_last_supported(backward, elem_bytes, channels, height, width, pooled_size,
+                                     sampling_ratio, num_rois):
+    """True if the channels-last ROIAlign entry points take this shape."""
+    fn = symbol('mobula_hip_roialign_nhwc_supported')
+    if fn is None:
+        return False
+    fn.argtypes = [ctypes.c_int] * 8 + [ctypes.c_longlong]
+    fn.restype = ctypes.c_int
+    return bool(fn(int(bool(backward)), int(elem_bytes), int(channels), int(height), int(width),
+                   int(pooled_size[0]), int(pooled_size[1]), int(sampling_ratio), int(num_rois)))
+
+
 def begin_call(stream, extents):
     lib = library()
     if stream is None:

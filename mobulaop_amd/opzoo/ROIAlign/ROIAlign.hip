@@ -29,6 +29,7 @@ struct Problem {
   int R, C, H, W, PH, PW, S;
   long long N;      // images in the feature map
   float scale;
+  bool nhwc = false;   // map [N,H,W,C] and pooled tensor [R,PH,PW,C] instead of [N,C,H,W] / [R,C,PH,PW]
 };
 
 // Shape checks shared by every entry point.  Returns false (with the error
@@ -104,16 +105,49 @@ int grid_for(long long n, int block) {
 
 bool use_tiled();
 
+// True if the channels-last entry points take the shape (they have no
+// straightforward fallback: the caller converts to NCHW instead).
+template <typename T>
+bool nhwc_forward_supported(const Problem& p) {
+  return roialign::blocked_rows_per_pass<T>(p.C, p.H, p.W, p.PH, p.PW) > 0 &&
+         static_cast<long long>(p.H) * p.W * p.C * static_cast<long long>(sizeof(T)) < (1ll << 31);
+}
+
 template <typename T>
 void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipStream_t stream) {
   if (p.n_out == 0) return;
   using FB = roialign::FwdBlocked;
-  const long long pixels = static_cast<long long>(p.H) * p.W;
   constexpr int CB = roialign::BlockOf<T>::CB;
+  const long long pixels = static_cast<long long>(p.H) * p.W;
   const int cblk = (p.C + CB - 1) / CB;
   const int rpp = roialign::blocked_rows_per_pass<T>(p.C, p.H, p.W, p.PH, p.PW);
   const long long grid = roialign::blocked_grid(p.R, cblk);
-  if (use_tiled() && rpp > 0 && p.N > 0 && p.N < 65536 && cblk < 65536 && grid < (1ll << 31)) {
+  const bool fits = rpp > 0 && p.N > 0 && p.N < 65536 && cblk < 65536 && grid < (1ll << 31);
+  const bool small_grid = p.S == 1 || p.S == 2;   // else: sampling grids above 2 x 2, merged lists
+  if (p.nhwc) {
+    // the map is read where it lies: no copy, only the ROI ordering before the gather
+    if (!fits || !nhwc_forward_supported<T>(p) || reinterpret_cast<size_t>(x) % 16 != 0 ||
+        reinterpret_cast<size_t>(y) % 16 != 0) {
+      set_error("roi_align_forward_nhwc: shape C=%d H=%d W=%d pooled %dx%d (or the alignment of the tensors) "
+                "is not taken by the channels-last path", p.C, p.H, p.W, p.PH, p.PW);
+      return;
+    }
+    int* const order = static_cast<int*>(mobula_hip::workspace(sizeof(int) * p.R));
+    if (failed()) return;
+    roialign::roi_order_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
+    if (small_grid) {
+      mobula_hip::KernelTimer timer("forward_blocked_kernel", stream);
+      roialign::forward_blocked_kernel<T, true><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+          x, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, p.PH, p.R);
+    } else {
+      mobula_hip::KernelTimer timer("forward_merged_kernel", stream);
+      roialign::forward_merged_kernel<T, true><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+          x, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, p.PH, p.R);
+    }
+    MOBULA_HIP_TRY(hipGetLastError());
+    return;
+  }
+  if (use_tiled() && fits) {
     // channel-blocked copy of the map, spatial ROI order, then the gather
     const size_t xt_bytes = (sizeof(T) * p.N * cblk * CB * pixels + 255) / 256 * 256;
     char* const ws = static_cast<char*>(mobula_hip::workspace(xt_bytes + sizeof(int) * p.R));
@@ -133,14 +167,14 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
       roialign::transpose_to_blocked_kernel<T, false><<<tgrid, 256, 0, stream>>>(
           x, xt, p.C, static_cast<int>(pixels));
     side.join();
-    if (p.S == 1 || p.S == 2) {
+    if (small_grid) {
       mobula_hip::KernelTimer timer("forward_blocked_kernel", stream);
-      roialign::forward_blocked_kernel<T><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+      roialign::forward_blocked_kernel<T, false><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
           xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
     } else {
-      // larger (or adaptive) sampling grids: every pixel of a bin is loaded once
+      // every pixel of a bin is loaded once
       mobula_hip::KernelTimer timer("forward_merged_kernel", stream);
-      roialign::forward_merged_kernel<T><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+      roialign::forward_merged_kernel<T, false><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
           xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
     }
     MOBULA_HIP_TRY(hipGetLastError());
@@ -158,8 +192,8 @@ struct TilePlan {
   int* cursors;                // bump pointers: [0] ROI lists, [1] work lists
   int* tile_rois;
   roialign::ListLayout layout;
-  roialign::AxisUnit* lists;   // null unless requested
-  float* dyb;                  // channel-blocked copy of dy, with the lists
+  roialign::AxisUnit* lists;
+  float* dyb;                  // channel-blocked copy of dy (null for channels-last tensors)
   size_t dyb_bytes, list_bytes;
   roialign::WorkRange* ranges; // per (tile, tile row)
   roialign::WorkEntry* entries;
@@ -170,7 +204,7 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // Runs the pre-pass (ROI boxes and sample tables, per-tile ROI and work lists) for tiles of th x tw
 // pixels.  Returns false if the problem is too large for the list buffers (or
 // on error); the caller then uses the straightforward kernels.
-bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_lists,
+bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_dyb,
                 hipStream_t stream, TilePlan* plan) {
   roialign::TileGrid& g = plan->grid;
   g.th = th; g.tw = tw;
@@ -184,31 +218,29 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
   const size_t b_cnt = 256;   // the two bump pointers
   const size_t b_list = align_up(sizeof(int) * std::max<long long>(list_cap, 1), 256);
   plan->layout = roialign::make_list_layout(g, p.PW);
-  const long long n_units = with_lists ? plan->layout.roi_stride * p.R : 0;
+  const long long n_units = plan->layout.roi_stride * p.R;
   if (n_units > (1ll << 25)) return false;   // 512 MiB of sample lists: not worth it
   const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256) + 256;  // blocks are read whole
   const int cblk = (p.C + 31) / 32;
-  const size_t b_dyt = with_lists ? align_up(sizeof(float) * 32 * plan->layout.col_stride * p.R * p.PH * cblk, 256) : 0;
+  const size_t b_dyt = with_dyb ? align_up(sizeof(float) * 32 * plan->layout.col_stride * p.R * p.PH * cblk, 256) : 0;
   // work lists: every tap of every ROI once per tile column it spans
-  const long long n_entries =
-      with_lists ? static_cast<long long>(p.R) * 2 * p.PH * std::max(p.S, 1) * g.tx +
-                       11 * roialign::kTileRows * g.total : 0;
+  const long long n_entries = static_cast<long long>(p.R) * 2 * p.PH * std::max(p.S, 1) * g.tx +
+                              11 * roialign::kTileRows * g.total;
   if (n_entries > (1ll << 27)) return false;
   // the consumer addresses both with 32-bit byte offsets
   if (b_dyt >= (1ull << 31) || b_units >= (1ull << 31)) return false;
   plan->dyb_bytes = b_dyt; plan->list_bytes = b_units;
-  const size_t b_ranges = with_lists ? align_up(sizeof(roialign::WorkRange) * g.total * roialign::kTileRows, 256) : 0;
-  const size_t b_entries = with_lists ? align_up(sizeof(roialign::WorkEntry) * n_entries, 256) + 512 : 0;
+  const size_t b_ranges = align_up(sizeof(roialign::WorkRange) * g.total * roialign::kTileRows, 256);
+  const size_t b_entries = align_up(sizeof(roialign::WorkEntry) * n_entries, 256) + 512;
   char* base = static_cast<char*>(mobula_hip::workspace(b_recs + b_cnt + b_list + b_units + b_dyt +
                                                         b_ranges + b_entries + 256));
   if (failed()) return false;
   plan->boxes = reinterpret_cast<roialign::TileBox*>(base);
   plan->cursors = reinterpret_cast<int*>(base + b_recs);
   plan->tile_rois = reinterpret_cast<int*>(base + b_recs + b_cnt);
-  plan->lists = with_lists ? reinterpret_cast<roialign::AxisUnit*>(base + b_recs + b_cnt + b_list)
-                           : nullptr;
+  plan->lists = reinterpret_cast<roialign::AxisUnit*>(base + b_recs + b_cnt + b_list);
   char* cur = base + b_recs + b_cnt + b_list + b_units;
-  plan->dyb = with_lists ? reinterpret_cast<float*>(cur) : nullptr;
+  plan->dyb = with_dyb ? reinterpret_cast<float*>(cur) : nullptr;
   cur += b_dyt;
   plan->ranges = reinterpret_cast<roialign::WorkRange*>(cur);
   cur += b_ranges;
@@ -227,15 +259,41 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_l
 
 bool use_tiled() { return mobula_hip::option("roialign_impl", kAuto) != kNaive; }
 
+bool nhwc_backward_supported(const Problem& p) {
+  return roialign::backward_blocked_supports(p.PH, p.PW, p.S) && p.C % 4 == 0 &&
+         static_cast<long long>(p.R) * p.PH * p.PW * p.C * 4 < (1ll << 31);
+}
+
 void backward_device(const Problem& p, const float* dy, const float* rois, float* dx, bool assign,
                      hipStream_t stream) {
   if (p.N <= 0) return;
   using BB = roialign::BwdBlocked;
   TilePlan plan;
+  if (p.nhwc) {
+    // dy and dx are used where they lie: only the pre-pass before the tile owners
+    const int cblk = (p.C + BB::CB - 1) / BB::CB;
+    if (!nhwc_backward_supported(p) || reinterpret_cast<size_t>(dy) % 16 != 0 ||
+        reinterpret_cast<size_t>(dx) % 16 != 0 ||
+        !plan_tiles(p, rois, BB::TH, BB::TW, /*with_dyb=*/false, stream, &plan) ||
+        roialign::backward_blocked_grid(plan.grid.total, cblk) >= (1ll << 31)) {
+      if (!failed())
+        set_error("roi_align_backward_nhwc: shape C=%d pooled %dx%d sampling_ratio %d (or the alignment of the "
+                  "tensors) is not taken by the channels-last path", p.C, p.PH, p.PW, p.S);
+      return;
+    }
+    const unsigned dy_bytes = static_cast<unsigned>(sizeof(float) * p.n_out);
+    mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
+    roialign::backward_blocked_kernel<true><<<static_cast<unsigned>(
+        roialign::backward_blocked_grid(plan.grid.total, cblk)), BB::NT, 0, stream>>>(
+        dy, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H, p.W, p.PH, p.PW,
+        cblk, dy_bytes, static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
+    MOBULA_HIP_TRY(hipGetLastError());
+    return;
+  }
   // the pre-pass (small, latency-bound kernels) runs beside the dy transposition
   mobula_hip::SideStream side(stream);
   if (use_tiled() && roialign::backward_blocked_supports(p.PH, p.PW, p.S) &&
-      plan_tiles(p, rois, BB::TH, BB::TW, /*with_lists=*/true, side.get(), &plan)) {
+      plan_tiles(p, rois, BB::TH, BB::TW, /*with_dyb=*/true, side.get(), &plan)) {
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
     // channel blocks per workgroup of the dy transposition: what 64 KB of LDS hold, at most 4
@@ -251,7 +309,7 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
       side.join();
       {
         mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-        roialign::backward_blocked_kernel<<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
+        roialign::backward_blocked_kernel<false><<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
             plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
             p.W, p.PH, p.PW, cblk, static_cast<unsigned>(plan.dyb_bytes),
             static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
@@ -336,6 +394,67 @@ MOBULA_KERNEL roi_align_backward_assign_kernel(const int nthreads, const T* top_
   if (!describe(&p, "roi_align_backward_assign", nthreads, spatial_scale, channels, height, width,
                 pooled_height, pooled_width, sampling_ratio, 10, 11, 1, num_images))
     return;
+  backward_device(p, top_diff, bottom_rois, bottom_diff, /*assign=*/true, call_state().stream);
+}
+
+// Not in the reference: the same three operations on channels-last tensors, the
+// map as [N,H,W,C] and the pooled tensor as [R,PH,PW,C] (what a torch tensor in
+// torch.channels_last format holds).  The kernels read and write these where
+// they lie, so the copies into the blocked layouts are not made.  Shapes the
+// fast kernels do not take are an error here (see
+// mobula_hip_roialign_nhwc_supported); device memory only.
+template <typename T>
+MOBULA_KERNEL roi_align_forward_nhwc_kernel(const int nthreads, const T* bottom_data,
+                                            const float spatial_scale, const int channels,
+                                            const int height, const int width,
+                                            const int pooled_height, const int pooled_width,
+                                            const int sampling_ratio, const float* bottom_rois,
+                                            T* top_data) {
+  Problem p;
+  if (!describe(&p, "roi_align_forward_nhwc", nthreads, spatial_scale, channels, height, width,
+                pooled_height, pooled_width, sampling_ratio, 1, 9, 10, -1))
+    return;
+  p.nhwc = true;
+  hipStream_t stream = call_state().stream;
+  if (p.N < 0) p.N = images_from_rois(bottom_rois, p.R, stream);
+  if (failed()) return;
+  forward_device<T>(p, bottom_data, bottom_rois, top_data, stream);
+}
+
+template <typename T>
+MOBULA_KERNEL roi_align_backward_nhwc_kernel(const int nthreads, const T* top_diff,
+                                             const float spatial_scale, const int channels,
+                                             const int height, const int width,
+                                             const int pooled_height, const int pooled_width,
+                                             const int sampling_ratio, T* bottom_diff,
+                                             const float* bottom_rois) {
+  Problem p;
+  if (!describe(&p, "roi_align_backward_nhwc", nthreads, spatial_scale, channels, height, width,
+                pooled_height, pooled_width, sampling_ratio, 9, 10, 1, -1))
+    return;
+  p.nhwc = true;
+  hipStream_t stream = call_state().stream;
+  if (p.N < 0) p.N = images_from_rois(bottom_rois, p.R, stream);
+  if (failed()) return;
+  backward_device(p, top_diff, bottom_rois, bottom_diff, /*assign=*/false, stream);
+}
+
+template <typename T>
+MOBULA_KERNEL roi_align_backward_nhwc_assign_kernel(const int nthreads, const T* top_diff,
+                                                    const float spatial_scale, const int channels,
+                                                    const int height, const int width,
+                                                    const int pooled_height, const int pooled_width,
+                                                    const int sampling_ratio, const int num_images,
+                                                    T* bottom_diff, const float* bottom_rois) {
+  Problem p;
+  if (num_images < 0) {
+    set_error("roi_align_backward_nhwc_assign: num_images=%d", num_images);
+    return;
+  }
+  if (!describe(&p, "roi_align_backward_nhwc_assign", nthreads, spatial_scale, channels, height, width,
+                pooled_height, pooled_width, sampling_ratio, 10, 11, 1, num_images))
+    return;
+  p.nhwc = true;
   backward_device(p, top_diff, bottom_rois, bottom_diff, /*assign=*/true, call_state().stream);
 }
 
@@ -461,6 +580,74 @@ void roi_align_backward_assign_a8793cbe(const int device_id, const int nthreads,
                         bottom_rois);
 }
 
+// Channels-last variants (extensions): device pointers only.
+#define MOBULA_NHWC_ENTRY(call)                                                            \
+  if (device_id < 0) {                                                                     \
+    set_error("the channels-last entry points take device memory only");                   \
+    return;                                                                                \
+  }                                                                                        \
+  {                                                                                        \
+    mobula_hip::DeviceScope scope(device_id);                                              \
+    if (scope.ok()) call;                                                                  \
+    mobula_hip::finish_call();                                                             \
+  }
+
+void roi_align_forward_nhwc_ab78de3c(const int device_id, const int nthreads, const float* bottom_data,
+                                     const float spatial_scale, const int channels, const int height,
+                                     const int width, const int pooled_height, const int pooled_width,
+                                     const int sampling_ratio, const float* bottom_rois, float* top_data) {
+  MOBULA_NHWC_ENTRY(roi_align_forward_nhwc_kernel<float>(nthreads, bottom_data, spatial_scale, channels, height,
+                                                         width, pooled_height, pooled_width, sampling_ratio,
+                                                         bottom_rois, top_data))
+}
+
+void roi_align_forward_nhwc_e874c59a(const int device_id, const int nthreads, const __half* bottom_data,
+                                     const float spatial_scale, const int channels, const int height,
+                                     const int width, const int pooled_height, const int pooled_width,
+                                     const int sampling_ratio, const float* bottom_rois, __half* top_data) {
+  MOBULA_NHWC_ENTRY(roi_align_forward_nhwc_kernel<__half>(nthreads, bottom_data, spatial_scale, channels, height,
+                                                          width, pooled_height, pooled_width, sampling_ratio,
+                                                          bottom_rois, top_data))
+}
+
+void roi_align_backward_nhwc_f318a24e(const int device_id, const int nthreads, const float* top_diff,
+                                      const float spatial_scale, const int channels, const int height,
+                                      const int width, const int pooled_height, const int pooled_width,
+                                      const int sampling_ratio, float* bottom_diff, const float* bottom_rois) {
+  MOBULA_NHWC_ENTRY(roi_align_backward_nhwc_kernel<float>(nthreads, top_diff, spatial_scale, channels, height,
+                                                          width, pooled_height, pooled_width, sampling_ratio,
+                                                          bottom_diff, bottom_rois))
+}
+
+void roi_align_backward_nhwc_assign_a8793cbe(const int device_id, const int nthreads, const float* top_diff,
+                                             const float spatial_scale, const int channels, const int height,
+                                             const int width, const int pooled_height, const int pooled_width,
+                                             const int sampling_ratio, const int num_images, float* bottom_diff,
+                                             const float* bottom_rois) {
+  MOBULA_NHWC_ENTRY(roi_align_backward_nhwc_assign_kernel<float>(nthreads, top_diff, spatial_scale, channels,
+                                                                 height, width, pooled_height, pooled_width,
+                                                                 sampling_ratio, num_images, bottom_diff,
+                                                                 bottom_rois))
+}
+#undef MOBULA_NHWC_ENTRY
+
+// 1 if the channels-last entry points take the shape, else 0.  backward != 0 asks
+// about the two backward entry points (fp32 only), elem_bytes is 4 (fp32) or 2 (fp16).
+int mobula_hip_roialign_nhwc_supported(int backward, int elem_bytes, int channels, int height, int width,
+                                       int pooled_height, int pooled_width, int sampling_ratio,
+                                       long long num_rois) {
+  if (channels <= 0 || height <= 0 || width <= 0 || pooled_height <= 0 || pooled_width <= 0 || num_rois < 0 ||
+      num_rois > (1ll << 30))
+    return 0;
+  Problem p;
+  p.R = static_cast<int>(num_rois); p.C = channels; p.H = height; p.W = width;
+  p.PH = pooled_height; p.PW = pooled_width; p.S = sampling_ratio;
+  if (backward) return elem_bytes == 4 && nhwc_backward_supported(p) ? 1 : 0;
+  if (elem_bytes == 4) return nhwc_forward_supported<float>(p) ? 1 : 0;
+  if (elem_bytes == 2) return nhwc_forward_supported<__half>(p) ? 1 : 0;
+  return 0;
+}
+
 void roi_align_forward_e874c59a(const int device_id, const int nthreads, const __half* bottom_data,
                                 const float spatial_scale, const int channels, const int height,
                                 const int width, const int pooled_height, const int pooled_width,
@@ -474,4 +661,6 @@ void roi_align_forward_e874c59a(const int device_id, const int nthreads, const _
 
 static mobula_hip::ExportRegistrar roialign_exports(
     "roi_align_forward_ab78de3c roi_align_backward_f318a24e roi_align_backward_assign_a8793cbe "
-    "roi_align_forward_e874c59a");
+    "roi_align_forward_e874c59a roi_align_forward_nhwc_ab78de3c roi_align_forward_nhwc_e874c59a "
+    "roi_align_backward_nhwc_f318a24e roi_align_backward_nhwc_assign_a8793cbe "
+    "mobula_hip_roialign_nhwc_supported");

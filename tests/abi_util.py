@@ -77,6 +77,43 @@ def backward(dy, rois, shape, scale, S, dx=None, assign=False, declare_extents=T
     return dx
 
 
+def forward_nhwc(x, rois, pooled, scale, S, dev=0, stream=None):
+    """x: cuda tensor [N,H,W,C] (fp32 or fp16); returns y [R,PH,PW,C]."""
+    N, H, W, C = x.shape
+    PH, PW = pooled
+    R = rois.shape[0]
+    y = torch.empty((R, PH, PW, C), dtype=x.dtype, device=x.device)
+    ext = [-1, x.numel(), -1, -1, -1, -1, -1, -1, -1, rois.numel(), y.numel()]
+    lib = _begin(ext, stream)
+    fn = lib.roi_align_forward_nhwc_ab78de3c if x.dtype == torch.float32 else lib.roi_align_forward_nhwc_e874c59a
+    fn(ctypes.c_int(dev), ctypes.c_int(y.numel()), _ptr(x), *_geom(scale, C, H, W, PH, PW, S),
+       _ptr(rois), _ptr(y))
+    _end(lib)
+    return y
+
+
+def backward_nhwc(dy, rois, shape, scale, S, dx=None, assign=False, dev=0, stream=None):
+    """dy: cuda fp32 [R,PH,PW,C]; shape = (N,H,W,C) of dx."""
+    N, H, W, C = shape
+    PH, PW = dy.shape[1], dy.shape[2]
+    if dx is None:
+        dx = (torch.full(shape, float('nan'), dtype=dy.dtype, device=dy.device) if assign
+              else torch.zeros(shape, dtype=dy.dtype, device=dy.device))
+    lib = native.library()
+    if assign:
+        _begin([-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()], stream)
+        lib.roi_align_backward_nhwc_assign_a8793cbe(
+            ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
+            ctypes.c_int(N), _ptr(dx), _ptr(rois))
+    else:
+        _begin([-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()], stream)
+        lib.roi_align_backward_nhwc_f318a24e(
+            ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
+            _ptr(dx), _ptr(rois))
+    _end(lib)
+    return dx
+
+
 def set_impl(name):
     native.set_option('roialign_impl', IMPL[name])
 

@@ -129,3 +129,23 @@ def test_runs_on_the_callers_stream(mobula):
         doubled = y * 2          # ordered after the kernel on the same stream
     side.synchronize()
     assert_parity(doubled, 2 * want_y, FWD_TOL, 'stream')
+
+
+def test_channels_last_tensors_take_the_channels_last_path(mobula):
+    # same numbers as with NCHW tensors; outputs and gradients come back channels-last
+    torch.manual_seed(5)
+    x = torch.randn(2, 32, 20, 24, device='cuda')
+    rois = torch.tensor([[0, 1, 2, 60, 50], [1, 10, 10, 90, 70], [1, -5, 3, 20, 100]], device='cuda',
+                        dtype=torch.float32)
+    kw = dict(pooled_size=(7, 7), spatial_scale=0.25, sampling_ratio=2)
+    xa = x.clone().requires_grad_(True)
+    ya = mobula.op.ROIAlign(xa, rois, **kw)
+    dy = torch.randn_like(ya)
+    ya.backward(dy)
+    xb = x.clone().to(memory_format=torch.channels_last).requires_grad_(True)
+    yb = mobula.op.ROIAlign(xb, rois, **kw)
+    assert yb.is_contiguous(memory_format=torch.channels_last) and not yb.is_contiguous()
+    yb.backward(dy)
+    assert xb.grad.is_contiguous(memory_format=torch.channels_last)
+    assert float((ya - yb).detach().abs().max()) <= 1e-5 * float(ya.detach().abs().max())
+    assert float((xa.grad - xb.grad).abs().max()) <= 1e-4 * float(xa.grad.abs().max())

@@ -136,6 +136,63 @@ def test_ragged_shapes(impl, shape):
         assert_parity(dx.cpu().numpy(), want, BWD_TOL, 'bwd assign=%s' % assign)
 
 
+@pytest.mark.parametrize('shape', [
+    # N, C, H, W, R, pooled, scale, S
+    (3, 68, 33, 47, 37, (7, 7), 0.25, 2),     # ragged last channel block
+    (2, 128, 18, 70, 50, (14, 14), 0.125, 2),
+    (2, 32, 40, 40, 25, (7, 7), 1.0, 1),
+])
+def test_channels_last_entry_points(shape):
+    # map [N,H,W,C], pooled tensor [R,PH,PW,C]: same numbers as the NCHW oracle, transposed
+    abi.set_impl('auto')
+    N, C, H, W, R, pooled, scale, S = shape
+    rng = np.random.default_rng(hash(shape) & 0xffff)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    ext_w, ext_h = W / scale, H / scale
+    c = np.stack([rng.uniform(-0.2 * ext_w, 1.2 * ext_w, R), rng.uniform(-0.2 * ext_h, 1.2 * ext_h, R)], 1)
+    wh = np.stack([rng.uniform(0, ext_w, R), rng.uniform(0, ext_h, R)], 1)
+    rois = np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+    dy = rng.standard_normal((R, C) + pooled).astype(np.float32)
+    y = abi.forward_nhwc(abi.to_dev(x.transpose(0, 2, 3, 1)), abi.to_dev(rois), pooled, scale, S)
+    assert_parity(y.cpu().numpy().transpose(0, 3, 1, 2), oracle.forward(x, rois, pooled, scale, S), FWD_TOL, 'fwd')
+    want = oracle.backward(dy, rois, x.shape, scale, S, impl='ordered')
+    dy_l = abi.to_dev(dy.transpose(0, 2, 3, 1))
+    for assign in (False, True):
+        dx = abi.backward_nhwc(dy_l, abi.to_dev(rois), (N, H, W, C), scale, S, assign=assign)
+        assert_parity(dx.cpu().numpy().transpose(0, 3, 1, 2), want, BWD_TOL, 'bwd assign=%s' % assign)
+    # accumulation into an existing gradient
+    base = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    dx = abi.backward_nhwc(dy_l, abi.to_dev(rois), (N, H, W, C), scale, S, dx=abi.to_dev(base))
+    assert_parity(dx.cpu().numpy().transpose(0, 3, 1, 2), want + base.transpose(0, 3, 1, 2), BWD_TOL, 'accumulate')
+
+
+def test_channels_last_fp16_and_adaptive_grid():
+    abi.set_impl('auto')
+    rng = np.random.default_rng(77)
+    N, C, H, W, R, pooled, scale = 2, 72, 30, 44, 60, (7, 7), 0.25
+    x16 = rng.standard_normal((N, C, H, W)).astype(np.float16)
+    c = np.stack([rng.uniform(0, W / scale, R), rng.uniform(0, H / scale, R)], 1)
+    wh = np.stack([rng.uniform(2, W / scale, R), rng.uniform(2, H / scale, R)], 1)
+    rois = np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+    for S in (2, 0):
+        y = abi.forward_nhwc(abi.to_dev(x16.transpose(0, 2, 3, 1)), abi.to_dev(rois), pooled, scale, S)
+        want = oracle.forward(x16.astype(np.float32), rois, pooled, scale, S)
+        assert_parity(y.cpu().numpy().astype(np.float32).transpose(0, 3, 1, 2),
+                      want.astype(np.float16).astype(np.float32), FP16_TOL, 'fp16 S=%d' % S)
+
+
+def test_channels_last_rejects_what_it_does_not_take():
+    x = torch.zeros(1, 8, 8, 6, device='cuda')          # six channels: no multiple of four
+    rois = torch.tensor([[0, 1, 1, 6, 6]], device='cuda', dtype=torch.float32)
+    with pytest.raises(RuntimeError, match='channels-last'):
+        abi.forward_nhwc(x, rois, (2, 2), 1.0, 2)
+    dy = torch.zeros(1, 7, 7, 8, device='cuda')          # adaptive grid: not taken by the backward
+    with pytest.raises(RuntimeError, match='channels-last'):
+        abi.backward_nhwc(dy, rois, (1, 8, 8, 8), 1.0, 0)
+    # the library is usable afterwards
+    assert abi.forward_nhwc(torch.zeros(1, 8, 8, 8, device='cuda'), rois, (2, 2), 1.0, 2).shape == (1, 2, 2, 8)
+
+
 @pytest.mark.parametrize('impl', IMPLS)
 def test_empty_roi_list_and_out_of_range_batch(impl):
     abi.set_impl(impl)
