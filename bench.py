@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # absent entries are reported as null.
 MEASURED_TRAFFIC = {
     ('cfg2', 'forward_blocked_kernel'): 473.4e6,    # 272.7 MB read + 200.7 MB written
-    ('cfg2', 'backward_blocked_kernel'): 564.6e6,   # 301.0 MB read + 295.0 MB written
+    ('cfg2', 'backward_blocked_kernel'): 564.6e6,   # 270.8 MB read + 293.8 MB written
 }
 
 
