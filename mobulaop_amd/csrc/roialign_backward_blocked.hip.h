@@ -1,10 +1,13 @@
 // Backward ROIAlign: tile owners accumulate in LDS, 16 bytes per lane.
 //
-// dx is cut into tiles of 16 rows x 56 columns x 32 channels.  One workgroup
-// owns one tile, keeps it in LDS as acc[row][column][channel] and is the only
-// writer of that piece of dx: no atomics anywhere and a summation order fixed
-// by the ROI order.  Wavefront w owns tile row w, so the sixteen wavefronts
-// never touch the same cell and need no barrier.  The 64 lanes of a wavefront
+// dx is cut into tiles of 16 rows x 56 columns x 32 channels, and a tile into
+// bands of TH rows.  One workgroup owns one band, keeps it in LDS as
+// acc[row][column][channel] and is the only writer of that piece of dx: no
+// atomics anywhere and a summation order fixed by the ROI order.  Wavefront w
+// owns row w of the band, so the wavefronts never touch the same cell and need
+// no barrier; nothing but the launch ties the wavefronts of a workgroup
+// together, and small bands (several workgroups resident per CU) keep a CU
+// busy when the rows of a tile have work lists of different length.  The 64 lanes of a wavefront
 // are 8 pooled columns x 8 channel quads: a lane folds the row taps of a ROI
 // into four gradients (its pooled column, its four channels) and adds them to
 // the two cells of each of its column samples with 16-byte LDS accesses.
@@ -19,7 +22,8 @@
 namespace roialign {
 
 struct BwdBlocked {
-  static constexpr int TH = kTileRows;   // tile rows = wavefronts
+  static constexpr int TH = 2;           // rows of a band = wavefronts of a workgroup
+  static constexpr int BANDS = kTileRows / TH;   // bands per tile
   static constexpr int TW = 56;          // tile columns
   static constexpr int CB = 32;          // channels per workgroup
   static constexpr int NW = TH;
@@ -78,6 +82,7 @@ transpose_dy_blocked_kernel(const float* __restrict__ dy, float* __restrict__ dy
 // Number of workgroups for `tiles` tiles and cblk channel blocks (job decode at
 // the top of backward_blocked_kernel).
 inline long long backward_blocked_grid(long long tiles, int cblk) {
+  tiles *= BwdBlocked::BANDS;   // one workgroup per band
   long long per_xcd;
   if (cblk >= 8) per_xcd = tiles * ((cblk + 7) / 8);
   else per_xcd = (tiles + (8 / cblk) - 1) / (8 / cblk);
@@ -98,7 +103,7 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
 
   // Job decode.  Workgroups are dealt to the 8 XCDs round-robin, so blockIdx % 8
   // names the XCD: it takes the channel blocks b with b % 8 == xcd (their slice
-  // of dyb then stays in that XCD's L2) and walks the tiles in order; with
+  // of dyb then stays in that XCD's L2) and walks the bands of the tiles in order; with
   // fewer than 8 blocks the tiles of a block are split into 8 / cblk ranges.
   const int xcd = blockIdx.x & 7;
   const long long wi = blockIdx.x >> 3;
@@ -112,15 +117,17 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
     const int parts = 8 / cblk;
     cb = xcd % cblk;
     const int part = xcd / cblk;
-    const long long range = (tg.total + parts - 1) / parts;
+    const long long range = (tg.total * K::BANDS + parts - 1) / parts;
     if (part >= parts || wi >= range) return;
     tile = part * range + wi;
   }
-  if (tile >= tg.total) return;
+  if (tile >= tg.total * K::BANDS) return;
+  const int band = static_cast<int>(tile % K::BANDS);
+  tile /= K::BANDS;
   const int n = static_cast<int>(tile / tg.per_image);
   const int t_in_img = static_cast<int>(tile % tg.per_image);
   const int ty = t_in_img / tg.tx, tx = t_in_img % tg.tx;
-  const int r0 = ty * K::TH, q0 = tx * K::TW;
+  const int r0 = ty * kTileRows + band * K::TH, q0 = tx * K::TW;
   const int c0 = cb * K::CB, nch = min(K::CB, C - c0);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // = the tile row owned
@@ -132,7 +139,7 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
   for (int i = lane; i < K::RS * K::CS / 4; i += 64)
     reinterpret_cast<float4*>(row)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 
-  const WorkRange wr = ranges[tile * kTileRows + wave];
+  const WorkRange wr = ranges[tile * kTileRows + band * K::TH + wave];
   const int n_entries = wr.count;   // a multiple of 2 * G, and G more entries follow: the lists are padded
   const int16v* const wl = reinterpret_cast<const int16v*>(entries + wr.begin);
   const int PWp = ll.col_stride;

@@ -274,7 +274,7 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     if (!nhwc_backward_supported(p) || reinterpret_cast<size_t>(dy) % 16 != 0 ||
         reinterpret_cast<size_t>(dx) % 16 != 0 ||
-        !plan_tiles(p, rois, BB::TH, BB::TW, /*with_dyb=*/false, stream, &plan) ||
+        !plan_tiles(p, rois, roialign::kTileRows, BB::TW, /*with_dyb=*/false, stream, &plan) ||
         roialign::backward_blocked_grid(plan.grid.total, cblk) >= (1ll << 31)) {
       if (!failed())
         set_error("roi_align_backward_nhwc: shape C=%d pooled %dx%d sampling_ratio %d (or the alignment of the "
@@ -293,7 +293,7 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
   // the pre-pass (small, latency-bound kernels) runs beside the dy transposition
   mobula_hip::SideStream side(stream);
   if (use_tiled() && roialign::backward_blocked_supports(p.PH, p.PW, p.S) &&
-      plan_tiles(p, rois, BB::TH, BB::TW, /*with_dyb=*/true, side.get(), &plan)) {
+      plan_tiles(p, rois, roialign::kTileRows, BB::TW, /*with_dyb=*/true, side.get(), &plan)) {
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
     // channel blocks per workgroup of the dy transposition: what 64 KB of LDS hold, at most 4
