@@ -176,6 +176,11 @@ inline long long blocked_grid(long long R, int cblk) {
   return 8 * ((per_xcd + K::NW - 1) / K::NW);
 }
 
+// The same for channels-last maps (see the job decode).
+inline long long blocked_grid_nhwc(long long R, int cblk) {
+  return 8 * (((R + 7) / 8 * cblk + FwdBlocked::NW - 1) / FwdBlocked::NW);
+}
+
 template <typename T, bool NHWC>
 __global__ void __launch_bounds__(FwdBlocked::NW * 64, 4)
 forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
@@ -202,7 +207,15 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   const long long wi = static_cast<long long>(blockIdx.x >> 3) * K::NW + wave;
   long long slot;
   int cb;
-  if (cblk >= 8) {
+  if (NHWC) {
+    // the caller's map: an XCD takes an eighth of the (spatially sorted) ROIs with
+    // all their channel blocks, neighbouring wavefronts read neighbouring lines
+    const long long range = (R + 7) / 8;
+    const long long s = wi / cblk;
+    if (s >= range) return;
+    slot = xcd * range + s;
+    cb = static_cast<int>(wi - s * cblk);
+  } else if (cblk >= 8) {
     const int nx = (cblk - xcd + 7) >> 3;
     slot = wi / nx;
     cb = xcd + 8 * static_cast<int>(wi % nx);

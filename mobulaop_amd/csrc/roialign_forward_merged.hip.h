@@ -92,7 +92,15 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   const long long wi = static_cast<long long>(blockIdx.x >> 3) * K::NW + wave;
   long long slot;
   int cb;
-  if (cblk >= 8) {
+  if (NHWC) {
+    // the caller's map: an XCD takes an eighth of the (spatially sorted) ROIs with
+    // all their channel blocks, neighbouring wavefronts read neighbouring lines
+    const long long range = (R + 7) / 8;
+    const long long s = wi / cblk;
+    if (s >= range) return;
+    slot = xcd * range + s;
+    cb = static_cast<int>(wi - s * cblk);
+  } else if (cblk >= 8) {
     const int nx = (cblk - xcd + 7) >> 3;
     slot = wi / nx;
     cb = xcd + 8 * static_cast<int>(wi % nx);

@@ -135,6 +135,7 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
     int* const order = static_cast<int*>(mobula_hip::workspace(sizeof(int) * p.R));
     if (failed()) return;
     roialign::roi_order_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
+    const long long grid = roialign::blocked_grid_nhwc(p.R, cblk);
     if (small_grid) {
       mobula_hip::KernelTimer timer("forward_blocked_kernel", stream);
       roialign::forward_blocked_kernel<T, true><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
