@@ -313,9 +313,23 @@ __device__ __forceinline__ int tile_of_block(int count) {
   return (blockIdx.x >> 3) < per && t < count ? t : -1;
 }
 
-// C[M, Ncols] = A[M, K] x B[K, Ncols], one 128x128 tile per workgroup.
-template <typename Ops, int MODE>
-__device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
+// Where a tile's results go: through the operand functor, or (piece != nullptr:
+// the tile covers part of K only) into a dense 128x128 piece buffer.
+template <typename Ops>
+struct StoreResult {
+  const Ops& ops;
+  float* piece;
+  __device__ void operator()(int m, int n, int lm, int ln, float v) const {
+    if (piece != nullptr) piece[lm * Tile::BN + ln] = v;
+    else ops.store(m, n, v);
+  }
+};
+
+// C[M, Ncols] = A[M, K] x B[K, Ncols], one 128x128 tile per workgroup, over the K
+// steps s_begin .. s_end - 1; results go to store(m, n, row in tile, column in tile, value).
+template <typename Ops, int MODE, typename Store>
+__device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0, int s_begin, int s_end,
+                                           const Store& store) {
   using T = Tile;
   constexpr bool BF16 = MODE != kFp32;
   constexpr int PARTS = MODE == kBf16x3 ? 2 : 1;   // head, tail
@@ -379,13 +393,13 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
     }
   };
 
-  const int steps = (ops.K + T::BK - 1) / T::BK;
+  const int steps = s_end;
   const int half = lane >> 5, col = lane & 31;
-  fetch(0);
+  fetch(s_begin);
   stage(0);
   __syncthreads();
-  for (int s = 0; s < steps; ++s) {
-    const int buf = s & 1;
+  for (int s = s_begin; s < steps; ++s) {
+    const int buf = (s - s_begin) & 1;
     if (s + 1 < steps) fetch(s + 1);
     if (BF16) {
       bf16x8 a[PARTS][2], b[PARTS][2];
@@ -436,19 +450,56 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0) {
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int row = 8 * (v >> 2) + 4 * half + (v & 3);
-        ops.store(m0 + wm + i * 32 + row, n0 + wn + j * 32 + col, acc[i][j][v]);
+        const int row = wm + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3), column = wn + j * 32 + col;
+        store(m0 + row, n0 + column, row, column, acc[i][j][v]);
       }
 }
+
+__host__ __device__ inline int k_steps(int K) { return (K + Tile::BK - 1) / Tile::BK; }
+
+// How a launch covers `count` tiles: the first `whole` tiles by one workgroup
+// each; each of the others by `pieces` workgroups that take `steps_per_piece`
+// K steps apiece and leave their sums in a piece buffer (added up, in order,
+// by reduce_pieces_kernel).  The split evens out the last round of a launch
+// whose tile count is a little more than a multiple of what the device holds
+// at a time, and fills the device when there are few tiles.
+struct TileSplit {
+  int whole, pieces, steps_per_piece;
+};
 
 // Tiles in column-major order: the row tiles of one column tile are neighbours
 // and read the same gathered operand.
 template <typename Ops, int MODE>
 __global__ void __launch_bounds__(Tile::NT)
-igemm_kernel(Ops ops, int row_tiles, int count) {
-  const int t = tile_of_block(count);
-  if (t < 0) return;
-  igemm_tile<Ops, MODE>(ops, (t % row_tiles) * Tile::BM, (t / row_tiles) * Tile::BN);
+igemm_kernel(Ops ops, int row_tiles, TileSplit split, float* __restrict__ piece_buffer) {
+  const int whole_blocks = tile_blocks(split.whole);
+  int t, s_begin = 0, s_end = k_steps(ops.K);
+  float* piece = nullptr;
+  if (static_cast<int>(blockIdx.x) < whole_blocks) {
+    t = tile_of_block(split.whole);
+    if (t < 0) return;
+  } else {
+    const int q = blockIdx.x - whole_blocks;
+    t = split.whole + q / split.pieces;
+    s_begin = (q % split.pieces) * split.steps_per_piece;
+    s_end = min(s_end, s_begin + split.steps_per_piece);
+    piece = piece_buffer + static_cast<size_t>(q) * Tile::BM * Tile::BN;
+  }
+  igemm_tile<Ops, MODE>(ops, (t % row_tiles) * Tile::BM, (t / row_tiles) * Tile::BN, s_begin, s_end,
+                        StoreResult<Ops>{ops, piece});
+}
+
+// Results of the split tiles: sum of their pieces, in piece order.
+template <typename Ops>
+__global__ void __launch_bounds__(256)
+reduce_pieces_kernel(Ops ops, int row_tiles, TileSplit split, const float* __restrict__ piece_buffer) {
+  constexpr int TILE = Tile::BM * Tile::BN;
+  const int local = blockIdx.x / (TILE / 256), e = (blockIdx.x % (TILE / 256)) * 256 + threadIdx.x;
+  const int t = split.whole + local;
+  const float* p = piece_buffer + static_cast<size_t>(local) * split.pieces * TILE + e;
+  float sum = 0.0f;
+  for (int i = 0; i < split.pieces; ++i) sum += p[static_cast<size_t>(i) * TILE];
+  ops.store((t % row_tiles) * Tile::BM + e / Tile::BN, (t / row_tiles) * Tile::BN + e % Tile::BN, sum);
 }
 
 // Slices of K times tiles, slice-major; every slice writes its own partial.
@@ -462,7 +513,8 @@ igemm_weight_kernel(BackwardWeightOps ops, int k_per_slice, int k_total, int row
   ops.k_begin = slice * k_per_slice;
   ops.K = min(k_per_slice, k_total - ops.k_begin);
   ops.partial += static_cast<size_t>(slice) * ops.M * ops.Ncols;
-  igemm_tile<BackwardWeightOps, MODE>(ops, (tile % row_tiles) * Tile::BM, (tile / row_tiles) * Tile::BN);
+  igemm_tile<BackwardWeightOps, MODE>(ops, (tile % row_tiles) * Tile::BM, (tile / row_tiles) * Tile::BN, 0,
+                                      k_steps(ops.K), StoreResult<BackwardWeightOps>{ops, nullptr});
 }
 
 // out[i] (+)= sum over slices of partial[s][i]

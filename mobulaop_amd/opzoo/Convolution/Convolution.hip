@@ -26,18 +26,64 @@ int compute_mode() {
   return mode == conv::kBf16 || mode == conv::kBf16x3 ? mode : conv::kFp32;
 }
 
-template <typename Ops>
-void launch_igemm(const Ops& ops, hipStream_t stream) {
+// Workgroups of igemm_kernel<Ops, MODE> the device holds at a time.
+template <typename Ops, int MODE>
+int resident_workgroups() {
+  static thread_local int cached_device = -1, cached = 0;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return 0;
+  if (device != cached_device) {
+    int per_cu = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, conv::igemm_kernel<Ops, MODE>, conv::Tile::NT, 0) !=
+            hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) {
+      (void)hipGetLastError();
+      return 0;
+    }
+    cached = per_cu * cus;
+    cached_device = device;
+  }
+  return cached;
+}
+
+// Most piece workgroups a launch uses (sizes the piece buffer): no more than the
+// device holds at a time, and no device is assumed to hold more than this.
+constexpr int kMaxPieceBlocks = 2048;
+
+conv::TileSplit split_tiles(int count, int steps, int resident) {
+  conv::TileSplit split{count, 1, steps};
+  resident = std::min(resident, kMaxPieceBlocks);
+  if (resident <= 0 || steps < 2) return split;
+  const int rest = count % resident;
+  // a last round that fills less than half of the device is cut along K
+  if (rest == 0 || rest > resident / 2) return split;
+  int pieces = std::min(resident / rest, steps);
+  if (pieces < 2) return split;
+  split.steps_per_piece = (steps + pieces - 1) / pieces;
+  split.pieces = (steps + split.steps_per_piece - 1) / split.steps_per_piece;
+  split.whole = count - rest;
+  return split;
+}
+
+template <typename Ops, int MODE>
+void launch_igemm_mode(const Ops& ops, float* piece_buffer, hipStream_t stream) {
   const int row_tiles = (ops.M + conv::Tile::BM - 1) / conv::Tile::BM;
   const int count = row_tiles * ((ops.Ncols + conv::Tile::BN - 1) / conv::Tile::BN);
-  const dim3 grid(conv::tile_blocks(count));
+  const conv::TileSplit split = split_tiles(count, conv::k_steps(ops.K), resident_workgroups<Ops, MODE>());
+  const int rest = count - split.whole;
+  const dim3 grid(conv::tile_blocks(split.whole) + rest * split.pieces);
+  conv::igemm_kernel<Ops, MODE><<<grid, conv::Tile::NT, 0, stream>>>(ops, row_tiles, split, piece_buffer);
+  if (rest > 0)
+    conv::reduce_pieces_kernel<Ops><<<rest * (conv::Tile::BM * conv::Tile::BN / 256), 256, 0, stream>>>(
+        ops, row_tiles, split, piece_buffer);
+}
+
+template <typename Ops>
+void launch_igemm(const Ops& ops, float* piece_buffer, hipStream_t stream) {
   switch (compute_mode()) {
-    case conv::kBf16:
-      conv::igemm_kernel<Ops, conv::kBf16><<<grid, conv::Tile::NT, 0, stream>>>(ops, row_tiles, count); break;
-    case conv::kBf16x3:
-      conv::igemm_kernel<Ops, conv::kBf16x3><<<grid, conv::Tile::NT, 0, stream>>>(ops, row_tiles, count); break;
-    default:
-      conv::igemm_kernel<Ops, conv::kFp32><<<grid, conv::Tile::NT, 0, stream>>>(ops, row_tiles, count);
+    case conv::kBf16: launch_igemm_mode<Ops, conv::kBf16>(ops, piece_buffer, stream); break;
+    case conv::kBf16x3: launch_igemm_mode<Ops, conv::kBf16x3>(ops, piece_buffer, stream); break;
+    default: launch_igemm_mode<Ops, conv::kFp32>(ops, piece_buffer, stream);
   }
 }
 
@@ -99,7 +145,7 @@ conv::Tap* make_taps(int count, int KH, int KW, int plane, int dil_h, int dil_w,
 // Workspace of a gathered product (forward, data gradient): the table of K
 // steps and the weights in [Mpad][taps][Cpad] order.  channels = what K runs
 // over besides the taps, plane_row = row length of the gathered tensor.
-struct GatherPlan { conv::GatherStep* steps; float* weights; int K; };
+struct GatherPlan { conv::GatherStep* steps; float* weights; float* pieces; int K; };
 
 bool plan_gather(GatherPlan* plan, const char* what, const conv::Geometry& g, const float* w, int M,
                  int channels, long long image_elems, int columns_per_image, int plane_row, int sign,
@@ -116,10 +162,13 @@ bool plan_gather(GatherPlan* plan, const char* what, const conv::Geometry& g, co
   if (k >= (1ll << 31) || wcount >= (1ll << 31)) { set_error("%s: weights too large", what); return false; }
   const int count = taps * per_tap;
   const size_t step_bytes = (sizeof(conv::GatherStep) * count + 255) / 256 * 256;
-  char* ws = static_cast<char*>(mobula_hip::workspace(step_bytes + sizeof(float) * wcount));
+  const size_t weight_bytes = (sizeof(float) * wcount + 255) / 256 * 256;
+  const size_t piece_bytes = sizeof(float) * kMaxPieceBlocks * conv::Tile::BM * conv::Tile::BN;
+  char* ws = static_cast<char*>(mobula_hip::workspace(step_bytes + weight_bytes + piece_bytes));
   if (failed()) return false;
   plan->steps = reinterpret_cast<conv::GatherStep*>(ws);
   plan->weights = reinterpret_cast<float*>(ws + step_bytes);
+  plan->pieces = reinterpret_cast<float*>(ws + step_bytes + weight_bytes);
   plan->K = static_cast<int>(k);
   conv::build_gather_steps_kernel<<<(count + 255) / 256, 256, 0, stream>>>(plan->steps, count, per_tap, g.KW,
                                                                           g.dil_h, g.dil_w, plane_row, sign);
@@ -196,7 +245,7 @@ MOBULA_KERNEL conv2d_forward_kernel(const int n, const T* x, const T* weight, co
                      g.OH * g.OW, g.W, +1, g.C * taps, taps, stream))
       return;
     ops.wp = plan.weights; ops.steps = plan.steps; ops.K = plan.K;
-    launch_igemm(ops, stream);
+    launch_igemm(ops, plan.pieces, stream);
   }
   MOBULA_HIP_TRY(hipGetLastError());
 }
@@ -234,7 +283,7 @@ MOBULA_KERNEL conv2d_backward_data_kernel(const int n, const T* dy, const T* wei
                      static_cast<long long>(g.D) * g.OH * g.OW, g.H * g.W, g.OW, -1, taps, g.C * taps, stream))
       return;
     ops.wp = plan.weights; ops.steps = plan.steps; ops.K = plan.K;
-    launch_igemm(ops, stream);
+    launch_igemm(ops, plan.pieces, stream);
   }
   MOBULA_HIP_TRY(hipGetLastError());
 }
