@@ -22,7 +22,7 @@
 namespace roialign {
 
 struct BwdBlocked {
-  static constexpr int TH = 2;           // rows of a band = wavefronts of a workgroup
+  static constexpr int TH = 1;           // rows of a band = wavefronts of a workgroup
   static constexpr int BANDS = kTileRows / TH;   // bands per tile
   static constexpr int TW = 56;          // tile columns
   static constexpr int CB = 32;          // channels per workgroup
@@ -171,13 +171,16 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
     // a lane whose pooled column or channels do not exist loads from outside the buffer (zero, no access)
     const int dy_lane = pwb + grp < PW && quad * 4 < nch ? static_cast<int>(grp * dy_pw) + quad * 16
                                                          : static_cast<int>(0x80000000u);
-    const int list_lane = grp * 16;
-    auto issue = [&](const int16v& e, u32x4 (&d)[K::G], u32x4 (&u)[K::G]) {
+    // The 16-byte column sample of the lane's pooled column comes as one dword per
+    // lane (lane & 3 picks it; a 4-byte load costs the texture path half of a
+    // 16-byte one) and is spread over the quad with DPP moves where it is used.
+    const int list_lane = grp * 16 + (lane & 3) * 4;
+    auto issue = [&](const int16v& e, u32x4 (&d)[K::G], unsigned (&u)[K::G]) {
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
         const unsigned roi = e[4 * j], ph = e[4 * j + 1];
         d[j] = __builtin_amdgcn_raw_buffer_load_b128(dy_buf, dy_lane, roi * dy_roi + ph * dy_ph + dy_fixed, 0);
-        u[j] = __builtin_amdgcn_raw_buffer_load_b128(list_buf, list_lane, roi * list_roi + list_fixed, 0);
+        u[j] = __builtin_amdgcn_raw_buffer_load_b32(list_buf, list_lane, roi * list_roi + list_fixed, 0);
       }
     };
     float g[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -193,7 +196,7 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
       *reinterpret_cast<float4*>(a) = lo;
       *reinterpret_cast<float4*>(a + K::CS) = hi;
     };
-    auto process = [&](const int16v& e, const u32x4 (&d)[K::G], const u32x4 (&u)[K::G]) {
+    auto process = [&](const int16v& e, const u32x4 (&d)[K::G], const unsigned (&u)[K::G]) {
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
         const float wy = __int_as_float(e[4 * j + 2]);
@@ -203,9 +206,13 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
         for (int i = 0; i < 4; ++i) g[i] = fmaf(__uint_as_float(d[j][i]), wy, keep * g[i]);
         if ((fl & 2) != 0) {
           // last tap of this ROI on this row: spread g over the column samples
-          const int cf = u[j][1];
-          const int pos0 = u[j][0] & 0xffff, pos1 = u[j][0] >> 16;
-          const float l0 = __uint_as_float(u[j][2]), l1 = __uint_as_float(u[j][3]);
+          // dword k of the quad's four: quad_perm [k, k, k, k]
+          const int uj = static_cast<int>(u[j]);
+          const unsigned cells = static_cast<unsigned>(__builtin_amdgcn_mov_dpp(uj, 0x00, 0xf, 0xf, true));
+          const int cf = __builtin_amdgcn_mov_dpp(uj, 0x55, 0xf, 0xf, true);
+          const int pos0 = cells & 0xffff, pos1 = cells >> 16;
+          const float l0 = __int_as_float(__builtin_amdgcn_mov_dpp(uj, 0xaa, 0xf, 0xf, true));
+          const float l1 = __int_as_float(__builtin_amdgcn_mov_dpp(uj, 0xff, 0xf, 0xf, true));
           const int turns = 1 << ((__builtin_amdgcn_readfirstlane(cf) >> kColStrideShift) & kColStrideMask);
           auto add_both = [&] {
             if ((cf & 3) != 0) add_sample(pos0, (cf & 1) ? 1.0f - l0 : 0.0f, (cf & 2) ? l0 : 0.0f);
@@ -223,7 +230,8 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
 
     if (n_entries > 0) {
       int16v e_cur = wl[0], e_nx = wl[1], e_n2;
-      u32x4 d_a[K::G], d_b[K::G], u_a[K::G], u_b[K::G];
+      u32x4 d_a[K::G], d_b[K::G];
+      unsigned u_a[K::G], u_b[K::G];
       issue(e_cur, d_a, u_a);
       for (int e0 = 0; e0 < n_entries; e0 += 2 * K::G) {
         // group at e0 lives in set a, group at e0 + G in set b
