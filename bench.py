@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # absent entries are reported as null.
 MEASURED_TRAFFIC = {
     ('cfg2', 'forward_blocked_kernel'): 473.4e6,    # 272.7 MB read + 200.7 MB written
-    ('cfg2', 'backward_blocked_kernel'): 573.3e6,   # 274.9 MB read + 298.4 MB written
+    ('cfg2', 'backward_blocked_kernel'): 575.7e6,   # 277.1 MB read + 298.6 MB written
 }
 
 
