@@ -1,13 +1,14 @@
 // Backward ROIAlign: tile owners accumulate in LDS, 16 bytes per lane.
 //
 // dx is cut into tiles of 16 rows x 56 columns x 32 channels, and a tile into
-// bands of TH rows.  One workgroup owns one band, keeps it in LDS as
-// acc[row][column][channel] and is the only writer of that piece of dx: no
-// atomics anywhere and a summation order fixed by the ROI order.  Wavefront w
-// owns row w of the band, so the wavefronts never touch the same cell and need
-// no barrier; nothing but the launch ties the wavefronts of a workgroup
-// together, and small bands (several workgroups resident per CU) keep a CU
-// busy when the rows of a tile have work lists of different length.  The 64 lanes of a wavefront
+// bands of TH rows (TH = 1: single rows).  One workgroup owns one band, keeps
+// it in LDS as acc[row][column][channel] and is the only writer of that piece
+// of dx: no atomics anywhere and a summation order fixed by the ROI order.
+// Wavefront w owns row w of the band, so wavefronts never touch the same cell
+// and need no barrier.  Nothing but the launch ties the wavefronts of a
+// workgroup together, so small bands (many workgroups resident per CU) keep a
+// CU busy when the rows of a tile have work lists of different length.
+// The 64 lanes of a wavefront
 // are 8 pooled columns x 8 channel quads: a lane folds the row taps of a ROI
 // into four gradients (its pooled column, its four channels) and adds them to
 // the two cells of each of its column samples with 16-byte LDS accesses.
