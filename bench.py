@@ -303,6 +303,8 @@ def main():
                      'algorithmic_bytes': dom_bytes, 'avg_ms': dom_ms},
         'kernels_ms': kernel_ms,
         'passes': passes,
+        # share of the map inside some ROI's box: the e*|x| term of the algorithmic bytes counts all of it
+        'touched_fraction': workloads.touched_fraction(w),
     }
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(w)

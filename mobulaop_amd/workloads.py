@@ -8,7 +8,7 @@ Each generator returns a dict with NumPy arrays `data` (NCHW), `rois`
 """
 import numpy as np
 
-__all__ = ['WORKLOADS', 'make_workload', 'algorithmic_bytes']
+__all__ = ['WORKLOADS', 'make_workload', 'algorithmic_bytes', 'touched_fraction']
 
 
 def _pack(data, rois, pooled, scale, ratio, rng, name, dy=True):
@@ -122,3 +122,23 @@ def algorithmic_bytes(w):
     ny = R * C * w['pooled_size'][0] * w['pooled_size'][1]
     b = e * nx + 20 * R + e * ny
     return b, b
+
+
+def touched_fraction(w):
+    """Fraction of the map's pixels (one pixel of a channel block = one 128-byte
+    line of the blocked layout) inside the box of at least one ROI: what part of
+    the e*|x| term of the algorithmic bytes the ROIs can actually reach."""
+    N, _, H, W = w['data'].shape
+    hit = np.zeros((N, H, W), dtype=bool)
+    s = w['spatial_scale']
+    for b, x1, y1, x2, y2 in w['rois']:
+        b = int(b)
+        if b < 0 or b >= N:
+            continue
+        xa, ya = x1 * s, y1 * s
+        xb, yb = xa + max(x2 * s - xa, 1.0), ya + max(y2 * s - ya, 1.0)
+        c0, c1 = int(np.floor(max(xa, 0.0))), int(np.floor(min(xb, W - 1))) + 1
+        r0, r1 = int(np.floor(max(ya, 0.0))), int(np.floor(min(yb, H - 1))) + 1
+        if c0 < W and r0 < H and c1 >= 0 and r1 >= 0:
+            hit[b, max(r0, 0):min(r1 + 1, H), max(c0, 0):min(c1 + 1, W)] = True
+    return float(hit.mean())
