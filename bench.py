@@ -255,6 +255,30 @@ def main():
     native.set_option('kernel_timing', 0)
     kernel_ms = {k: sum(v) / len(v) for k, v in kernel_ms.items()}
 
+    # End to end through the operator: mobula.op.ROIAlign on torch tensors with autograd
+    # (allocation of y and dx, Python binding, the same kernels), wall clock per step.
+    op_ms = None
+    if has_bwd and w['data'].dtype.itemsize == 4:
+        import mobulaop_amd as mobula
+        mobula.op.load('ROIAlign')
+        x_op = (x.permute(0, 3, 1, 2) if nhwc else x).detach().requires_grad_(True)
+        dy_op = dy.permute(0, 3, 1, 2) if nhwc else dy
+        kw = dict(pooled_size=pooled, spatial_scale=scale, sampling_ratio=S)
+
+        def op_step():
+            y_op = mobula.op.ROIAlign(x_op, rois, **kw)
+            y_op.backward(dy_op)
+            x_op.grad = None
+
+        for _ in range(args.warmup):
+            op_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            op_step()
+        torch.cuda.synchronize()
+        op_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
     fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
     bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps if has_bwd else 0.0
     ms_per_step = wall * 1e3 / args.steps
@@ -306,6 +330,8 @@ def main():
         # share of the map inside some ROI's box: the e*|x| term of the algorithmic bytes counts all of it
         'touched_fraction': workloads.touched_fraction(w),
     }
+    if op_ms is not None:
+        out['passes']['operator_fwd_bwd'] = {'ms': op_ms, 'rois_per_s': R / (op_ms * 1e-3)}
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(w)
     print(json.dumps(out))
