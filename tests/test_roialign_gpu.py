@@ -289,6 +289,13 @@ def test_full_size_properties(cfg):
     print('{}: backward run-to-run max abs diff {:.3e} (max |dx| {:.3e})'.format(
         cfg, diff, float(dx.abs().max())), flush=True)
     assert diff <= BWD_TOL * float(dx.abs().max())
+    # (7) channels-last tensors at full size: the same numbers as the NCHW entry points
+    y_l = abi.forward_nhwc(x.permute(0, 2, 3, 1).contiguous(), rois, pooled, scale, S)
+    assert_parity(y_l.permute(0, 3, 1, 2).cpu().numpy(), y.cpu().numpy(), FWD_TOL, cfg + ' fwd channels-last')
+    del y_l
+    dx_l = abi.backward_nhwc(dy.permute(0, 2, 3, 1).contiguous(), rois,
+                             (x.shape[0], x.shape[2], x.shape[3], x.shape[1]), scale, S, assign=True)
+    assert_parity(dx_l.permute(0, 3, 1, 2).cpu().numpy(), dx.cpu().numpy(), BWD_TOL, cfg + ' bwd channels-last')
 
 
 def test_fp16_full_size_subset():
