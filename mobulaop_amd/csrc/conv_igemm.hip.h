@@ -105,6 +105,7 @@ struct ForwardOps {
   typedef GatherStep Step;
   struct BCtx { __amdgpu_buffer_rsrc_t src; int anchor; int ih0, iw0; bool ok; };
   __device__ Step load_step(int s) const { return steps[s]; }
+  __device__ Step next_step(const Step&, int s) const { return steps[s]; }
   __device__ void fetch_a(int m, const Step&, int s, int ak, float (&out)[8]) const {
     const float4* p = reinterpret_cast<const float4*>(wp + static_cast<size_t>(m) * K + s * Tile::BK + ak);
     const float4 lo = p[0], hi = p[1];
@@ -151,6 +152,7 @@ struct BackwardDataOps {
   typedef GatherStep Step;
   struct BCtx { __amdgpu_buffer_rsrc_t src; int anchor; int ihp, iwp; bool ok; };
   __device__ Step load_step(int s) const { return steps[s]; }
+  __device__ Step next_step(const Step&, int s) const { return steps[s]; }
   __device__ void fetch_a(int m, const Step&, int s, int ak, float (&out)[8]) const {
     const float4* p = reinterpret_cast<const float4*>(wp + static_cast<size_t>(m) * K + s * Tile::BK + ak);
     const float4 lo = p[0], hi = p[1];
@@ -217,11 +219,19 @@ struct BackwardWeightOps {
   const Tap* __restrict__ taps;   // taps over x
   Geometry g; int M, Ncols, K;   // K = length of this slice
   int k_begin;                   // first k of this slice
-  struct Step { int img, r, left; };   // image and pixel of the step's first k; k left in the slice
+  // image, pixel (flat and as row / column) of the step's first k; k left in the slice
+  struct Step { int img, r, left, oh, ow; };
   struct BCtx { int off; int dh, dw; bool ok; };
   __device__ Step load_step(int s) const {
-    const int ohw = g.OH * g.OW, k = k_begin + s * Tile::BK, img = k / ohw;
-    return Step{img, k - img * ohw, K - s * Tile::BK};
+    const int ohw = g.OH * g.OW, k = k_begin + s * Tile::BK, img = k / ohw, r = k - img * ohw, oh = r / g.OW;
+    return Step{img, r, K - s * Tile::BK, oh, r - oh * g.OW};
+  }
+  // the step after e: sixteen pixels on, without the divisions
+  __device__ Step next_step(const Step& e, int) const {
+    Step n{e.img, e.r + Tile::BK, e.left - Tile::BK, e.oh, e.ow + Tile::BK};
+    while (n.ow >= g.OW) { n.ow -= g.OW; ++n.oh; }
+    while (n.oh >= g.OH) { n.oh -= g.OH; ++n.img; n.r -= g.OH * g.OW; }
+    return n;
   }
   __device__ void fetch_a(int m, const Step& e, int, int ak, float (&out)[8]) const {
     const int ohw = g.OH * g.OW;
@@ -249,9 +259,9 @@ struct BackwardWeightOps {
   }
   __device__ void fetch_b(const BCtx& c, const Step& e, int bk, float (&out)[8]) const {
     const int ohw = g.OH * g.OW, image = g.C * g.H * g.W;
-    int img = e.img, r = e.r + bk;   // scalar: the step and bk are uniform
-    if (r >= ohw) { r -= ohw; ++img; }
-    const int oh0 = r / g.OW, ow0 = r - oh0 * g.OW;
+    int img = e.img, r = e.r + bk, oh0 = e.oh, ow0 = e.ow + bk;   // scalar: the step and bk are uniform
+    while (ow0 >= g.OW) { ow0 -= g.OW; ++oh0; }
+    if (r >= ohw) { r -= ohw; oh0 -= g.OH; ++img; }
     if (g.stride_w == 1 && ow0 + 8 <= g.OW && bk + 8 <= e.left) {
       // eight pixels of one output row: one row check, loads from one address
       const __amdgpu_buffer_rsrc_t src = buffer_of(x + static_cast<size_t>(img) * image, image * 4u);
@@ -358,10 +368,10 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0, int s
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   float ra[8], rb[8];
+  typename Ops::Step step = ops.load_step(s_begin);
   auto fetch = [&](int s) {
-    const typename Ops::Step e = ops.load_step(s);
-    ops.fetch_a(m0 + a_m, e, s, a_k, ra);
-    ops.fetch_b(bctx, e, b_k, rb);
+    ops.fetch_a(m0 + a_m, step, s, a_k, ra);
+    ops.fetch_b(bctx, step, b_k, rb);
   };
   auto stage = [&](int buf) {
     if (BF16) {
@@ -400,7 +410,10 @@ __device__ __forceinline__ void igemm_tile(const Ops& ops, int m0, int n0, int s
   __syncthreads();
   for (int s = s_begin; s < steps; ++s) {
     const int buf = (s - s_begin) & 1;
-    if (s + 1 < steps) fetch(s + 1);
+    if (s + 1 < steps) {
+      step = ops.next_step(step, s + 1);
+      fetch(s + 1);
+    }
     if (BF16) {
       bf16x8 a[PARTS][2], b[PARTS][2];
 #pragma unroll
