@@ -77,6 +77,21 @@ void roi_align_forward_e874c59a(const int device_id, const int nthreads,
                                 const int sampling_ratio, const float* bottom_rois,
                                 unsigned short* top_data);
 
+/* Backward with binary16 top_diff / bottom_diff (fp32 rois; sums are formed in
+ * fp32 and rounded once per element).  The reference has float atomics only
+ * (context/cpu_ctx.h:37-62), hence no counterpart. */
+void roi_align_backward_23175303(const int device_id, const int nthreads, const unsigned short* top_diff,
+                                 const float spatial_scale, const int channels, const int height,
+                                 const int width, const int pooled_height, const int pooled_width,
+                                 const int sampling_ratio, unsigned short* bottom_diff,
+                                 const float* bottom_rois);
+void roi_align_backward_assign_7924dbc8(const int device_id, const int nthreads,
+                                        const unsigned short* top_diff, const float spatial_scale,
+                                        const int channels, const int height, const int width,
+                                        const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        unsigned short* bottom_diff, const float* bottom_rois);
+
 /* The three operations on channels-last tensors: the map as [N,H,W,C], the pooled
  * tensor as [R,PH,PW,C] (what a torch tensor in torch.channels_last format holds);
  * scalar arguments as above (channels, height, width name C, H, W).  No

@@ -18,6 +18,8 @@
 // dy is read from a channel-blocked copy dyb[R][C/32][PH][PWp][32] (PWp = PW
 // rounded up to 8): one 16-byte load per lane fetches a pooled row (1 KB).
 #pragma once
+#include <type_traits>
+
 #include "roialign_taps.hip.h"
 
 namespace roialign {
@@ -41,23 +43,27 @@ inline bool backward_blocked_supports(int PH, int PW, int S) { return lists_supp
 // does not exist.  One workgroup per (ROI, group of `per` channel blocks):
 // the input words of the group are contiguous and so are its output words.
 // LDS holds the input as it is; the transposition happens in the reads.
+// T is the element type of dy (float or __half); dyb is fp32 either way.
+template <typename T>
 __global__ void __launch_bounds__(256)
-transpose_dy_blocked_kernel(const float* __restrict__ dy, float* __restrict__ dyb, int C, int PH,
+transpose_dy_blocked_kernel(const T* __restrict__ dy, float* __restrict__ dyb, int C, int PH,
                             int PW, int PWp, int cblk, int per) {
   constexpr int CB = BwdBlocked::CB;
-  extern __shared__ __attribute__((aligned(16))) float tbuf[];   // [per * 32][PH * PW]
+  constexpr int VEC = 16 / sizeof(T);   // elements per 16-byte word
+  extern __shared__ __attribute__((aligned(16))) unsigned char tbuf_bytes[];   // [per * 32][PH * PW] of T
+  T* const tbuf = reinterpret_cast<T*>(tbuf_bytes);
   const int groups = (cblk + per - 1) / per;
   const int r = blockIdx.x / groups, grp = blockIdx.x % groups;
   const int cb0 = grp * per, nblk = min(per, cblk - cb0);
   const int c0 = cb0 * CB, nch = min(nblk * CB, C - c0);
   const int bins = PH * PW;
-  const float* src = dy + (static_cast<size_t>(r) * C + c0) * bins;
+  const T* src = dy + (static_cast<size_t>(r) * C + c0) * bins;
   const int n_in = nch * bins;
   if ((reinterpret_cast<size_t>(src) & 15) == 0) {
-    const int nvec = n_in >> 2;
+    const int nvec = n_in / VEC;
     for (int i = threadIdx.x; i < nvec; i += 256)
       reinterpret_cast<float4*>(tbuf)[i] = reinterpret_cast<const float4*>(src)[i];
-    for (int i = 4 * nvec + threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
+    for (int i = VEC * nvec + threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
   } else {
     for (int i = threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
   }
@@ -70,11 +76,11 @@ transpose_dy_blocked_kernel(const float* __restrict__ dy, float* __restrict__ dy
     float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     if (pw < PW) {
       const int c = blk * CB + 4 * cq;
-      const float* in = tbuf + c * bins + ph * PW + pw;
-      if (c + 0 < nch) v.x = in[0];
-      if (c + 1 < nch) v.y = in[bins];
-      if (c + 2 < nch) v.z = in[2 * bins];
-      if (c + 3 < nch) v.w = in[3 * bins];
+      const T* in = tbuf + c * bins + ph * PW + pw;
+      if (c + 0 < nch) v.x = to_float(in[0]);
+      if (c + 1 < nch) v.y = to_float(in[bins]);
+      if (c + 2 < nch) v.z = to_float(in[2 * bins]);
+      if (c + 3 < nch) v.w = to_float(in[3 * bins]);
     }
     *reinterpret_cast<float4*>(dst + static_cast<size_t>(q) * 4) = v;
   }
@@ -92,9 +98,11 @@ inline long long backward_blocked_grid(long long tiles, int cblk) {
 
 typedef int int16v __attribute__((ext_vector_type(16)));
 
-template <bool NHWC>
+// TO is the element type of dx (float or __half; sums are formed in fp32 and
+// rounded once); channels-last tensors are fp32 only.
+template <bool NHWC, typename TO>
 __global__ void __launch_bounds__(BwdBlocked::NT)
-backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
+backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
                         const WorkRange* __restrict__ ranges, const WorkEntry* __restrict__ entries,
                         const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll, int C, int H,
                         int W, int PH, int PW, int cblk, unsigned dyb_bytes, unsigned list_bytes,
@@ -248,7 +256,8 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
     }
   }
 
-  if (NHWC) {
+  if (NHWC && std::is_same<TO, float>::value) {
+    float* const dx = reinterpret_cast<float*>(dx_any);
     // dx[n][row][col][C]: a pixel's channels of this block are 128 contiguous bytes;
     // eight pixels per step, a lane moves its four channels
     float* const px0 = dx + ((static_cast<size_t>(n) * H + r0 + wave) * W + q0) * C + c0 + quad * 4;
@@ -268,14 +277,15 @@ backward_blocked_kernel(const float* __restrict__ dyb, float* __restrict__ dx,
     return;
   }
   // The owner writes its row: one channel plane at a time, lanes along x.
-  float* const out = dx + ((static_cast<size_t>(n) * C + c0) * H + r0 + wave) * W + q0;
+  TO* const out = dx_any + ((static_cast<size_t>(n) * C + c0) * H + r0 + wave) * W + q0;
   const size_t plane = static_cast<size_t>(H) * W;
   if (lane < cols) {
     const float* const src = row + (lane + 1) * K::CS;
     if (assign) {
-      for (int c = 0; c < nch; ++c) out[c * plane + lane] = src[c];
+      for (int c = 0; c < nch; ++c) out[c * plane + lane] = from_float<TO>(src[c]);
     } else {
-      for (int c = 0; c < nch; ++c) out[c * plane + lane] += src[c];
+      for (int c = 0; c < nch; ++c)
+        out[c * plane + lane] = from_float<TO>(to_float(out[c * plane + lane]) + src[c]);
     }
   }
 }

@@ -46,8 +46,10 @@ forward_naive_kernel(long long n_out, const T* __restrict__ x, float scale, int 
   }
 }
 
+// TI: element type of dy; the sums go into an fp32 map.
+template <typename TI>
 __global__ void __launch_bounds__(256)
-backward_naive_kernel(long long n_out, const float* __restrict__ dy, float scale, int C, int H,
+backward_naive_kernel(long long n_out, const TI* __restrict__ dy, float scale, int C, int H,
                       int W, int PH, int PW, int S, float* __restrict__ dx,
                       const float* __restrict__ rois, long long num_images) {
   const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
@@ -61,7 +63,7 @@ backward_naive_kernel(long long n_out, const float* __restrict__ dy, float scale
     const RoiGeom g = roi_geometry(rois + r * 5, scale, PH, PW, S);
     if (g.batch < 0 || g.batch >= num_images) continue;
     float* plane = dx + (static_cast<long long>(g.batch) * C + c) * H * W;
-    const float top = dy[idx];
+    const float top = to_float(dy[idx]);
     for (int iy = 0; iy < g.grid_h; ++iy) {
       const AxisSample sy = axis_sample(sample_coord(g.start_h, ph, g.bin_h, iy, g.grid_h), H);
       if (!sy.valid) continue;
@@ -94,6 +96,21 @@ __global__ void __launch_bounds__(256)
 zero_words_kernel(unsigned* __restrict__ p, long long n) {
   const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
   for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0u;
+}
+
+// out[i] = in[i] (widened), and the way back, for the fp16 detour of the
+// straightforward backward kernel.
+__global__ void __launch_bounds__(256)
+widen_kernel(const __half* __restrict__ in, float* __restrict__ out, long long n) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
+    out[i] = __half2float(in[i]);
+}
+__global__ void __launch_bounds__(256)
+narrow_kernel(const float* __restrict__ in, __half* __restrict__ out, long long n) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
+    out[i] = __float2half_rn(in[i]);
 }
 
 }  // namespace roialign

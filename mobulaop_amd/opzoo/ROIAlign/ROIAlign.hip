@@ -265,29 +265,32 @@ bool nhwc_backward_supported(const Problem& p) {
          static_cast<long long>(p.R) * p.PH * p.PW * p.C * 4 < (1ll << 31);
 }
 
-void backward_device(const Problem& p, const float* dy, const float* rois, float* dx, bool assign,
+template <typename T>
+void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bool assign,
                      hipStream_t stream) {
   if (p.N <= 0) return;
   using BB = roialign::BwdBlocked;
+  constexpr bool kFp32 = std::is_same<T, float>::value;
   TilePlan plan;
   if (p.nhwc) {
     // dy and dx are used where they lie: only the pre-pass before the tile owners
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
-    if (!nhwc_backward_supported(p) || reinterpret_cast<size_t>(dy) % 16 != 0 ||
+    if (!kFp32 || !nhwc_backward_supported(p) || reinterpret_cast<size_t>(dy) % 16 != 0 ||
         reinterpret_cast<size_t>(dx) % 16 != 0 ||
         !plan_tiles(p, rois, roialign::kTileRows, BB::TW, /*with_dyb=*/false, stream, &plan) ||
         roialign::backward_blocked_grid(plan.grid.total, cblk) >= (1ll << 31)) {
       if (!failed())
-        set_error("roi_align_backward_nhwc: shape C=%d pooled %dx%d sampling_ratio %d (or the alignment of the "
-                  "tensors) is not taken by the channels-last path", p.C, p.PH, p.PW, p.S);
+        set_error("roi_align_backward_nhwc: shape C=%d pooled %dx%d sampling_ratio %d (or the type or alignment "
+                  "of the tensors) is not taken by the channels-last path", p.C, p.PH, p.PW, p.S);
       return;
     }
     const unsigned dy_bytes = static_cast<unsigned>(sizeof(float) * p.n_out);
     mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-    roialign::backward_blocked_kernel<true><<<static_cast<unsigned>(
+    roialign::backward_blocked_kernel<true, float><<<static_cast<unsigned>(
         roialign::backward_blocked_grid(plan.grid.total, cblk)), BB::NT, 0, stream>>>(
-        dy, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H, p.W, p.PH, p.PW,
-        cblk, dy_bytes, static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
+        reinterpret_cast<const float*>(dy), reinterpret_cast<float*>(dx), plan.ranges, plan.entries, plan.lists,
+        plan.grid, plan.layout, p.C, p.H, p.W, p.PH, p.PW, cblk, dy_bytes,
+        static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
     MOBULA_HIP_TRY(hipGetLastError());
     return;
   }
@@ -298,19 +301,19 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
     // channel blocks per workgroup of the dy transposition: what 64 KB of LDS hold, at most 4
-    const size_t dy_blk_bytes = sizeof(float) * BB::CB * p.PH * p.PW;
+    const size_t dy_blk_bytes = sizeof(T) * BB::CB * p.PH * p.PW;
     const int dy_per = static_cast<int>(std::min<size_t>(4, (64 * 1024) / dy_blk_bytes));
     const long long dy_blocks = dy_per > 0 ? static_cast<long long>(p.R) * ((cblk + dy_per - 1) / dy_per) : 0;
     if (grid < (1ll << 31) && dy_blocks < (1ll << 31) && dy_per > 0) {
       const int pwp = plan.layout.col_stride;
       if (p.R > 0)
-        roialign::transpose_dy_blocked_kernel<<<static_cast<unsigned>(dy_blocks), 256,
-                                                dy_per * dy_blk_bytes, stream>>>(
+        roialign::transpose_dy_blocked_kernel<T><<<static_cast<unsigned>(dy_blocks), 256,
+                                                   dy_per * dy_blk_bytes, stream>>>(
             dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dy_per);
       side.join();
       {
         mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-        roialign::backward_blocked_kernel<false><<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
+        roialign::backward_blocked_kernel<false, T><<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
             plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
             p.W, p.PH, p.PW, cblk, static_cast<unsigned>(plan.dyb_bytes),
             static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
@@ -321,12 +324,22 @@ void backward_device(const Problem& p, const float* dy, const float* rois, float
   }
   side.join();
   if (failed()) return;
+  // straightforward kernel: float atomics into an fp32 map (the caller's, or for fp16 a scratch copy)
+  const long long map = static_cast<long long>(p.N) * p.C * p.H * p.W;
+  float* sums = reinterpret_cast<float*>(dx);
+  if (!kFp32) {
+    sums = static_cast<float*>(mobula_hip::workspace(sizeof(float) * map));
+    if (failed()) return;
+    if (!assign)
+      roialign::widen_kernel<<<grid_for(map, 256), 256, 0, stream>>>(reinterpret_cast<const __half*>(dx), sums, map);
+  }
   if (assign)
-    roialign::zero_words_kernel<<<grid_for(static_cast<long long>(p.N) * p.C * p.H * p.W, 256), 256, 0, stream>>>(
-        reinterpret_cast<unsigned*>(dx), static_cast<long long>(p.N) * p.C * p.H * p.W);
-  if (p.n_out == 0) return;
-  roialign::backward_naive_kernel<<<grid_for(p.n_out, 256), 256, 0, stream>>>(
-      p.n_out, dy, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, dx, rois, p.N);
+    roialign::zero_words_kernel<<<grid_for(map, 256), 256, 0, stream>>>(reinterpret_cast<unsigned*>(sums), map);
+  if (p.n_out > 0)
+    roialign::backward_naive_kernel<T><<<grid_for(p.n_out, 256), 256, 0, stream>>>(
+        p.n_out, dy, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, sums, rois, p.N);
+  if (!kFp32)
+    roialign::narrow_kernel<<<grid_for(map, 256), 256, 0, stream>>>(sums, reinterpret_cast<__half*>(dx), map);
   MOBULA_HIP_TRY(hipGetLastError());
 }
 
@@ -581,6 +594,28 @@ void roi_align_backward_assign_a8793cbe(const int device_id, const int nthreads,
                         bottom_rois);
 }
 
+// Backward with binary16 top_diff / bottom_diff (sums in fp32, rounded once).
+void roi_align_backward_23175303(const int device_id, const int nthreads, const __half* top_diff,
+                                 const float spatial_scale, const int channels, const int height,
+                                 const int width, const int pooled_height, const int pooled_width,
+                                 const int sampling_ratio, __half* bottom_diff, const float* bottom_rois) {
+  backward_entry<__half>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+                         pooled_height, pooled_width, sampling_ratio, -1, bottom_diff, bottom_rois);
+}
+
+void roi_align_backward_assign_7924dbc8(const int device_id, const int nthreads, const __half* top_diff,
+                                        const float spatial_scale, const int channels, const int height,
+                                        const int width, const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        __half* bottom_diff, const float* bottom_rois) {
+  if (num_images < 0) {
+    set_error("roi_align_backward_assign: num_images=%d", num_images);
+    return;
+  }
+  backward_entry<__half>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+                         pooled_height, pooled_width, sampling_ratio, num_images, bottom_diff, bottom_rois);
+}
+
 // Channels-last variants (extensions): device pointers only.
 #define MOBULA_NHWC_ENTRY(call)                                                            \
   if (device_id < 0) {                                                                     \
@@ -662,6 +697,7 @@ void roi_align_forward_e874c59a(const int device_id, const int nthreads, const _
 
 static mobula_hip::ExportRegistrar roialign_exports(
     "roi_align_forward_ab78de3c roi_align_backward_f318a24e roi_align_backward_assign_a8793cbe "
-    "roi_align_forward_e874c59a roi_align_forward_nhwc_ab78de3c roi_align_forward_nhwc_e874c59a "
+    "roi_align_forward_e874c59a roi_align_backward_23175303 roi_align_backward_assign_7924dbc8 "
+    "roi_align_forward_nhwc_ab78de3c roi_align_forward_nhwc_e874c59a "
     "roi_align_backward_nhwc_f318a24e roi_align_backward_nhwc_assign_a8793cbe "
     "mobula_hip_roialign_nhwc_supported");

@@ -61,16 +61,17 @@ def backward(dy, rois, shape, scale, S, dx=None, assign=False, declare_extents=T
         dx = (torch.full(shape, float('nan'), dtype=dy.dtype, device=dy.device) if assign
               else torch.zeros(shape, dtype=dy.dtype, device=dy.device))
     lib = native.library()
+    half = dy.dtype == torch.float16
     if assign:
         ext = [-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()]
         _begin(ext if declare_extents else [], stream)
-        lib.roi_align_backward_assign_a8793cbe(
+        (lib.roi_align_backward_assign_7924dbc8 if half else lib.roi_align_backward_assign_a8793cbe)(
             ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
             ctypes.c_int(N), _ptr(dx), _ptr(rois))
     else:
         ext = [-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()]
         _begin(ext if declare_extents else [], stream)
-        lib.roi_align_backward_f318a24e(
+        (lib.roi_align_backward_23175303 if half else lib.roi_align_backward_f318a24e)(
             ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
             _ptr(dx), _ptr(rois))
     _end(lib)

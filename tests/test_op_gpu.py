@@ -149,3 +149,23 @@ def test_channels_last_tensors_take_the_channels_last_path(mobula):
     assert xb.grad.is_contiguous(memory_format=torch.channels_last)
     assert float((ya - yb).detach().abs().max()) <= 1e-5 * float(ya.detach().abs().max())
     assert float((xa.grad - xb.grad).abs().max()) <= 1e-4 * float(xa.grad.abs().max())
+
+
+def test_half_precision_training_step(mobula):
+    # fp16 map and gradients through the operator: both passes run in the library
+    torch.manual_seed(6)
+    x32 = torch.randn(2, 64, 20, 24, device='cuda')
+    rois = torch.tensor([[0, 1, 2, 60, 50], [1, 10, 10, 90, 70], [1, -5, 3, 20, 100]], device='cuda',
+                        dtype=torch.float32)
+    kw = dict(pooled_size=(7, 7), spatial_scale=0.25, sampling_ratio=2)
+    xh = x32.half().requires_grad_(True)
+    yh = mobula.op.ROIAlign(xh, rois, **kw)
+    assert yh.dtype == torch.float16
+    dy = torch.randn_like(yh)
+    yh.backward(dy)
+    assert xh.grad.dtype == torch.float16
+    xf = x32.half().float().requires_grad_(True)
+    yf = mobula.op.ROIAlign(xf, rois, **kw)
+    yf.backward(dy.float())
+    assert float((yh.detach().float() - yf.detach()).abs().max()) <= 2e-3 * float(yf.detach().abs().max())
+    assert float((xh.grad.float() - xf.grad).abs().max()) <= 2e-3 * float(xf.grad.abs().max())

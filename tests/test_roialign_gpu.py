@@ -105,6 +105,28 @@ def test_fp16_channel_blocks(C, S):
     assert_parity(y.astype(np.float32), want.astype(np.float16).astype(np.float32), FP16_TOL, 'fp16')
 
 
+@pytest.mark.parametrize('S', [2, 0])
+@pytest.mark.parametrize('C', [72, 20])
+def test_fp16_backward(C, S):
+    # fp16 gradients: the checker's fp32 result on the fp16-rounded dy, rounded to fp16;
+    # S = 0 (and C = 20 in any case) goes through the straightforward kernel and an fp32 scratch map
+    abi.set_impl('auto')
+    rng = np.random.default_rng(300 * C + S)
+    N, H, W, R, pooled, scale = 2, 30, 44, 40, (7, 7), 0.25
+    dy16 = rng.standard_normal((R, C) + pooled).astype(np.float16)
+    c = np.stack([rng.uniform(0, W / scale, R), rng.uniform(0, H / scale, R)], 1)
+    wh = np.stack([rng.uniform(2, W / scale, R), rng.uniform(2, H / scale, R)], 1)
+    rois = np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+    want = oracle.backward(dy16.astype(np.float32), rois, (N, C, H, W), scale, S, impl='ordered')
+    dx = abi.backward(abi.to_dev(dy16), abi.to_dev(rois), (N, C, H, W), scale, S, assign=True)
+    assert dx.dtype == torch.float16
+    assert_parity(dx.cpu().numpy().astype(np.float32), want.astype(np.float16).astype(np.float32), FP16_TOL, 'assign')
+    base = rng.standard_normal((N, C, H, W)).astype(np.float16)
+    dx = abi.backward(abi.to_dev(dy16), abi.to_dev(rois), (N, C, H, W), scale, S, dx=abi.to_dev(base))
+    assert_parity(dx.cpu().numpy().astype(np.float32),
+                  (want + base.astype(np.float32)).astype(np.float16).astype(np.float32), FP16_TOL, 'accumulate')
+
+
 @pytest.mark.parametrize('impl', IMPLS)
 @pytest.mark.parametrize('shape', [
     # N, C, H, W, R, pooled, scale, S
