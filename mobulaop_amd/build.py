@@ -37,6 +37,8 @@ def hipcc_flags():
         '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
         '-Wall', '-Wno-unused-function', '-Wno-unknown-warning-option',
         '-I' + CSRC,
+        # modules compiled on load name the library by this, wherever the tree lies
+        '-Wl,-soname,libmobula_hip.so',
     ]
     if config.DEBUG:
         flags.append('-g')

@@ -120,6 +120,9 @@ class KernelTimer {
   } while (0)
 
 // Launcher functions are ordinary host functions; the macro only marks them
-// for the Python-side declaration scanner.
+// for the Python-side declaration scanner.  (Sources in the kernel dialect,
+// compiled on load, define the macros themselves before this header is seen.)
+#ifndef MOBULA_KERNEL
 #define MOBULA_KERNEL void
 #define MOBULA_FUNC
+#endif

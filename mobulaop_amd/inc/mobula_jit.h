@@ -1,0 +1,81 @@
+// Launch glue for operator sources compiled at load time (one small shared
+// object per function instantiation, see mobulaop_amd/op/jit.py).  A generated
+// entry point
+//     extern "C" void axpy_<hash>(const int device_id, const int n, ...)
+// creates a KernelCall, maps its pointer arguments (device pointers pass
+// through; host pointers, device id -1, are mirrored on the staging device using
+// the element counts the binding declared for the call) and launches the
+// kernel on the calling thread's stream.  Errors are recorded for the binding
+// to raise; nothing terminates the process.
+#pragma once
+#include <algorithm>
+#include <type_traits>
+
+#include "runtime.h"
+
+namespace mobula_jit {
+
+class KernelCall {
+ public:
+  KernelCall(const char* name, int device_id)
+      : name_(name), host_(device_id < 0),
+        scope_(device_id < 0 ? static_cast<int>(mobula_hip::option("host_staging_device", 0)) : device_id) {
+    auto& st = mobula_hip::call_state();
+    saved_stream_ = st.stream;
+    if (host_) st.stream = nullptr;   // the caller's stream belongs to another device, if to any
+  }
+  ~KernelCall() {
+    auto& st = mobula_hip::call_state();
+    if (host_) {
+      if (!mobula_hip::failed()) stage_.flush(nullptr);
+      st.stream = saved_stream_;
+      st.extents.clear();
+    } else {
+      mobula_hip::finish_call();
+    }
+  }
+  bool ok() const { return scope_.ok() && !mobula_hip::failed(); }
+
+  // Pointer argument number `index` (0-based, device id not counted) of
+  // elem_bytes-sized elements; writable ones are copied back for host callers.
+  template <typename T>
+  T* arg(T* p, int index, bool writable) {
+    if (!host_ || p == nullptr) return p;
+    const long long count = mobula_hip::arg_extent(index);
+    if (count < 0) {
+      mobula_hip::set_error("%s: host memory needs the element count of argument %d", name_, index);
+      return p;
+    }
+    typedef typename std::remove_const<T>::type M;
+    const size_t bytes = sizeof(T) * static_cast<size_t>(count);
+    void* dev = writable ? stage_.inout(const_cast<M*>(p), bytes, /*upload=*/true)
+                         : stage_.in(p, bytes);
+    return static_cast<T*>(dev);
+  }
+
+  // kernel<<<blocks of 256 threads for n iterations>>>(args...) on the call's stream.
+  template <typename Kernel, typename... Args>
+  void launch(long long n, Kernel kernel, Args... args) {
+    if (!ok() || n <= 0) return;
+    int cus = 0, device = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    const long long blocks = std::min<long long>((n + 255) / 256, static_cast<long long>(cus) * 8);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                       mobula_hip::call_state().stream, args...);
+    const hipError_t status = hipGetLastError();
+    if (status != hipSuccess) mobula_hip::set_error("%s: launch failed: %s", name_, hipGetErrorString(status));
+  }
+
+ private:
+  const char* name_;
+  bool host_;
+  mobula_hip::DeviceScope scope_;
+  mobula_hip::HostStaging stage_;
+  hipStream_t saved_stream_ = nullptr;
+};
+
+}  // namespace mobula_jit

@@ -7,9 +7,11 @@ declarations and binds one `mobula.func.<name>` per declaration, then executes
 the Python file (reference: mobula/op/loader.py:538-659 for the scan and load,
 :366-382 for symbol lookup).
 
-Unlike the reference there is no per-call JIT: every instantiation is compiled
-ahead of time into the launcher library, and resolving one that the library
-does not export raises NameError with the list of what it does export.
+The bundled operators (`.hip`: hand-written launchers) are compiled ahead of
+time into the launcher library; resolving an instantiation of theirs that the
+library does not export raises NameError with the list of what it does export.
+A `.cpp` source in MobulaOP's kernel dialect (MOBULA_KERNEL + parfor) is
+compiled on first use, one instantiation at a time (op/jit.py).
 """
 import ctypes
 import importlib.util
@@ -89,6 +91,11 @@ class OpLoader:
         if key not in _RESOLVED:
             sym_name = get_idcode_hash(idcode)
             fn = native.symbol(sym_name)
+            source = cpp_info.cpp_fname if cpp_info is not None else ''
+            if fn is None and source.endswith('.cpp'):
+                # an operator source in the kernel dialect: compiled on first use
+                from . import jit
+                fn = jit.resolve(cfunc, arg_types, source, sym_name)
             if fn is None:
                 raise NameError('No function `{}` (symbol {}) in {}, current functions: {}'.format(
                     idcode, sym_name, native.LIB_PATH, native.exported_names()))
