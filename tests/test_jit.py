@@ -46,6 +46,15 @@ def test_instantiations_compile_and_export_their_symbols(axpy_ops):
         path = jit.compile_instantiation(decl, types, decl.loader_kwargs['cpp_info'].cpp_fname, symbol)
         assert os.path.exists(path)
         assert hasattr(ctypes.CDLL(path), symbol)
+    # the other kernels of the source, as the GPU tests call them
+    f32p, i32p = ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int)
+    for name, types in (
+            ('weighted_histogram', _types((ctypes.c_int, True), (i32p, True), (f32p, True), (f32p, False))),
+            ('row_energy', _types((ctypes.c_int, True), (ctypes.c_int, True), (f32p, True), (f32p, False)))):
+        decl = getattr(axpy_ops, name).func
+        symbol = get_idcode_hash(get_func_idcode(name, types))
+        path = jit.compile_instantiation(decl, types, decl.loader_kwargs['cpp_info'].cpp_fname, symbol)
+        assert hasattr(ctypes.CDLL(path), symbol)
     assert axpy_ops.padded_length(13, 8) == 16      # MOBULA_FUNC: runs on the host
 
 
