@@ -184,6 +184,39 @@ def test_resnet_block_shape_properties(compute):
     assert abs(lhs - float((w.double() * dw.double()).sum())) <= bound
 
 
+def test_bf16_mode_is_exact_on_bf16_valued_operands():
+    # Mode 1 rounds both operands of every product to bf16 and accumulates in fp32: against
+    # the same products of the rounded operands in fp32 only the order of the sums differs,
+    # well inside the 1e-3 bound (the 1e-2 of the other tests is the rounding of the inputs)
+    N, C, H, W, D = 3, 64, 20, 20, 96
+    g = torch.Generator().manual_seed(61)
+    x = torch.randn(N, C, H, W, generator=g)
+    w = torch.randn(D, C, 3, 3, generator=g) * 0.1
+    dy = torch.randn(N, D, H, W, generator=g)
+    rnd = lambda t: t.bfloat16().float()
+    xr, wr = rnd(x).requires_grad_(True), rnd(w).requires_grad_(True)
+    F.conv2d(xr, wr, padding=1).backward(rnd(dy))
+    y_ref = F.conv2d(rnd(x), rnd(w), padding=1)
+    native.set_option('conv_compute', 1)
+    try:
+        xd, wd, dyd = x.cuda(), w.cuda(), dy.cuda()
+        geo = _ci(N, C, H, W, D, 3, 3, 1, 1, 1, 1, 1, 1)
+        y = torch.empty(N, D, H, W, device='cuda')
+        _call('conv2d_forward_c6a7aa85', ctypes.c_int(y.numel()), _ptr(xd), _ptr(wd), _ptr(wd), ctypes.c_int(0),
+              *geo, _ptr(y))
+        dx = torch.empty_like(xd)
+        _call('conv2d_backward_data_ecf81c91', ctypes.c_int(dx.numel()), _ptr(dyd), _ptr(wd), ctypes.c_int(0),
+              *geo, _ptr(dx))
+        dw = torch.empty_like(wd)
+        _call('conv2d_backward_weight_ecf81c91', ctypes.c_int(dw.numel()), _ptr(dyd), _ptr(xd), ctypes.c_int(0),
+              *geo, _ptr(dw))
+    finally:
+        native.set_option('conv_compute', 0)
+    _close(y, y_ref, 'y', 1e-4)
+    _close(dx, xr.grad, 'dx', 1e-4)
+    _close(dw, wr.grad, 'dw', 1e-4)
+
+
 def test_errors_surface_as_exceptions():
     x = torch.zeros(1, 1, 4, 4, device='cuda')
     w = torch.zeros(1, 1, 3, 3, device='cuda')
