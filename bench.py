@@ -279,6 +279,17 @@ def main():
         torch.cuda.synchronize()
         op_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # Backward twice from the same inputs: the largest difference between the two
+    # results (the reference's atomics give a different summation order each run).
+    repeat_diff = None
+    if has_bwd:
+        dx_again = torch.empty_like(dx)
+        run_backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream)
+        run_backward(dy, rois, x.shape, scale, S, dx=dx_again, assign=True, stream=stream)
+        torch.cuda.synchronize()
+        repeat_diff = float((dx.float() - dx_again.float()).abs().max())
+        del dx_again
+
     fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
     bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps if has_bwd else 0.0
     ms_per_step = wall * 1e3 / args.steps
@@ -329,7 +340,11 @@ def main():
         'passes': passes,
         # share of the map inside some ROI's box: the e*|x| term of the algorithmic bytes counts all of it
         'touched_fraction': workloads.touched_fraction(w),
+        # what a kernel with no reuse of corner values would move per forward pass
+        'gather_bytes': workloads.gather_bytes(w),
     }
+    if repeat_diff is not None:
+        out['backward_run_to_run_max_abs'] = repeat_diff
     if op_ms is not None:
         out['passes']['operator_fwd_bwd'] = {'ms': op_ms, 'rois_per_s': R / (op_ms * 1e-3)}
     if not args.no_cpu_baseline:

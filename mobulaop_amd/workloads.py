@@ -8,7 +8,7 @@ Each generator returns a dict with NumPy arrays `data` (NCHW), `rois`
 """
 import numpy as np
 
-__all__ = ['WORKLOADS', 'make_workload', 'algorithmic_bytes', 'touched_fraction']
+__all__ = ['WORKLOADS', 'make_workload', 'algorithmic_bytes', 'touched_fraction', 'gather_bytes']
 
 
 def _pack(data, rois, pooled, scale, ratio, rng, name, dy=True):
@@ -142,3 +142,22 @@ def touched_fraction(w):
         if c0 < W and r0 < H and c1 >= 0 and r1 >= 0:
             hit[b, max(r0, 0):min(r1 + 1, H), max(c0, 0):min(c1 + 1, W)] = True
     return float(hit.mean())
+
+
+def gather_bytes(w):
+    """Bytes a kernel without any reuse would pull through the caches in one
+    forward pass: four corner values for each sample of each output,
+    4 * e * S_h * S_w per output (the adaptive grid is ceil(roi/pooled) per ROI)."""
+    e = w['data'].dtype.itemsize
+    C = w['data'].shape[1]
+    PH, PW = w['pooled_size']
+    S = w['sampling_ratio']
+    rois = w['rois'].astype(np.float32)
+    if S > 0:
+        samples = np.full(rois.shape[0], S * S, dtype=np.int64)
+    else:
+        s = np.float32(w['spatial_scale'])
+        rw = np.maximum(rois[:, 3] * s - rois[:, 1] * s, np.float32(1))
+        rh = np.maximum(rois[:, 4] * s - rois[:, 2] * s, np.float32(1))
+        samples = (np.ceil(rh / np.float32(PH)) * np.ceil(rw / np.float32(PW))).astype(np.int64)
+    return int(4 * e * C * PH * PW * samples.sum())

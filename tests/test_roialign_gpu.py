@@ -63,6 +63,20 @@ def test_scaled_configs_against_oracle(impl, cfg, down):
     assert_parity(dx, want_dx, BWD_TOL, cfg + ' bwd assign')
 
 
+def test_tiled_backward_repeats_bit_for_bit():
+    """The tiled backward owns every dx element in one wavefront and adds in list
+    order (no float atomics), so two runs agree exactly; the reference's
+    atomics (ROIAlign.cpp:149-156) give a few ulp of run-to-run noise."""
+    abi.set_impl('tiled')
+    w = workloads.make_workload('cfg3', scale_down=16)   # heavy overlap, adversarial boxes
+    scale, S = w['spatial_scale'], w['sampling_ratio']
+    rois, dy = abi.to_dev(w['rois']), abi.to_dev(w['dy'])
+    first = abi.backward(dy, rois, w['data'].shape, scale, S, assign=True)
+    for _ in range(3):
+        again = abi.backward(dy, rois, w['data'].shape, scale, S, assign=True)
+        assert torch.equal(first, again)
+
+
 @pytest.mark.parametrize('impl', IMPLS)
 def test_backward_accumulates_into_existing_gradient(impl):
     abi.set_impl(impl)
