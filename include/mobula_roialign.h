@@ -52,6 +52,15 @@ void roi_align_backward_f318a24e(const int device_id, const int nthreads, const 
                                  const int sampling_ratio, float* bottom_diff,
                                  const float* bottom_rois);
 
+/* The reference's <double> instantiation of the forward (same kernel template,
+ * T = double: map, boxes, scale and result in binary64).
+ * Replaces: roi_align_forward_kernel<double>, opzoo/ROIAlign/ROIAlign.cpp:9-76
+ * under the name mobula/func.py:13-50 derives for it. */
+void roi_align_forward_6b9e6c9b(const int device_id, const int nthreads, const double* bottom_data,
+                                const double spatial_scale, const int channels, const int height,
+                                const int width, const int pooled_height, const int pooled_width,
+                                const int sampling_ratio, const double* bottom_rois, double* top_data);
+
 /* Makes device_id the current device.
  * Replaces: set_device, mobula/cpp/include/context/context.h:15-17. */
 void set_device(const int device_id);
@@ -67,6 +76,20 @@ void roi_align_backward_assign_a8793cbe(const int device_id, const int nthreads,
                                         const int pooled_height, const int pooled_width,
                                         const int sampling_ratio, const int num_images,
                                         float* bottom_diff, const float* bottom_rois);
+
+/* Backward in binary64, accumulating and overwriting.  The names are what the
+ * reference's scheme gives the <double> instantiations, but the reference cannot
+ * build them: its atomic_add takes float only
+ * (mobula/cpp/include/context/cpu_ctx.h:37, context/hip_ctx.h:108-114). */
+void roi_align_backward_2b6c6dfa(const int device_id, const int nthreads, const double* top_diff,
+                                 const double spatial_scale, const int channels, const int height,
+                                 const int width, const int pooled_height, const int pooled_width,
+                                 const int sampling_ratio, double* bottom_diff, const double* bottom_rois);
+void roi_align_backward_assign_4620f85e(const int device_id, const int nthreads, const double* top_diff,
+                                        const double spatial_scale, const int channels, const int height,
+                                        const int width, const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        double* bottom_diff, const double* bottom_rois);
 
 /* Forward with IEEE binary16 storage of bottom_data / top_data (passed as
  * 16-bit patterns), fp32 rois and fp32 accumulation. */

@@ -82,7 +82,8 @@ backward_naive_kernel(long long n_out, const TI* __restrict__ dy, float scale, i
 
 // max(batch index)+1 over all ROIs, for callers that did not say how many
 // images the feature map holds.
-__global__ void max_batch_kernel(const float* __restrict__ rois, int R, int* __restrict__ out) {
+template <typename B>
+__global__ void max_batch_kernel(const B* __restrict__ rois, int R, int* __restrict__ out) {
   int m = 0;
   for (int r = blockIdx.x * blockDim.x + threadIdx.x; r < R; r += gridDim.x * blockDim.x)
     m = max(m, static_cast<int>(rois[r * 5]) + 1);

@@ -52,13 +52,14 @@ class CFuncDef:
     FUNC = 2
 
     def __init__(self, func_name, func_kind, arg_names=None, arg_types=None, rtn_type=None,
-                 template_list=None, loader=None, loader_kwargs=None):
+                 template_list=None, loader=None, loader_kwargs=None, template_defaults=None):
         self.func_name = func_name
         self.func_kind = func_kind
         self.arg_names = arg_names or []
         self.arg_types = arg_types
         self.rtn_type = rtn_type
         self.template_list = template_list or []
+        self.template_defaults = template_defaults or {}   # `typename B = T` -> {'B': 'T'}
         self.loader = loader
         self.loader_kwargs = loader_kwargs or {}
 
@@ -192,8 +193,13 @@ class MobulaFunc:
         for t in decl.arg_types:
             if isinstance(t, TemplateType):
                 if t.tname not in by_name:
-                    assert pending, Exception('missing template type for {}'.format(t.tname))
-                    by_name[t.tname] = pending.pop(0)
+                    if pending:
+                        by_name[t.tname] = pending.pop(0)
+                    else:  # a default names a type, or a parameter given before it
+                        default = decl.template_defaults.get(t.tname)
+                        assert default is not None, Exception(
+                            'missing template type for {}'.format(t.tname))
+                        by_name[t.tname] = by_name.get(default, default)
                 arg_types.append(t(getattr(ctypes, 'c_' + by_name[t.tname], None) or
                                    native.ctype_by_name(by_name[t.tname])))
             else:

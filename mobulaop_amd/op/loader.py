@@ -34,15 +34,20 @@ _RESOLVED = {}
 
 
 def _template_names(line):
+    """`template <typename T, typename B = T>` -> (['T', 'B'], {'B': 'T'}); None if the
+    line opens no template."""
     m = _TEMPLATE_RE.search(line)
     if m is None:
         return None
-    names = []
+    names, defaults = [], {}
     for piece in m.group(1).split(','):
+        piece, _, default = piece.partition('=')
         words = piece.split()
         if len(words) == 2 and words[0] in ('typename', 'class'):
             names.append(words[1])
-    return names
+            if default.strip():
+                defaults[words[1]] = default.strip()
+    return names, defaults
 
 
 def parse_parameter_decl(decl):
@@ -112,13 +117,13 @@ class OpLoader:
 
 def _scan_source(fname):
     info = SourceInfo(fname)
-    templates, pending, depth, kind = [], None, 0, None
+    templates, defaults, pending, depth, kind = [], {}, None, 0, None
     with open(fname) as fin:
         for line in fin:
             if pending is None:
                 names = _template_names(line)
                 if names is not None:
-                    templates = names
+                    templates, defaults = names
                 m = _HEAD_RE.search(line)
                 if m is None:
                     continue
@@ -147,8 +152,9 @@ def _scan_source(fname):
                 func_name=func_name, func_kind=kind,
                 arg_names=[n for _, n in params], arg_types=[t for t, _ in params],
                 rtn_type=rtn_type, template_list=list(templates) if used else [],
+                template_defaults={k: v for k, v in defaults.items() if k in used},
                 loader=OpLoader, loader_kwargs=dict(cpp_info=info))
-            templates = []
+            templates, defaults = [], {}
     assert pending is None, Exception('unbalanced parentheses in a declaration of ' + fname)
     return {name: CFuncDef(**kw) for name, kw in info.function_args.items()}
 

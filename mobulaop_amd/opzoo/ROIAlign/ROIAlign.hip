@@ -11,6 +11,7 @@
 
 #include "runtime.h"
 #include "roialign_naive.hip.h"
+#include "roialign_f64.hip.h"
 #include "roialign_backward_blocked.hip.h"
 #include "roialign_forward_blocked.hip.h"
 #include "roialign_forward_merged.hip.h"
@@ -29,6 +30,7 @@ struct Problem {
   int R, C, H, W, PH, PW, S;
   long long N;      // images in the feature map
   float scale;
+  double scale64 = 0.0;  // the scale as given, for the binary64 kernels
   bool nhwc = false;   // map [N,H,W,C] and pooled tensor [R,PH,PW,C] instead of [N,C,H,W] / [R,C,PH,PW]
 };
 
@@ -87,7 +89,8 @@ bool describe(Problem* p, const char* what, int nthreads, float scale, int C, in
 
 // Number of images when the caller gave neither extents nor a count: read the
 // largest batch index back from the device (one blocking copy).
-long long images_from_rois(const float* d_rois, int R, hipStream_t stream) {
+template <typename B>
+long long images_from_rois(const B* d_rois, int R, hipStream_t stream) {
   if (R == 0) return 0;
   int* d_max = static_cast<int*>(mobula_hip::workspace(256));
   if (failed()) return 0;
@@ -343,7 +346,27 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
   MOBULA_HIP_TRY(hipGetLastError());
 }
 
-long long host_images(const float* rois, int R) {
+// binary64: the straightforward kernels only.
+void forward_device(const Problem& p, const double* x, const double* rois, double* y, hipStream_t stream) {
+  if (p.n_out == 0) return;
+  roialign::roialign_f64_kernel<0><<<grid_for(p.n_out, 256), 256, 0, stream>>>(
+      p.n_out, x, p.scale64, p.C, p.H, p.W, p.PH, p.PW, p.S, rois, y, p.N);
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+void backward_device(const Problem& p, const double* dy, const double* rois, double* dx, bool assign,
+                     hipStream_t stream) {
+  const long long map = static_cast<long long>(p.N) * p.C * p.H * p.W;
+  if (assign && map > 0)
+    roialign::zero_words_kernel<<<grid_for(2 * map, 256), 256, 0, stream>>>(reinterpret_cast<unsigned*>(dx), 2 * map);
+  if (p.n_out > 0)
+    roialign::roialign_f64_kernel<1><<<grid_for(p.n_out, 256), 256, 0, stream>>>(
+        p.n_out, dy, p.scale64, p.C, p.H, p.W, p.PH, p.PW, p.S, rois, dx, p.N);
+  MOBULA_HIP_TRY(hipGetLastError());
+}
+
+template <typename B>
+long long host_images(const B* rois, int R) {
   long long n = 0;
   for (int r = 0; r < R; ++r) n = std::max<long long>(n, static_cast<long long>(rois[5 * r]) + 1);
   return n;
@@ -355,34 +378,40 @@ long long host_images(const float* rois, int R) {
 // Launchers (scanned by the Python loader).
 // ---------------------------------------------------------------------------
 
-template <typename T>
+// T: element type of the map and of the pooled tensor; B: type of the boxes and of
+// the scale.  The reference has one parameter for both (ROIAlign.cpp:9-16): its
+// float and double instantiations are <float>, <double> here too (B defaults to
+// T); binary16 maps come with binary32 boxes, <half, float>.
+template <typename T, typename B = T>
 MOBULA_KERNEL roi_align_forward_kernel(const int nthreads, const T* bottom_data,
-                                       const float spatial_scale, const int channels,
+                                       const B spatial_scale, const int channels,
                                        const int height, const int width,
                                        const int pooled_height, const int pooled_width,
-                                       const int sampling_ratio, const float* bottom_rois,
+                                       const int sampling_ratio, const B* bottom_rois,
                                        T* top_data) {
   Problem p;
-  if (!describe(&p, "roi_align_forward", nthreads, spatial_scale, channels, height, width,
-                pooled_height, pooled_width, sampling_ratio, 1, 9, 10, -1))
+  if (!describe(&p, "roi_align_forward", nthreads, static_cast<float>(spatial_scale), channels, height,
+                width, pooled_height, pooled_width, sampling_ratio, 1, 9, 10, -1))
     return;
+  p.scale64 = spatial_scale;
   hipStream_t stream = call_state().stream;
   if (p.N < 0) p.N = images_from_rois(bottom_rois, p.R, stream);
   if (failed()) return;
-  forward_device<T>(p, bottom_data, bottom_rois, top_data, stream);
+  forward_device(p, bottom_data, bottom_rois, top_data, stream);
 }
 
-template <typename T>
+template <typename T, typename B = T>
 MOBULA_KERNEL roi_align_backward_kernel(const int nthreads, const T* top_diff,
-                                        const float spatial_scale, const int channels,
+                                        const B spatial_scale, const int channels,
                                         const int height, const int width,
                                         const int pooled_height, const int pooled_width,
                                         const int sampling_ratio, T* bottom_diff,
-                                        const float* bottom_rois) {
+                                        const B* bottom_rois) {
   Problem p;
-  if (!describe(&p, "roi_align_backward", nthreads, spatial_scale, channels, height, width,
-                pooled_height, pooled_width, sampling_ratio, 9, 10, 1, -1))
+  if (!describe(&p, "roi_align_backward", nthreads, static_cast<float>(spatial_scale), channels, height,
+                width, pooled_height, pooled_width, sampling_ratio, 9, 10, 1, -1))
     return;
+  p.scale64 = spatial_scale;
   hipStream_t stream = call_state().stream;
   if (p.N < 0) p.N = images_from_rois(bottom_rois, p.R, stream);
   if (failed()) return;
@@ -393,21 +422,22 @@ MOBULA_KERNEL roi_align_backward_kernel(const int nthreads, const T* top_diff,
 // written exactly once; elements no ROI touches become zero), i.e. the
 // operator's "zero dx, then scatter" (opzoo/ROIAlign/ROIAlign.py:33-39) as one
 // entry point.  num_images is the N of the [N,C,H,W] gradient.
-template <typename T>
+template <typename T, typename B = T>
 MOBULA_KERNEL roi_align_backward_assign_kernel(const int nthreads, const T* top_diff,
-                                               const float spatial_scale, const int channels,
+                                               const B spatial_scale, const int channels,
                                                const int height, const int width,
                                                const int pooled_height, const int pooled_width,
                                                const int sampling_ratio, const int num_images,
-                                               T* bottom_diff, const float* bottom_rois) {
+                                               T* bottom_diff, const B* bottom_rois) {
   Problem p;
   if (num_images < 0) {
     set_error("roi_align_backward_assign: num_images=%d", num_images);
     return;
   }
-  if (!describe(&p, "roi_align_backward_assign", nthreads, spatial_scale, channels, height, width,
-                pooled_height, pooled_width, sampling_ratio, 10, 11, 1, num_images))
+  if (!describe(&p, "roi_align_backward_assign", nthreads, static_cast<float>(spatial_scale), channels,
+                height, width, pooled_height, pooled_width, sampling_ratio, 10, 11, 1, num_images))
     return;
+  p.scale64 = spatial_scale;
   backward_device(p, top_diff, bottom_rois, bottom_diff, /*assign=*/true, call_state().stream);
 }
 
@@ -480,12 +510,12 @@ namespace {
 
 int staging_device() { return static_cast<int>(mobula_hip::option("host_staging_device", 0)); }
 
-template <typename T>
-void forward_entry(int device_id, int nthreads, const T* x, float scale, int C, int H, int W,
-                   int PH, int PW, int S, const float* rois, T* y) {
+template <typename T, typename B>
+void forward_entry(int device_id, int nthreads, const T* x, B scale, int C, int H, int W,
+                   int PH, int PW, int S, const B* rois, T* y) {
   if (device_id >= 0) {
     mobula_hip::DeviceScope scope(device_id);
-    if (scope.ok()) roi_align_forward_kernel<T>(nthreads, x, scale, C, H, W, PH, PW, S, rois, y);
+    if (scope.ok()) roi_align_forward_kernel<T, B>(nthreads, x, scale, C, H, W, PH, PW, S, rois, y);
     mobula_hip::finish_call();
     return;
   }
@@ -495,34 +525,34 @@ void forward_entry(int device_id, int nthreads, const T* x, float scale, int C, 
   const hipStream_t saved_stream = st.stream;
   st.stream = nullptr;
   Problem p;
-  if (scope.ok() && describe(&p, "roi_align_forward", nthreads, scale, C, H, W, PH, PW, S, 1, 9,
-                             10, -1)) {
+  if (scope.ok() && describe(&p, "roi_align_forward", nthreads, static_cast<float>(scale), C, H, W, PH,
+                             PW, S, 1, 9, 10, -1)) {
     if (p.N < 0) p.N = host_images(rois, p.R);
     st.extents.assign(11, -1);
     st.extents[1] = p.N * C * H * W;
     mobula_hip::HostStaging stage;
     const T* dx = static_cast<const T*>(stage.in(x, sizeof(T) * p.N * C * H * W));
-    const float* dr = static_cast<const float*>(stage.in(rois, sizeof(float) * 5 * p.R));
+    const B* dr = static_cast<const B*>(stage.in(rois, sizeof(B) * 5 * p.R));
     T* dy = static_cast<T*>(stage.inout(y, sizeof(T) * p.n_out, /*upload=*/false));
-    if (!failed()) roi_align_forward_kernel<T>(nthreads, dx, scale, C, H, W, PH, PW, S, dr, dy);
+    if (!failed()) roi_align_forward_kernel<T, B>(nthreads, dx, scale, C, H, W, PH, PW, S, dr, dy);
     if (!failed()) stage.flush(nullptr);
   }
   st.stream = saved_stream;
   st.extents.clear();
 }
 
-template <typename T>
-void backward_entry(int device_id, int nthreads, const T* dy, float scale, int C, int H, int W,
-                    int PH, int PW, int S, int num_images, T* dx, const float* rois) {
+template <typename T, typename B>
+void backward_entry(int device_id, int nthreads, const T* dy, B scale, int C, int H, int W,
+                    int PH, int PW, int S, int num_images, T* dx, const B* rois) {
   const bool assign = num_images >= 0;
   if (device_id >= 0) {
     mobula_hip::DeviceScope scope(device_id);
     if (scope.ok()) {
       if (assign)
-        roi_align_backward_assign_kernel<T>(nthreads, dy, scale, C, H, W, PH, PW, S, num_images,
-                                            dx, rois);
+        roi_align_backward_assign_kernel<T, B>(nthreads, dy, scale, C, H, W, PH, PW, S, num_images,
+                                               dx, rois);
       else
-        roi_align_backward_kernel<T>(nthreads, dy, scale, C, H, W, PH, PW, S, dx, rois);
+        roi_align_backward_kernel<T, B>(nthreads, dy, scale, C, H, W, PH, PW, S, dx, rois);
     }
     mobula_hip::finish_call();
     return;
@@ -533,21 +563,21 @@ void backward_entry(int device_id, int nthreads, const T* dy, float scale, int C
   st.stream = nullptr;
   Problem p;
   const int e_map = assign ? 10 : 9, e_rois = assign ? 11 : 10;
-  if (scope.ok() && describe(&p, "roi_align_backward", nthreads, scale, C, H, W, PH, PW, S, e_map,
-                             e_rois, 1, assign ? num_images : -1)) {
+  if (scope.ok() && describe(&p, "roi_align_backward", nthreads, static_cast<float>(scale), C, H, W, PH,
+                             PW, S, e_map, e_rois, 1, assign ? num_images : -1)) {
     if (p.N < 0) p.N = host_images(rois, p.R);
     mobula_hip::HostStaging stage;
     const T* ddy = static_cast<const T*>(stage.in(dy, sizeof(T) * p.n_out));
-    const float* dr = static_cast<const float*>(stage.in(rois, sizeof(float) * 5 * p.R));
+    const B* dr = static_cast<const B*>(stage.in(rois, sizeof(B) * 5 * p.R));
     T* ddx = static_cast<T*>(stage.inout(dx, sizeof(T) * p.N * C * H * W, /*upload=*/!assign));
     st.extents.assign(12, -1);
     st.extents[e_map] = p.N * C * H * W;
     if (!failed()) {
       if (assign)
-        roi_align_backward_assign_kernel<T>(nthreads, ddy, scale, C, H, W, PH, PW, S,
-                                            static_cast<int>(p.N), ddx, dr);
+        roi_align_backward_assign_kernel<T, B>(nthreads, ddy, scale, C, H, W, PH, PW, S,
+                                               static_cast<int>(p.N), ddx, dr);
       else
-        roi_align_backward_kernel<T>(nthreads, ddy, scale, C, H, W, PH, PW, S, ddx, dr);
+        roi_align_backward_kernel<T, B>(nthreads, ddy, scale, C, H, W, PH, PW, S, ddx, dr);
     }
     if (!failed()) stage.flush(nullptr);
   }
@@ -565,7 +595,7 @@ void roi_align_forward_ab78de3c(const int device_id, const int nthreads, const f
                                 const int width, const int pooled_height, const int pooled_width,
                                 const int sampling_ratio, const float* bottom_rois,
                                 float* top_data) {
-  forward_entry<float>(device_id, nthreads, bottom_data, spatial_scale, channels, height, width,
+  forward_entry<float, float>(device_id, nthreads, bottom_data, spatial_scale, channels, height, width,
                        pooled_height, pooled_width, sampling_ratio, bottom_rois, top_data);
 }
 
@@ -574,8 +604,42 @@ void roi_align_backward_f318a24e(const int device_id, const int nthreads, const 
                                  const int width, const int pooled_height, const int pooled_width,
                                  const int sampling_ratio, float* bottom_diff,
                                  const float* bottom_rois) {
-  backward_entry<float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+  backward_entry<float, float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
                         pooled_height, pooled_width, sampling_ratio, -1, bottom_diff, bottom_rois);
+}
+
+// double instantiations.  The reference builds the forward only (its atomic_add
+// takes float); the two backward symbols follow its naming scheme.
+void roi_align_forward_6b9e6c9b(const int device_id, const int nthreads, const double* bottom_data,
+                                const double spatial_scale, const int channels, const int height,
+                                const int width, const int pooled_height, const int pooled_width,
+                                const int sampling_ratio, const double* bottom_rois,
+                                double* top_data) {
+  forward_entry<double, double>(device_id, nthreads, bottom_data, spatial_scale, channels, height, width,
+                                pooled_height, pooled_width, sampling_ratio, bottom_rois, top_data);
+}
+
+void roi_align_backward_2b6c6dfa(const int device_id, const int nthreads, const double* top_diff,
+                                 const double spatial_scale, const int channels, const int height,
+                                 const int width, const int pooled_height, const int pooled_width,
+                                 const int sampling_ratio, double* bottom_diff,
+                                 const double* bottom_rois) {
+  backward_entry<double, double>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+                                 pooled_height, pooled_width, sampling_ratio, -1, bottom_diff, bottom_rois);
+}
+
+void roi_align_backward_assign_4620f85e(const int device_id, const int nthreads, const double* top_diff,
+                                        const double spatial_scale, const int channels, const int height,
+                                        const int width, const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        double* bottom_diff, const double* bottom_rois) {
+  if (num_images < 0) {
+    set_error("roi_align_backward_assign: num_images=%d", num_images);
+    return;
+  }
+  backward_entry<double, double>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+                                 pooled_height, pooled_width, sampling_ratio, num_images, bottom_diff,
+                                 bottom_rois);
 }
 
 // Extensions (no counterpart in the reference); names follow the same scheme.
@@ -589,7 +653,7 @@ void roi_align_backward_assign_a8793cbe(const int device_id, const int nthreads,
     set_error("roi_align_backward_assign: num_images=%d", num_images);
     return;
   }
-  backward_entry<float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+  backward_entry<float, float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
                         pooled_height, pooled_width, sampling_ratio, num_images, bottom_diff,
                         bottom_rois);
 }
@@ -599,7 +663,7 @@ void roi_align_backward_23175303(const int device_id, const int nthreads, const 
                                  const float spatial_scale, const int channels, const int height,
                                  const int width, const int pooled_height, const int pooled_width,
                                  const int sampling_ratio, __half* bottom_diff, const float* bottom_rois) {
-  backward_entry<__half>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+  backward_entry<__half, float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
                          pooled_height, pooled_width, sampling_ratio, -1, bottom_diff, bottom_rois);
 }
 
@@ -612,7 +676,7 @@ void roi_align_backward_assign_7924dbc8(const int device_id, const int nthreads,
     set_error("roi_align_backward_assign: num_images=%d", num_images);
     return;
   }
-  backward_entry<__half>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
+  backward_entry<__half, float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
                          pooled_height, pooled_width, sampling_ratio, num_images, bottom_diff, bottom_rois);
 }
 
@@ -689,7 +753,7 @@ void roi_align_forward_e874c59a(const int device_id, const int nthreads, const _
                                 const int width, const int pooled_height, const int pooled_width,
                                 const int sampling_ratio, const float* bottom_rois,
                                 __half* top_data) {
-  forward_entry<__half>(device_id, nthreads, bottom_data, spatial_scale, channels, height, width,
+  forward_entry<__half, float>(device_id, nthreads, bottom_data, spatial_scale, channels, height, width,
                         pooled_height, pooled_width, sampling_ratio, bottom_rois, top_data);
 }
 
@@ -697,6 +761,7 @@ void roi_align_forward_e874c59a(const int device_id, const int nthreads, const _
 
 static mobula_hip::ExportRegistrar roialign_exports(
     "roi_align_forward_ab78de3c roi_align_backward_f318a24e roi_align_backward_assign_a8793cbe "
+    "roi_align_forward_6b9e6c9b roi_align_backward_2b6c6dfa roi_align_backward_assign_4620f85e "
     "roi_align_forward_e874c59a roi_align_backward_23175303 roi_align_backward_assign_7924dbc8 "
     "roi_align_forward_nhwc_ab78de3c roi_align_forward_nhwc_e874c59a "
     "roi_align_backward_nhwc_f318a24e roi_align_backward_nhwc_assign_a8793cbe "

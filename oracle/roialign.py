@@ -75,6 +75,45 @@ def forward(data, rois, pooled_size, spatial_scale, sampling_ratio, impl='oracle
     return out
 
 
+def _f64(a):
+    a = np.ascontiguousarray(a, dtype=np.float64)
+    return a, a.ctypes.data_as(ctypes.c_void_p)
+
+
+def forward_f64(data, rois, pooled_size, spatial_scale, sampling_ratio, impl='oracle'):
+    """The double instantiation: float64 `data`, `rois` and scale.  impl: oracle |
+    ref_omp | ref_serial (the compiled reference, forward only)."""
+    data, pd = _f64(data)
+    rois, pr = _f64(rois)
+    N, C, H, W = data.shape
+    PH, PW = pooled_size
+    R = rois.shape[0]
+    out = np.zeros((R, C, PH, PW), dtype=np.float64)
+    po = out.ctypes.data_as(ctypes.c_void_p)
+    geometry = [ctypes.c_double(spatial_scale)] + [ctypes.c_int(v) for v in (C, H, W, PH, PW, sampling_ratio)]
+    if impl == 'oracle':
+        _lib().oracle_roi_align_forward_f64(ctypes.c_int(R), ctypes.c_int(N), pd, *geometry, pr, po)
+    else:
+        _ref(impl[4:]).roi_align_forward_6b9e6c9b(ctypes.c_int(-1), ctypes.c_int(out.size), pd, *geometry,
+                                                  pr, po)
+    return out
+
+
+def backward_f64(dy, rois, data_shape, spatial_scale, sampling_ratio, dx=None):
+    """dx[N,C,H,W] in float64, accumulated into `dx` (zeros if None); oracle only."""
+    dy, pdy = _f64(dy)
+    rois, pr = _f64(rois)
+    N, C, H, W = data_shape
+    PH, PW = dy.shape[2], dy.shape[3]
+    if dx is None:
+        dx = np.zeros(data_shape, dtype=np.float64)
+    assert dx.dtype == np.float64 and dx.flags.c_contiguous
+    geometry = [ctypes.c_double(spatial_scale)] + [ctypes.c_int(v) for v in (C, H, W, PH, PW, sampling_ratio)]
+    _lib().oracle_roi_align_backward_f64(ctypes.c_int(rois.shape[0]), ctypes.c_int(N), pdy, *geometry,
+                                         dx.ctypes.data_as(ctypes.c_void_p), pr)
+    return dx
+
+
 def backward(dy, rois, data_shape, spatial_scale, sampling_ratio, impl='oracle', dx=None):
     """dx[N,C,H,W] accumulated into `dx` (zeros if None).
 
@@ -100,15 +139,12 @@ def backward(dy, rois, data_shape, spatial_scale, sampling_ratio, impl='oracle',
 
 
 # ---------------------------------------------------------------------------
-# Independent slow restatement (NumPy float32 scalars, explicit loops).  Written
+# Independent slow restatement (NumPy scalars of one type, explicit loops).  Written
 # from the algorithm description, structured differently from the C file (it
 # builds per-axis sample tables first), so a slip in either shows up as a
 # mismatch.  Tiny shapes only.
 # ---------------------------------------------------------------------------
-_F = np.float32
-
-
-def _axis_table(start, bin_size, pooled, grid, size):
+def _axis_table(start, bin_size, pooled, grid, size, _F):
     """Per (p, i): (valid, low, high, l, h) along one axis."""
     table = []
     for p in range(pooled):
@@ -131,8 +167,10 @@ def _axis_table(start, bin_size, pooled, grid, size):
     return table
 
 
-def brute_force(data, rois, pooled_size, spatial_scale, sampling_ratio, dy=None):
-    """Returns (y, dx); dx is None when dy is None."""
+def brute_force(data, rois, pooled_size, spatial_scale, sampling_ratio, dy=None, dtype=np.float32):
+    """Returns (y, dx); dx is None when dy is None.  Every operation is rounded to
+    `dtype` (float32: the reference's float kernels, float64: its double ones)."""
+    _F = dtype
     data = np.asarray(data, dtype=_F)
     rois = np.asarray(rois, dtype=_F)
     N, C, H, W = data.shape
@@ -150,8 +188,8 @@ def brute_force(data, rois, pooled_size, spatial_scale, sampling_ratio, dy=None)
         gh = sampling_ratio if sampling_ratio > 0 else int(np.ceil(_F(rh / _F(PH))))
         gw = sampling_ratio if sampling_ratio > 0 else int(np.ceil(_F(rw / _F(PW))))
         cnt = _F(gh * gw)
-        ty = _axis_table(sh, bh, PH, gh, H)
-        tx = _axis_table(sw, bw, PW, gw, W)
+        ty = _axis_table(sh, bh, PH, gh, H, _F)
+        tx = _axis_table(sw, bw, PW, gw, W, _F)
         for c in range(C):
             plane = data[b, c]
             for ph in range(PH):

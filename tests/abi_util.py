@@ -34,8 +34,8 @@ def _end(lib):
         raise RuntimeError(msg.decode())
 
 
-def _geom(scale, C, H, W, PH, PW, S):
-    return [ctypes.c_float(scale)] + [ctypes.c_int(v) for v in (C, H, W, PH, PW, S)]
+def _geom(scale, C, H, W, PH, PW, S, real=ctypes.c_float):
+    return [real(scale)] + [ctypes.c_int(v) for v in (C, H, W, PH, PW, S)]
 
 
 def forward(x, rois, pooled, scale, S, declare_extents=True, stream=None, dev=0):
@@ -46,6 +46,12 @@ def forward(x, rois, pooled, scale, S, declare_extents=True, stream=None, dev=0)
     y = torch.empty((R, C, PH, PW), dtype=x.dtype, device=x.device)
     ext = [-1, x.numel(), -1, -1, -1, -1, -1, -1, -1, rois.numel(), y.numel()]
     lib = _begin(ext if declare_extents else [], stream)
+    if x.dtype == torch.float64:   # the double instantiation: boxes and scale are double too
+        assert rois.dtype == torch.float64
+        lib.roi_align_forward_6b9e6c9b(ctypes.c_int(dev), ctypes.c_int(y.numel()), _ptr(x),
+                                       *_geom(scale, C, H, W, PH, PW, S, ctypes.c_double), _ptr(rois), _ptr(y))
+        _end(lib)
+        return y
     fn = lib.roi_align_forward_ab78de3c if x.dtype == torch.float32 else lib.roi_align_forward_e874c59a
     fn(ctypes.c_int(dev), ctypes.c_int(y.numel()), _ptr(x), *_geom(scale, C, H, W, PH, PW, S),
        _ptr(rois), _ptr(y))
@@ -62,6 +68,21 @@ def backward(dy, rois, shape, scale, S, dx=None, assign=False, declare_extents=T
               else torch.zeros(shape, dtype=dy.dtype, device=dy.device))
     lib = native.library()
     half = dy.dtype == torch.float16
+    if dy.dtype == torch.float64:
+        assert rois.dtype == torch.float64
+        geom = _geom(scale, C, H, W, PH, PW, S, ctypes.c_double)
+        if assign:
+            _begin([-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()]
+                   if declare_extents else [], stream)
+            lib.roi_align_backward_assign_4620f85e(ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *geom,
+                                                   ctypes.c_int(N), _ptr(dx), _ptr(rois))
+        else:
+            _begin([-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()]
+                   if declare_extents else [], stream)
+            lib.roi_align_backward_2b6c6dfa(ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *geom,
+                                            _ptr(dx), _ptr(rois))
+        _end(lib)
+        return dx
     if assign:
         ext = [-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()]
         _begin(ext if declare_extents else [], stream)

@@ -34,13 +34,19 @@ def test_library_exports_every_declared_symbol():
 def test_symbol_names_follow_the_reference_scheme(mobula):
     from mobulaop_amd.func import get_func_idcode, get_idcode_hash
     from mobulaop_amd.dtype import c_half
-    cases = [('roi_align_forward', ctypes.c_float, 'roi_align_forward_ab78de3c'),
-             ('roi_align_backward', ctypes.c_float, 'roi_align_backward_f318a24e'),
-             ('roi_align_backward_assign', ctypes.c_float, 'roi_align_backward_assign_a8793cbe'),
-             ('roi_align_forward', c_half, 'roi_align_forward_e874c59a')]
-    for fname, ctype, want in cases:
+    # (function, element type T, box type B, symbol); the float and double names are
+    # the reference's own (mobula/func.py:13-50 over ROIAlign.cpp:10-16, 79-83)
+    cases = [('roi_align_forward', ctypes.c_float, ctypes.c_float, 'roi_align_forward_ab78de3c'),
+             ('roi_align_backward', ctypes.c_float, ctypes.c_float, 'roi_align_backward_f318a24e'),
+             ('roi_align_forward', ctypes.c_double, ctypes.c_double, 'roi_align_forward_6b9e6c9b'),
+             ('roi_align_backward', ctypes.c_double, ctypes.c_double, 'roi_align_backward_2b6c6dfa'),
+             ('roi_align_backward_assign', ctypes.c_float, ctypes.c_float,
+              'roi_align_backward_assign_a8793cbe'),
+             ('roi_align_forward', c_half, ctypes.c_float, 'roi_align_forward_e874c59a')]
+    for fname, elem, box, want in cases:
         decl = getattr(mobula.func, fname).func
-        types = [t(ctype) if hasattr(t, 'tname') else t for t in decl.arg_types]
+        bound = {'T': elem, 'B': box}
+        types = [t(bound[t.tname]) if hasattr(t, 'tname') else t for t in decl.arg_types]
         assert get_idcode_hash(get_func_idcode(fname, types)) == want
 
 

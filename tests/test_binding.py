@@ -61,7 +61,7 @@ def test_argument_count_and_type_errors(mobula):
         mobula.func.roi_align_forward(1, [1, 2, 3], 1.0, 1, 2, 2, 1, 1, 1, r, y)  # not a tensor
     with pytest.raises(AssertionError):                               # T bound to float, then double
         mobula.func.roi_align_forward(1, x, 1.0, 1, 2, 2, 1, 1, 1, r, y.astype(np.float64))
-    with pytest.raises(AssertionError):                               # rois must be float
+    with pytest.raises(NameError):                # float map with double boxes: no such instantiation
         mobula.func.roi_align_forward(1, x, 1.0, 1, 2, 2, 1, 1, 1, r.astype(np.float64), y)
     with pytest.raises(KeyError):                                     # missing keyword
         mobula.func.roi_align_forward(nthreads=1, bottom_data=x)

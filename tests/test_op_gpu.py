@@ -169,3 +169,23 @@ def test_half_precision_training_step(mobula):
     yf.backward(dy.float())
     assert float((yh.detach().float() - yf.detach()).abs().max()) <= 2e-3 * float(yf.detach().abs().max())
     assert float((xh.grad.float() - xf.grad).abs().max()) <= 2e-3 * float(xf.grad.abs().max())
+
+
+def test_double_tensors_through_the_operator(mobula):
+    """float64 data and boxes resolve to the double instantiation; autograd gets dx."""
+    rng = np.random.default_rng(9)
+    xh = rng.standard_normal((2, 3, 12, 14))
+    rh = np.array([[0, 2.5, 3.5, 30.25, 28.0], [1, -4, 0, 20, 44], [1, 8, 8, 8, 8]], dtype=np.float64)
+    dyh = rng.standard_normal((3, 3, 4, 4))
+    x = torch.from_numpy(xh).cuda().requires_grad_(True)
+    rois = torch.from_numpy(rh).cuda()
+    y = mobula.op.ROIAlign(x, rois, pooled_size=(4, 4), spatial_scale=0.25, sampling_ratio=0)
+    assert y.dtype == torch.float64
+    np.testing.assert_array_equal(y.detach().cpu().numpy(), oracle.forward_f64(xh, rh, (4, 4), 0.25, 0))
+    y.backward(torch.from_numpy(dyh).cuda())
+    np.testing.assert_allclose(x.grad.cpu().numpy(), oracle.backward_f64(dyh, rh, xh.shape, 0.25, 0),
+                               rtol=0, atol=1e-13)
+    # host arrays take the same symbols (device id -1: staged through the GPU)
+    out = np.zeros((3, 3, 4, 4))
+    mobula.func.roi_align_forward(out.size, xh, 0.25, 3, 12, 14, 4, 4, 0, rh, out)
+    np.testing.assert_array_equal(out, oracle.forward_f64(xh, rh, (4, 4), 0.25, 0))

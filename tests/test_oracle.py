@@ -173,3 +173,76 @@ def test_golden_fixtures():
         np.testing.assert_array_equal(y, z['y'], err_msg=name)
         dx = oracle.backward(z['dy'], z['rois'], z['data'].shape, scale, S, impl='ordered')
         np.testing.assert_array_equal(dx, z['dx'], err_msg=name)
+
+
+# ---------------------------------------------------------------------------
+# The double instantiation (oracle/roialign_oracle_f64.c).
+# ---------------------------------------------------------------------------
+def _random_case_f64(rng, **kw):
+    x, rois, dy, pooled, scale = _random_case(rng, **kw)
+    # fresh float64 draws (not widened float32 values): every mantissa bit in play
+    return (x + 1e-9 * rng.standard_normal(x.shape), rois.astype(np.float64) + 1e-7 * rng.random(rois.shape)
+            * (np.arange(5) > 0), dy + 1e-9 * rng.standard_normal(dy.shape), pooled, scale)
+
+
+def test_f64_known_answer_and_plane():
+    x = np.arange(2 * 3 * 4 * 4, dtype=np.float64).reshape(2, 3, 4, 4)
+    rois = np.array([[0, 1, 1, 3, 3]], dtype=np.float64)
+    y = oracle.forward_f64(x, rois, (2, 2), 1.0, 1)
+    for c in range(3):
+        np.testing.assert_array_equal(y[0, c], np.array([[7.5, 8.5], [11.5, 12.5]]) + 16 * c)
+    dx = oracle.backward_f64(np.ones_like(y), rois, x.shape, 1.0, 1)
+    want = np.zeros_like(x)
+    want[0, :, 1:4, 1:4] = [[.25, .5, .25], [.5, 1, .5], [.25, .5, .25]]
+    np.testing.assert_array_equal(dx, want)
+    # a plane a*y + b*x + c is reproduced at the bin centres when every sample is inside
+    H, W = 12, 15
+    yy, xx = np.mgrid[0:H, 0:W]
+    plane = (3.0 * yy + 2.0 * xx + 1.0)[None, None]
+    out = oracle.forward_f64(plane, np.array([[0, 1, 1, 5, 5]], dtype=np.float64), (2, 2), 1.0, 2)
+    np.testing.assert_allclose(out[0, 0], [[11, 15], [17, 21]], rtol=1e-14)
+
+
+@pytest.mark.parametrize('S', [0, 1, 2, 3])
+def test_f64_against_independent_numpy_loop_and_adjoint(S):
+    rng = np.random.default_rng(300 + S)
+    x, rois, dy, pooled, scale = _random_case_f64(rng, N=2, C=2, H=9, W=11, R=6, span=50.0)
+    rois[0, 1:] = [-20, -20, 15, 10]      # partly outside
+    rois[1, 1:] = [12, 12, 12, 12]        # zero size
+    y = oracle.forward_f64(x, rois, pooled, scale, S)
+    dx = oracle.backward_f64(dy, rois, x.shape, scale, S)
+    want_y, want_dx = oracle.brute_force(x, rois, pooled, scale, S, dy=dy, dtype=np.float64)
+    np.testing.assert_array_equal(y, want_y)
+    np.testing.assert_allclose(dx, want_dx, rtol=0, atol=1e-14)
+    # the operator is linear in x: <fwd(x), dy> == <x, bwd(dy)>
+    lhs, rhs = float((y * dy).sum()), float((x * dx).sum())
+    assert abs(lhs - rhs) <= 1e-12 * max(1.0, np.abs(y * dy).sum())
+    # and genuinely double: the float32 kernels differ from it at float32 precision only
+    y32 = oracle.forward(x, rois, pooled, scale, S)
+    assert 0 < np.abs(y32 - y).max() < 1e-4
+
+
+@needs_ref
+@pytest.mark.parametrize('S', [0, 2])
+def test_f64_bit_exact_against_compiled_reference(S):
+    rng = np.random.default_rng(400 + S)
+    x, rois, _, pooled, scale = _random_case_f64(rng, N=3, C=3, H=20, W=27, R=30, span=140.0)
+    rois[0, 1:] = [200, 200, 260, 260]
+    rois[1, 1:] = [10, 10, 10, 10]
+    rois[2, 1:] = [33.3, 20.1, 33.6, 20.2]
+    rois[3, 1:] = [-30, -30, 50, 20]
+    for impl in ('ref_omp', 'ref_serial'):
+        np.testing.assert_array_equal(oracle.forward_f64(x, rois, pooled, scale, S),
+                                      oracle.forward_f64(x, rois, pooled, scale, S, impl=impl))
+
+
+def test_f64_golden_fixtures():
+    folder = os.path.join(GOLDEN, 'f64')
+    files = sorted(f for f in os.listdir(folder) if f.endswith('.npz'))
+    assert files, 'no double fixtures committed'
+    for name in files:
+        z = np.load(os.path.join(folder, name))
+        pooled = tuple(int(v) for v in z['pooled_size'])
+        y = oracle.forward_f64(z['data'], z['rois'], pooled, float(z['spatial_scale']),
+                               int(z['sampling_ratio']))
+        np.testing.assert_array_equal(y, z['y'], err_msg=name)

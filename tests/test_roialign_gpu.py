@@ -229,6 +229,45 @@ def test_channels_last_rejects_what_it_does_not_take():
     assert abi.forward_nhwc(torch.zeros(1, 8, 8, 8, device='cuda'), rois, (2, 2), 1.0, 2).shape == (1, 2, 2, 8)
 
 
+F64_TOL = 1e-12   # binary64: only the backward's summation order may differ
+
+
+@pytest.mark.parametrize('S', [2, 0])
+def test_double_instantiation(S):
+    """roi_align_forward_6b9e6c9b (the reference's <double> forward) and the two
+    double backward entry points, against the double oracle and the fixtures the
+    compiled reference wrote."""
+    folder = os.path.join(GOLDEN, 'f64')
+    for name in sorted(f for f in os.listdir(folder) if f.endswith('.npz')):
+        z = np.load(os.path.join(folder, name))
+        pooled = tuple(int(v) for v in z['pooled_size'])
+        y = abi.forward(abi.to_dev(z['data']), abi.to_dev(z['rois']), pooled, float(z['spatial_scale']),
+                        int(z['sampling_ratio']))
+        assert y.dtype == torch.float64
+        np.testing.assert_array_equal(y.cpu().numpy(), z['y'], err_msg=name)   # same operations, same order
+    rng = np.random.default_rng(77 + S)
+    N, C, H, W, R, pooled, scale = 3, 5, 21, 30, 50, (5, 6), 0.3
+    xh = rng.standard_normal((N, C, H, W))
+    c, wh = rng.uniform(-10, 110, size=(R, 2)), rng.uniform(0, 90, size=(R, 2))
+    rh = np.concatenate([rng.integers(0, N, size=(R, 1)), c - wh / 2, c + wh / 2], axis=1)
+    rh[0, 1:] = [400, 400, 500, 500]
+    rh[1, 1:] = [20, 20, 20, 20]
+    dyh = rng.standard_normal((R, C) + pooled)
+    x, rois, dy = abi.to_dev(xh), abi.to_dev(rh), abi.to_dev(dyh)
+    np.testing.assert_array_equal(abi.forward(x, rois, pooled, scale, S).cpu().numpy(),
+                                  oracle.forward_f64(xh, rh, pooled, scale, S))
+    want_dx = oracle.backward_f64(dyh, rh, xh.shape, scale, S)
+    assert_parity(abi.backward(dy, rois, x.shape, scale, S).cpu().numpy(), want_dx, F64_TOL, 'bwd')
+    assert_parity(abi.backward(dy, rois, x.shape, scale, S, assign=True).cpu().numpy(), want_dx, F64_TOL,
+                  'bwd assign')
+    seed = torch.ones_like(x)
+    assert_parity(abi.backward(dy, rois, x.shape, scale, S, dx=seed).cpu().numpy(), want_dx + 1.0, F64_TOL,
+                  'bwd accumulate')
+    # without declared extents the image count comes from the (double) boxes
+    np.testing.assert_array_equal(abi.forward(x, rois, pooled, scale, S, declare_extents=False).cpu().numpy(),
+                                  oracle.forward_f64(xh, rh, pooled, scale, S))
+
+
 @pytest.mark.parametrize('impl', IMPLS)
 def test_empty_roi_list_and_out_of_range_batch(impl):
     abi.set_impl(impl)
