@@ -1,6 +1,6 @@
 // Launcher runtime shared by every operator in the library: per-thread call
-// state (stream, argument extents, error text), per-device scratch memory and
-// staging of host buffers through device memory.
+// state (stream, argument extents, error text), scratch memory per thread and
+// device, and staging of host buffers through device memory.
 //
 // Replaces the reference's HIP "context" (mobula/cpp/include/context/hip_ctx.h:
 // 36-106): that one creates, synchronises and destroys a stream around every
@@ -22,6 +22,7 @@ struct CallState {
   bool synchronous = true;          // wait for completion before returning
   std::vector<long long> extents;   // element count per argument, -1 = unknown
   std::string error;                // empty = no error
+  bool used_workspace = false;      // the call took the scratch buffer (see workspace())
 };
 
 CallState& call_state();
@@ -34,8 +35,11 @@ inline bool failed() { return !call_state().error.empty(); }
 // finish_call().
 long long arg_extent(int index);
 
-// Grow-only scratch buffer of the current device.  The pointer stays valid
-// until a later call asks for more bytes on the same device.
+// Grow-only scratch buffer of the calling thread on the current device, for
+// work on the call's stream.  The pointer stays valid until a later call of the
+// thread asks for more bytes on the same device.  A thread that changes streams
+// between asynchronous calls is ordered behind its previous call; every entry
+// point ends with finish_call(), which keeps the book for that.
 void* workspace(size_t bytes);
 
 long long option(const char* name, long long fallback);
@@ -81,6 +85,9 @@ void finish_call();
 class SideStream {
  public:
   explicit SideStream(hipStream_t main);
+  ~SideStream();                       // joins if join() was not reached
+  SideStream(const SideStream&) = delete;
+  SideStream& operator=(const SideStream&) = delete;
   hipStream_t get() const { return side_; }
   void join();
 

@@ -31,28 +31,56 @@ long long arg_extent(int index) {
 }
 
 namespace {
-struct Scratch { void* ptr = nullptr; size_t bytes = 0; };
+// One scratch buffer per calling thread and device: calls of different threads
+// never share one.  Calls of one thread are ordered by their stream; when a
+// thread moves to another stream while the buffer may still be in use on the
+// previous one (asynchronous calls), the new stream waits for `idle`.
+struct Scratch {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  hipStream_t last = nullptr;   // stream of the last call that used the buffer
+  hipEvent_t idle = nullptr;    // recorded behind that call when it did not wait itself
+  bool busy = false;            // `idle` is recorded and not known to have passed
+};
+struct ScratchOfThread {
+  std::map<int, Scratch> per_device;
+  ~ScratchOfThread() {
+    for (auto& it : per_device) {
+      if (it.second.ptr != nullptr) (void)hipFree(it.second.ptr);
+      if (it.second.idle != nullptr) (void)hipEventDestroy(it.second.idle);
+    }
+  }
+};
+Scratch* scratch_of_current_device() {
+  static thread_local ScratchOfThread mine;
+  int device = 0;
+  MOBULA_HIP_TRY(hipGetDevice(&device));
+  return failed() ? nullptr : &mine.per_device[device];
+}
 std::mutex g_mutex;
-std::map<int, Scratch> g_scratch;
 std::map<std::string, long long> g_options;
 }  // namespace
 
 void* workspace(size_t bytes) {
-  int device = 0;
-  MOBULA_HIP_TRY(hipGetDevice(&device));
-  if (failed()) return nullptr;
-  std::lock_guard<std::mutex> lock(g_mutex);
-  Scratch& s = g_scratch[device];
-  if (s.bytes < bytes) {
-    if (s.ptr != nullptr) MOBULA_HIP_TRY(hipFree(s.ptr));  // waits for pending work
-    s.ptr = nullptr;
-    s.bytes = 0;
-    size_t want = bytes + bytes / 4 + (1u << 20);
-    MOBULA_HIP_TRY(hipMalloc(&s.ptr, want));
-    if (failed()) { s.ptr = nullptr; return nullptr; }
-    s.bytes = want;
+  Scratch* const s = scratch_of_current_device();
+  if (s == nullptr) return nullptr;
+  CallState& st = call_state();
+  if (s->busy && s->last != st.stream) {
+    MOBULA_HIP_TRY(hipStreamWaitEvent(st.stream, s->idle, 0));
+    if (failed()) return nullptr;
   }
-  return s.ptr;
+  if (s->bytes < bytes) {
+    if (s->ptr != nullptr) MOBULA_HIP_TRY(hipFree(s->ptr));  // waits for pending work
+    s->ptr = nullptr;
+    s->bytes = 0;
+    size_t want = bytes + bytes / 4 + (1u << 20);
+    MOBULA_HIP_TRY(hipMalloc(&s->ptr, want));
+    if (failed()) { s->ptr = nullptr; return nullptr; }
+    s->bytes = want;
+  }
+  s->last = st.stream;
+  st.used_workspace = true;
+  return s->ptr;
 }
 
 long long option(const char* name, long long fallback) {
@@ -148,6 +176,13 @@ SideStream::SideStream(hipStream_t main) : main_(main), side_(main) {
   joined_ = st.join;
 }
 
+SideStream::~SideStream() {
+  // a path that left early: the caller's stream still has to wait for the helpers
+  if (side_ != main_ && (hipEventRecord(joined_, side_) != hipSuccess ||
+                         hipStreamWaitEvent(main_, joined_, 0) != hipSuccess))
+    (void)hipGetLastError();
+}
+
 void SideStream::join() {
   if (side_ == main_) return;
   MOBULA_HIP_TRY(hipEventRecord(joined_, side_));
@@ -192,6 +227,23 @@ KernelTimer::~KernelTimer() {
 void finish_call() {
   CallState& st = call_state();
   if (st.synchronous && !failed()) MOBULA_HIP_TRY(hipStreamSynchronize(st.stream));
+  if (st.used_workspace) {
+    st.used_workspace = false;
+    Scratch* const s = scratch_of_current_device();
+    if (s != nullptr) {
+      s->busy = false;
+      if (!st.synchronous) {   // the buffer stays in use until the stream gets here
+        if (s->idle == nullptr && hipEventCreateWithFlags(&s->idle, hipEventDisableTiming) != hipSuccess)
+          s->idle = nullptr;
+        if (s->idle != nullptr && hipEventRecord(s->idle, st.stream) == hipSuccess) {
+          s->busy = true;
+        } else {               // no event: wait here instead
+          (void)hipGetLastError();
+          MOBULA_HIP_TRY(hipStreamSynchronize(st.stream));
+        }
+      }
+    }
+  }
   st.extents.clear();
 }
 

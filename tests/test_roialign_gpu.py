@@ -268,6 +268,46 @@ def test_double_instantiation(S):
                                   oracle.forward_f64(xh, rh, pooled, scale, S))
 
 
+def test_asynchronous_calls_on_two_streams_and_two_threads():
+    """The library's scratch memory (the blocked copy of the map, the backward's
+    lists) belongs to the calling thread: a thread that moves to another stream is
+    ordered behind its own previous call, and two threads never share a buffer."""
+    import threading
+    cases = []
+    for k, (cfg, down) in enumerate([('cfg2', 16), ('cfg1', 8)]):
+        w = workloads.make_workload(cfg, scale_down=down)
+        want = oracle.forward(w['data'], w['rois'], w['pooled_size'], w['spatial_scale'], w['sampling_ratio'])
+        want_dx = oracle.backward(w['dy'], w['rois'], w['data'].shape, w['spatial_scale'],
+                                  w['sampling_ratio'], impl='ordered')
+        cases.append((w, abi.to_dev(w['data']), abi.to_dev(w['rois']), abi.to_dev(w['dy']), want, want_dx))
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+
+    def run(order, out):
+        for k in order:   # back to back, nothing waits in between
+            w, x, rois, dy, _, _ = cases[k]
+            s = streams[k].cuda_stream
+            y = abi.forward(x, rois, w['pooled_size'], w['spatial_scale'], w['sampling_ratio'], stream=s)
+            dx = abi.backward(dy, rois, x.shape, w['spatial_scale'], w['sampling_ratio'], assign=True, stream=s)
+            out.append((k, y, dx))
+
+    # one thread, alternating streams
+    got = []
+    run([0, 1, 0, 1, 1, 0], got)
+    torch.cuda.synchronize()
+    # two threads at once, one stream each
+    per_thread = [[], []]
+    threads = [threading.Thread(target=run, args=([k] * 4, per_thread[k])) for k in (0, 1)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    for k, y, dx in got + per_thread[0] + per_thread[1]:
+        assert_parity(y.cpu().numpy(), cases[k][4], FWD_TOL, 'fwd')
+        assert_parity(dx.cpu().numpy(), cases[k][5], BWD_TOL, 'bwd')
+
+
 @pytest.mark.parametrize('impl', IMPLS)
 def test_empty_roi_list_and_out_of_range_batch(impl):
     abi.set_impl(impl)
