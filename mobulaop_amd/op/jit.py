@@ -14,6 +14,7 @@ import ctypes
 import hashlib
 import os
 import shutil
+import stat
 import subprocess
 
 from ..config import config
@@ -95,14 +96,18 @@ def wrapper_source(cfunc, arg_types, source, symbol, include=None):
 
 
 def _build_dir(source):
-    path = os.path.join(os.path.dirname(os.path.abspath(source)), 'build')
+    here = os.path.dirname(os.path.abspath(source))
+    path = os.path.join(here, 'build')
+    # beside the source only if that directory is marked writable for its owner:
+    # os.access() says yes to root for a tree that was deliberately made read-only
     try:
-        os.makedirs(path, exist_ok=True)
-        if os.access(path, os.W_OK):
+        if os.stat(here).st_mode & stat.S_IWUSR and os.access(here, os.W_OK):
+            os.makedirs(path, exist_ok=True)
             return path
     except OSError:
         pass
-    path = os.path.join(os.path.expanduser('~'), '.cache', 'mobulaop_amd', 'jit')
+    path = os.environ.get('MOBULA_JIT_CACHE') or os.path.join(os.path.expanduser('~'), '.cache',
+                                                               'mobulaop_amd', 'jit')
     os.makedirs(path, exist_ok=True)
     return path
 

@@ -97,3 +97,23 @@ def test_user_operator_class_through_autograd(axpy_ops):
     assert float((y - (3 * x + b)).detach().abs().max()) <= 1e-6
     y.backward(torch.ones_like(y))
     assert float((x.grad - 3).abs().max()) <= 1e-6 and float((b.grad - 1).abs().max()) <= 1e-6
+
+
+def test_build_directory_is_never_created_in_a_read_only_source_tree(tmp_path, monkeypatch):
+    """A source directory without the owner's write bit is left alone even when the
+    process could write there (root): the shared objects go to the cache instead."""
+    import stat
+    from mobulaop_amd.op import jit
+    src_dir = tmp_path / 'readonly' / 'Op'
+    src_dir.mkdir(parents=True)
+    (src_dir / 'Op.cpp').write_text('// empty\n')
+    src_dir.chmod(stat.S_IRUSR | stat.S_IXUSR | stat.S_IRGRP | stat.S_IXGRP)
+    monkeypatch.setenv('MOBULA_JIT_CACHE', str(tmp_path / 'cache'))
+    try:
+        chosen = jit._build_dir(str(src_dir / 'Op.cpp'))
+        assert chosen == str(tmp_path / 'cache')
+        assert not (src_dir / 'build').exists()
+    finally:
+        src_dir.chmod(stat.S_IRWXU)
+    # a writable source directory still gets its build/ beside the source
+    assert jit._build_dir(str(src_dir / 'Op.cpp')) == str(src_dir / 'build')
