@@ -236,6 +236,9 @@ double mobula_hip_last_kernel_ms(const char** name);
 
 int mobula_hip_device_count(void);
 
+/* 1 if a kernel may dereference p (device, pinned or managed memory), else 0. */
+int mobula_hip_device_can_read(const void* p);
+
 /* Space-separated list of the operator entry points in this build. */
 const char* mobula_hip_exports(void);
 

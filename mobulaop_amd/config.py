@@ -13,6 +13,11 @@ class _Defaults:
     OFFLOAD_ARCH = 'gfx950'
     DEBUG = False
     SHOW_BUILDING_COMMAND = False
+    # Where operator sources compiled on load keep their shared objects: beside the
+    # source (`<operator>/build/`) or, with BUILD_IN_LOCAL_PATH False, under
+    # `<BUILD_PATH>/build/<operator>_<hash of its parent directory>/`.
+    BUILD_PATH = './'
+    BUILD_IN_LOCAL_PATH = True
     # Device used to execute calls whose tensors live in host memory.
     HOST_STAGING_DEVICE = 0
     # Kept for source compatibility with scripts that set them; the HIP path

@@ -298,6 +298,21 @@ double mobula_hip_last_kernel_ms(const char** name) {
   return ms;
 }
 
+// 1 if a kernel may dereference p: device memory, or host memory the device
+// reaches (pinned, managed); 0 for ordinary host memory and for null.
+int mobula_hip_device_can_read(const void* p) {
+  if (p == nullptr) return 0;
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeHost ||
+                 attr.type == hipMemoryTypeManaged
+             ? 1
+             : 0;
+}
+
 int mobula_hip_device_count(void) {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess) return 0;

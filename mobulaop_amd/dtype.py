@@ -55,6 +55,26 @@ class DType:
         return self.ctype(value)
 
 
+class CStruct:
+    """A pointer to a user structure registered with `mobula.glue.register_cstruct`
+    (reference: mobula/internal/dtype.py:71-80).  The argument a caller passes is
+    turned into the ctypes structure by `constructor`."""
+
+    def __init__(self, name, is_const, cstruct, constructor):
+        self.name = name
+        self.cname = name + '*'     # constness is not part of the name, as in the reference
+        self.cstruct = cstruct
+        self.constructor = constructor
+        self.is_pointer = True
+        self.is_const = is_const
+
+    def __repr__(self):
+        return self.cname
+
+    def __call__(self, *args, **kwargs):
+        return self.constructor(*args, **kwargs)
+
+
 class TemplateType:
     """An argument whose type is a template parameter (`T`, `const T*`, ...)."""
 

@@ -23,7 +23,7 @@ import warnings
 from . import glue
 from . import native
 from .config import config
-from .dtype import DType, TemplateType, UnknownCType
+from .dtype import CStruct, DType, TemplateType, UnknownCType
 
 __all__ = ['MobulaFunc', 'CFuncDef', 'bind', 'get_func_idcode', 'get_idcode_hash']
 
@@ -44,6 +44,30 @@ class _TensorArg:
         self.var = var
         self.ptype = ptype
         self.view = view  # glue Tensor wrapper
+
+
+class _StructArg:
+    """A registered structure, passed by address."""
+    __slots__ = ('value',)
+
+    def __init__(self, value):
+        self.value = value
+
+
+def _pointer_fields(value):
+    """(field path, address) of every non-null pointer field of a ctypes structure,
+    nested structures included."""
+    for name, ftype in getattr(value, '_fields_', ()):
+        field = getattr(value, name)
+        if isinstance(field, ctypes.Structure):
+            for sub, addr in _pointer_fields(field):
+                yield name + '.' + sub, addr
+        elif isinstance(field, ctypes._Pointer):
+            addr = ctypes.cast(field, ctypes.c_void_p).value
+            if addr:
+                yield name, addr
+        elif ftype is ctypes.c_void_p and field:
+            yield name, int(field)
 
 
 class CFuncDef:
@@ -78,6 +102,18 @@ class CFuncDef:
                         copy_back.append((arg.var, dense))
                 raw.append(ptr)
                 extents.append(int(arg.view.numel))
+            elif isinstance(arg, _StructArg):
+                if self.func_kind == CFuncDef.KERNEL:
+                    # the kernel reads the structure's copy on the GPU and follows its pointers there
+                    for path, addr in _pointer_fields(arg.value):
+                        if not native.device_can_read(addr):
+                            raise TypeError(
+                                '{}: field `{}` of the structure argument points to ordinary host memory, '
+                                'which a kernel cannot read; build the structure from a GPU tensor'.format(
+                                    self.func_name, path))
+                keep_alive.append(arg.value)
+                raw.append(ctypes.byref(arg.value))
+                extents.append(1)
             else:
                 raw.append(arg)
                 extents.append(-1)
@@ -90,7 +126,14 @@ class CFuncDef:
             out = cfunc(ctypes.c_int(-1 if dev_id is None else dev_id), *raw)
             native.end_call(self.func_name)
         elif self.func_kind == CFuncDef.FUNC:
+            # a host function; if it launches kernels itself they go to the tensors'
+            # stream, and what it reports as fatal is raised here
+            stream = None
+            if dev_id is not None and glue_mod is not None and hasattr(glue_mod, 'current_stream'):
+                stream = glue_mod.current_stream(dev_id)
+            native.begin_call(stream=stream, extents=extents)
             out = cfunc(*raw)
+            native.end_call(self.func_name)
         else:
             raise TypeError('Unsupported func kind: {}'.format(self.func_kind))
         for target, dense in copy_back:
@@ -121,6 +164,17 @@ class MobulaFunc:
         glue_mod = self._common_glue(args)
         try:
             for var, ptype in zip(args, decl.arg_types):
+                if isinstance(ptype, CStruct):
+                    if isinstance(var, ptype.cstruct):
+                        value = var
+                    else:
+                        try:
+                            value = ptype.constructor(var)
+                        except TypeError:
+                            value = ptype.constructor(*var)
+                    arg_datas.append(_StructArg(value))
+                    arg_types.append(ptype)
+                    continue
                 if ptype.is_pointer and not (isinstance(ptype, DType) and
                                              ptype.ctype is ctypes.c_void_p):
                     data, var_dev, ctype = self._tensor_info(var, ptype, template_map)

@@ -2,6 +2,6 @@
 NumPy op object (reference: mobula/glue/__init__.py:1-4)."""
 from . import common
 from . import backend
-from .common import register, CUSTOM_OP_LIST
+from .common import register, register_cstruct, CUSTOM_OP_LIST
 
 common.backend = backend

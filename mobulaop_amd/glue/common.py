@@ -14,6 +14,18 @@ import numpy as np
 from ..dtype import c_half
 
 CUSTOM_OP_LIST = {}
+CSTRUCT_CONSTRUCTOR = {}  # structure name in operator sources -> (ctypes.Structure class, constructor)
+
+
+def register_cstruct(name, cstruct, constructor=None):
+    """Let operator sources loaded from now on take `name*` parameters: a call passes
+    either what `constructor` accepts (default: the structure class itself) or a tuple
+    of its positional arguments (reference: mobula/glue/common.py:197-202)."""
+    if constructor is None:
+        constructor = cstruct
+    assert callable(constructor), 'constructor {} should be callable'.format(name)
+    CSTRUCT_CONSTRUCTOR[name] = (cstruct, constructor)
+
 OP_MODULE_GLOBALS = None  # set to mobula.op's namespace when that package is imported
 backend = None            # set by glue/__init__.py
 

@@ -31,6 +31,7 @@ class KernelCall {
       st.stream = saved_stream_;
       st.extents.clear();
     } else {
+      if (copies_ && !mobula_hip::failed()) stage_.flush(st.stream);   // structures come back
       mobula_hip::finish_call();
     }
   }
@@ -53,6 +54,27 @@ class KernelCall {
     return static_cast<T*>(dev);
   }
 
+  // A structure the caller passes by address (host memory, whatever the device
+  // id): the kernel gets a copy in device memory, and the caller's structure is
+  // updated from it afterwards.  Pointers inside it are used as they are.
+  template <typename T>
+  T* struct_arg(T* p) {
+    if (p == nullptr || !ok()) return p;
+    typedef typename std::remove_const<T>::type M;
+    copies_ = true;
+    return static_cast<T*>(stage_.inout(const_cast<M*>(p), sizeof(T), /*upload=*/true));
+  }
+
+  // kernel<<<one workgroup of 1024 threads>>>(args...): for kernels whose threads
+  // synchronise with each other (Reduce, __syncthreads).
+  template <typename Kernel, typename... Args>
+  void launch_together(long long n, Kernel kernel, Args... args) {
+    if (!ok() || n <= 0) return;
+    hipLaunchKernelGGL(kernel, dim3(1), dim3(1024), 0, mobula_hip::call_state().stream, args...);
+    const hipError_t status = hipGetLastError();
+    if (status != hipSuccess) mobula_hip::set_error("%s: launch failed: %s", name_, hipGetErrorString(status));
+  }
+
   // kernel<<<blocks of 256 threads for n iterations>>>(args...) on the call's stream.
   template <typename Kernel, typename... Args>
   void launch(long long n, Kernel kernel, Args... args) {
@@ -73,9 +95,73 @@ class KernelCall {
  private:
   const char* name_;
   bool host_;
+  bool copies_ = false;
   mobula_hip::DeviceScope scope_;
   mobula_hip::HostStaging stage_;
   hipStream_t saved_stream_ = nullptr;
 };
 
+// True if a kernel may dereference `p`: null, device memory, or host memory the
+// device can reach (pinned or managed).  Ordinary host memory is refused: a
+// kernel that touched it would fault.
+template <typename T>
+bool device_can_read(T* p) {
+  if (p == nullptr) return true;
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeHost ||
+         attr.type == hipMemoryTypeManaged;
+}
+template <typename T>
+bool device_can_read(T) { return true; }   // passed by value
+
 }  // namespace mobula_jit
+
+// KERNEL_RUN(kernel)(n, args...) in a host function of an operator source
+// (reference: context/hip_ctx.h:62-106): launches over n iterations on the
+// calling thread's stream and waits, as the reference does.  Every pointer
+// argument must be memory the device can reach; otherwise nothing is launched
+// and the call fails with an error.
+namespace mobula {
+template <typename Kernel>
+class KernelRunner {
+ public:
+  explicit KernelRunner(Kernel kernel, void* stream = nullptr) : kernel_(kernel), stream_(stream) {}
+  template <typename... Args>
+  void operator()(const int n, Args... args) {
+    if (mobula_hip::failed() || n <= 0) return;
+    const bool reachable = (mobula_jit::device_can_read(args) && ...);
+    if (!reachable) {
+      mobula_hip::set_error("KERNEL_RUN: a pointer argument is ordinary host memory; pass device tensors");
+      return;
+    }
+    int cus = 0, device = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    const hipStream_t stream = stream_ != nullptr ? static_cast<hipStream_t>(stream_)
+                                                  : mobula_hip::call_state().stream;
+    const long long blocks = std::min<long long>((static_cast<long long>(n) + 255) / 256,
+                                                 static_cast<long long>(cus) * 8);
+    hipLaunchKernelGGL(kernel_, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, n, args...);
+    MOBULA_HIP_TRY(hipGetLastError());
+    if (!mobula_hip::failed()) MOBULA_HIP_TRY(hipStreamSynchronize(stream));
+  }
+
+ private:
+  Kernel kernel_;
+  void* stream_;
+};
+}  // namespace mobula
+
+#define KERNEL_RUN(a) (mobula::KernelRunner<decltype(&(a))>(&(a)))
+#define KERNEL_RUN_STREAM(a, strm) (mobula::KernelRunner<decltype(&(a))>(&(a), strm))
+#define KERNEL_RUN_BEGIN(device_id) \
+  {                                 \
+    mobula_hip::DeviceScope mobula_kernel_run_scope_(device_id);
+#define KERNEL_RUN_END() }

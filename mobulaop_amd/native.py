@@ -97,6 +97,14 @@ def roialign_channels_last_supported(backward, elem_bytes, channels, height, wid
                    int(pooled_size[0]), int(pooled_size[1]), int(sampling_ratio), int(num_rois)))
 
 
+def device_can_read(address):
+    """True if a kernel may dereference `address` (device, pinned or managed memory)."""
+    fn = library().mobula_hip_device_can_read
+    fn.argtypes = [ctypes.c_void_p]
+    fn.restype = ctypes.c_int
+    return bool(fn(ctypes.c_void_p(address)))
+
+
 def begin_call(stream, extents):
     lib = library()
     if stream is None:

@@ -13,12 +13,13 @@ shared object of its own, kept in `<operator directory>/build/`).
 import ctypes
 import hashlib
 import os
+import re
 import shutil
 import stat
 import subprocess
 
 from ..config import config
-from ..dtype import DType, TemplateType
+from ..dtype import CStruct, DType, TemplateType
 from ..func import CFuncDef
 from .. import native
 
@@ -41,6 +42,8 @@ def _base_name(dtype):
 
 
 def _c_type(dtype):
+    if isinstance(dtype, CStruct):
+        return dtype.name + '*'   # converts to the kernel's `const Name*` where it asks for that
     base = _base_name(dtype)
     text = _C_SPELLING.get(base, base)
     if dtype.is_const:
@@ -57,6 +60,36 @@ def _template_arguments(cfunc, arg_types):
             assert bound.setdefault(declared.tname, spelled) == spelled, TypeError(
                 'template parameter {} bound to two types'.format(declared.tname))
     return [bound[name] for name in cfunc.template_list]
+
+
+_TOGETHER_RE = re.compile(r'\b(Reduce|__syncthreads|get_num_threads|get_thread_num)\b')
+
+
+def kernel_body(text, kernel_name):
+    """The text between the braces of `MOBULA_KERNEL <kernel_name>(...) {...}`, or ''."""
+    m = re.search(r'MOBULA_KERNEL\s+' + re.escape(kernel_name) + r'\s*\(', text)
+    if m is None:
+        return ''
+    i, depth = m.end(), 1
+    while i < len(text) and depth:          # the parameter list
+        depth += {'(': 1, ')': -1}.get(text[i], 0)
+        i += 1
+    start = text.find('{', i)
+    if start < 0:
+        return ''
+    i, depth = start + 1, 1
+    while i < len(text) and depth:
+        depth += {'{': 1, '}': -1}.get(text[i], 0)
+        i += 1
+    return text[start + 1:i - 1]
+
+
+def synchronises_its_threads(source, kernel_name):
+    """True if the kernel must run as one workgroup: its body reduces over the
+    launch, uses a barrier, or deals out work by thread number itself."""
+    with open(source) as fin:
+        text = re.sub(r'//[^\n]*|/\*.*?\*/', ' ', fin.read(), flags=re.S)
+    return _TOGETHER_RE.search(kernel_body(text, kernel_name)) is not None
 
 
 def wrapper_source(cfunc, arg_types, source, symbol, include=None):
@@ -76,20 +109,31 @@ def wrapper_source(cfunc, arg_types, source, symbol, include=None):
         lines.append('  mobula_jit::KernelCall call("{}", device_id);'.format(cfunc.func_name))
         passed = []
         for i, (t, n) in enumerate(zip(arg_types, names)):
-            if t.is_pointer and _base_name(t) != 'void':
+            if isinstance(t, CStruct):
+                lines.append('  {} {}_mapped = call.struct_arg({});'.format(_c_type(t), n, n))
+                passed.append(n + '_mapped')
+            elif t.is_pointer and _base_name(t) != 'void':
                 lines.append('  {} {}_mapped = call.arg({}, {}, {});'.format(
                     _c_type(t), n, n, i, 'false' if t.is_const else 'true'))
                 passed.append(n + '_mapped')
             else:
                 passed.append(n)
-        lines.append('  call.launch({}, {}_kernel{}, {});'.format(names[0], cfunc.func_name, inst,
-                                                                 ', '.join(passed)))
+        how = 'launch_together' if synchronises_its_threads(source, cfunc.func_name + '_kernel') else 'launch'
+        lines.append('  call.{}({}, {}_kernel{}, {});'.format(how, names[0], cfunc.func_name, inst,
+                                                             ', '.join(passed)))
         lines.append('}')
     else:
+        # a host function: a failed CHECK / LOG(FATAL) becomes the call's error
         rtn = cfunc.rtn_type or 'void'
         lines.append('{} {}({}) {{'.format(rtn, symbol, params))
-        lines.append('  {}{}{}({});'.format('' if rtn == 'void' else 'return ', cfunc.func_name, inst,
-                                            ', '.join(names)))
+        lines.append('  try {')
+        lines.append('    {}{}{}({});'.format('' if rtn == 'void' else 'return ', cfunc.func_name, inst,
+                                              ', '.join(names)))
+        lines.append('  } catch (const mobula::FatalError& e) {')
+        lines.append('    mobula_hip::set_error("%s", e.what());')
+        lines.append('  }')
+        if rtn != 'void':
+            lines.append('  return {}();'.format(rtn))
         lines.append('}')
     lines.append('}  // extern "C"')
     return '\n'.join(lines) + '\n'
@@ -97,6 +141,13 @@ def wrapper_source(cfunc, arg_types, source, symbol, include=None):
 
 def _build_dir(source):
     here = os.path.dirname(os.path.abspath(source))
+    if not config.BUILD_IN_LOCAL_PATH:
+        # reference: mobula/building/build_path.py:7-20
+        tag = hashlib.md5(os.path.dirname(here).encode()).hexdigest()[:8]
+        path = os.path.normpath(os.path.join(config.BUILD_PATH, 'build',
+                                             '{}_{}'.format(os.path.basename(here), tag)))
+        os.makedirs(path, exist_ok=True)
+        return path
     path = os.path.join(here, 'build')
     # beside the source only if that directory is marked writable for its owner:
     # os.access() says yes to root for a tree that was deliberately made read-only

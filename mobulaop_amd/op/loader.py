@@ -18,7 +18,8 @@ import importlib.util
 import os
 import re
 
-from ..dtype import DType, TemplateType, CTYPENAME2CTYPE
+from ..dtype import DType, CStruct, TemplateType, CTYPENAME2CTYPE
+from ..glue.common import CSTRUCT_CONSTRUCTOR
 from ..func import CFuncDef, bind, get_func_idcode, get_idcode_hash
 from .. import native
 
@@ -68,6 +69,10 @@ def parse_parameter_decl(decl):
     ctype = CTYPENAME2CTYPE.get(type_name) or getattr(ctypes, 'c_' + type_name, None)
     if ctype is not None:
         return DType(ctypes.POINTER(ctype) if is_pointer else ctype, is_const=is_const), var_name
+    if type_name in CSTRUCT_CONSTRUCTOR:
+        assert is_pointer, Exception('a registered structure is passed by pointer: ' + decl)
+        cstruct, constructor = CSTRUCT_CONSTRUCTOR[type_name]
+        return CStruct(type_name, is_const=is_const, cstruct=cstruct, constructor=constructor), var_name
     return TemplateType(tname=type_name, is_pointer=is_pointer, is_const=is_const), var_name
 
 

@@ -117,3 +117,159 @@ def test_build_directory_is_never_created_in_a_read_only_source_tree(tmp_path, m
         src_dir.chmod(stat.S_IRWXU)
     # a writable source directory still gets its build/ beside the source
     assert jit._build_dir(str(src_dir / 'Op.cpp')) == str(src_dir / 'build')
+
+
+# ---------------------------------------------------------------------------
+# Kernels whose threads work together, structure arguments, host functions that
+# log / check / launch (tests/ops/Reductions, tests/ops/Records).
+# ---------------------------------------------------------------------------
+class Span(ctypes.Structure):
+    _fields_ = [('data', ctypes.POINTER(ctypes.c_float)), ('size', ctypes.c_int)]
+
+
+class Pair(ctypes.Structure):
+    _fields_ = [('count', ctypes.c_int), ('weight', ctypes.c_float)]
+
+
+def _span_of(tensor):
+    """Structure constructor: a view of a float32 tensor of either glue."""
+    view = mobula.glue.backend.get_var_glue(tensor).Tensor(tensor)
+    ptr = view.data_ptr
+    return Span(ctypes.cast(ptr, ctypes.POINTER(ctypes.c_float)), int(view.numel))
+
+
+@pytest.fixture(scope='module')
+def more_ops():
+    mobula.glue.register_cstruct('Span', Span, _span_of)
+    mobula.glue.register_cstruct('Pair', Pair)
+    mobula.op.load('Reductions', OPS)
+    mobula.op.load('Records', OPS)
+    return mobula.func
+
+
+_F32P, _F64P, _I32P = (ctypes.POINTER(t) for t in (ctypes.c_float, ctypes.c_double, ctypes.c_int))
+_INT = (ctypes.c_int, True)
+
+
+def _compile(funcs, name, types):
+    decl = getattr(funcs, name).func
+    symbol = get_idcode_hash(get_func_idcode(name, types))
+    source = decl.loader_kwargs['cpp_info'].cpp_fname
+    path = jit.compile_instantiation(decl, types, source, symbol)
+    assert hasattr(ctypes.CDLL(path), symbol)
+    return jit.wrapper_source(decl, types, source, symbol)
+
+
+def test_synchronising_kernels_are_launched_as_one_workgroup(more_ops):
+    # every instantiation the GPU test below calls is compiled here (no GPU needed)
+    for ptr in (_F32P, _F64P):
+        for name in ('largest', 'plain_total', 'careful_total'):
+            code = _compile(more_ops, name, _types(_INT, (ptr, True), (ptr, False)))
+            assert 'call.launch_together(' in code
+        code = _compile(more_ops, 'row_weights', _types(_INT, _INT, (ptr, True), (ptr, False), (ptr, False)))
+        assert 'call.launch_together(' in code
+    code = _compile(more_ops, 'contiguous_shares', _types(_INT, (_I32P, False), (_I32P, False)))
+    assert 'call.launch_together(' in code
+    # a kernel that only uses parfor keeps the many-workgroup launch
+    code = _compile(more_ops, 'fill', _types(_INT, (ctypes.c_float, True), (_F32P, False)))
+    assert 'call.launch(' in code and 'launch_together' not in code
+    # the text scan looks at the kernel's own body, comments excluded
+    source = more_ops.largest.func.loader_kwargs['cpp_info'].cpp_fname
+    assert jit.synchronises_its_threads(source, 'row_weights_kernel')
+    assert 'Reduce' in jit.kernel_body(open(source).read(), 'largest_kernel')
+    records = more_ops.fill.func.loader_kwargs['cpp_info'].cpp_fname
+    assert not jit.synchronises_its_threads(records, 'fill_kernel')
+
+
+def test_structures_and_host_functions(more_ops, capfd):
+    # symbol names carry `Name*` for a structure, as in the reference (internal/dtype.py:71-74)
+    decl = more_ops.span_scale.func
+    assert [repr(t) for t in decl.arg_types] == ['const int', 'Span*', 'const float']
+    code = _compile(more_ops, 'span_scale', [decl.arg_types[0], decl.arg_types[1], decl.arg_types[2]])
+    assert 'call.struct_arg(span)' in code
+    # host functions run here: a tuple is spread over the structure's constructor
+    assert more_ops.pair_total((3, 0.5)) == 3.5
+    assert more_ops.pair_total(Pair(4, 0.25)) == 4.25
+    assert 'pair of 3 and 0.5' in capfd.readouterr().out          # LOG(INFO) goes to stdout
+    assert more_ops.positive_or_fail(11) == 11
+    with pytest.raises(RuntimeError, match='need a positive value'):   # a failed CHECK: an error, not exit()
+        more_ops.positive_or_fail(-2)
+    assert more_ops.positive_or_fail(5) == 5                           # and the library is usable afterwards
+    _compile(more_ops, 'fill_with_sevens', _types(_INT, (_F32P, False)))
+
+
+@pytest.mark.gpu
+def test_reductions_run_on_the_gpu(more_ops):
+    import math
+    import torch
+    rng = np.random.default_rng(3)
+    for dtype, tol in ((torch.float32, 1e-6), (torch.float64, 1e-15)):
+        for n in (1, 63, 1024, 100003):
+            xh = rng.standard_normal(n) * 10.0 ** rng.integers(-3, 4, size=n)
+            x = torch.from_numpy(xh).to('cuda', dtype)
+            out = torch.zeros(4, device='cuda', dtype=dtype)
+            more_ops.largest(n, x, out)
+            assert float(out[0]) == float(x.max())
+            exact = math.fsum(x.double().cpu().tolist())
+            scale = float(x.abs().double().sum())
+            more_ops.careful_total(n, x, out)
+            assert abs(float(out[0]) - exact) <= tol * max(abs(exact), 1e-30) + 4 * tol * scale / max(n, 1) ** 0.5
+            more_ops.plain_total(n, x, out)
+            assert abs(float(out[0]) - exact) <= 64 * tol * scale
+            assert float(out[1]) == 0.0          # only out[0] is written
+    x = torch.randn(5, 3001, device='cuda', dtype=torch.float64) * 4
+    w = torch.empty_like(x)
+    cell = torch.zeros(1, device='cuda', dtype=torch.float64)
+    more_ops.row_weights(3001, 5, x, cell, w)
+    # against float64 arithmetic on the host (this ROCm build's float64 softmax on the
+    # GPU is itself only accurate to ~1e-8)
+    xh = x.cpu().numpy()
+    e = np.exp(xh - xh.max(axis=1, keepdims=True))
+    assert np.abs(w.cpu().numpy() - e / e.sum(axis=1, keepdims=True)).max() <= 1e-15
+    owner = torch.full((10007,), -1, device='cuda', dtype=torch.int32)
+    threads = torch.zeros(1, device='cuda', dtype=torch.int32)
+    more_ops.contiguous_shares(10007, owner, threads)
+    t = int(threads[0])
+    assert t == 1024
+    share, extra = divmod(10007, t)
+    want = np.repeat(np.arange(t), [share + (k < extra) for k in range(t)])
+    np.testing.assert_array_equal(owner.cpu().numpy(), want)
+    # host arrays go through the staging copies like any other kernel
+    xh = rng.standard_normal(777).astype(np.float32)
+    out = np.zeros(2, dtype=np.float32)
+    more_ops.largest(777, xh, out)
+    assert out[0] == xh.max()
+
+
+@pytest.mark.gpu
+def test_structures_and_host_launches_on_the_gpu(more_ops):
+    import torch
+    x = torch.arange(1000, device='cuda', dtype=torch.float32)
+    more_ops.span_scale(1, x, 3.0)                     # the constructor builds the Span from the tensor
+    assert torch.equal(x, torch.arange(1000, device='cuda', dtype=torch.float32) * 3)
+    # a structure that points into ordinary host memory never reaches a kernel
+    with pytest.raises(TypeError, match='host memory'):
+        more_ops.span_scale(1, np.ones(8, dtype=np.float32), 2.0)
+    out = torch.zeros(4099, device='cuda')
+    more_ops.fill_with_sevens(out.numel(), out)        # KERNEL_RUN inside a host function
+    assert float(out.min()) == 7.0 == float(out.max())
+    with pytest.raises(RuntimeError, match='host memory'):
+        more_ops.fill_with_sevens(8, np.zeros(8, dtype=np.float32))
+    more_ops.fill_with_sevens(out.numel(), out)
+
+
+def test_build_path_configuration(axpy_ops, tmp_path):
+    """BUILD_IN_LOCAL_PATH False sends the shared objects to BUILD_PATH/build/<operator>_<hash>/
+    (reference behaviour: tests/test_building/test_building.py:47-67)."""
+    source = axpy_ops.axpy.func.loader_kwargs['cpp_info'].cpp_fname
+    local = jit._build_dir(source)
+    assert local == os.path.join(os.path.dirname(source), 'build')
+    with mobula.config.TempConfig(BUILD_PATH=str(tmp_path), BUILD_IN_LOCAL_PATH=False):
+        moved = jit._build_dir(source)
+        assert moved.startswith(os.path.join(str(tmp_path), 'build', 'Axpy_')) and os.path.isdir(moved)
+        types = _types((ctypes.c_int, True), (ctypes.c_int, True))
+        decl = axpy_ops.padded_length.func
+        symbol = get_idcode_hash(get_func_idcode('padded_length', types))
+        path = jit.compile_instantiation(decl, types, source, symbol)
+        assert os.path.dirname(path) == moved and hasattr(ctypes.CDLL(path), symbol)
+    assert jit._build_dir(source) == local
