@@ -84,7 +84,7 @@ void finish_call();
 // 0 (or if the stream cannot be created) get() is the caller's stream itself.
 class SideStream {
  public:
-  explicit SideStream(hipStream_t main);
+  explicit SideStream(hipStream_t main, bool wanted = true);   // !wanted: get() is `main`
   ~SideStream();                       // joins if join() was not reached
   SideStream(const SideStream&) = delete;
   SideStream& operator=(const SideStream&) = delete;

@@ -153,8 +153,8 @@ ExportRegistrar::ExportRegistrar(const char* names) {
   export_list() += names;
 }
 
-SideStream::SideStream(hipStream_t main) : main_(main), side_(main) {
-  if (option("side_stream", 1) == 0) return;
+SideStream::SideStream(hipStream_t main, bool wanted) : main_(main), side_(main) {
+  if (!wanted || option("side_stream", 1) == 0) return;
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return;
   SideState& st = side_state(device);

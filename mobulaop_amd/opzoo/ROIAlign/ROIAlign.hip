@@ -25,6 +25,11 @@ using mobula_hip::set_error;
 
 enum Impl { kAuto = 0, kTiled = 1, kNaive = 2 };
 
+// Helper kernels move to a second stream only above these sizes (measured: below
+// them the hand-over costs more than the overlap gains).
+constexpr int kSideStreamRois = 4096;
+constexpr long long kSideStreamBytes = 64ll << 20;
+
 struct Problem {
   long long n_out;  // R*C*PH*PW
   int R, C, H, W, PH, PW, S;
@@ -159,7 +164,9 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
     T* const xt = reinterpret_cast<T*>(ws);
     int* const order = reinterpret_cast<int*>(ws + xt_bytes);
     // the ROI ordering (one small workgroup) runs beside the transposition
-    mobula_hip::SideStream side(stream);
+    // (handing work to a second stream and waiting for it costs 10-15 us: only
+    // worth it when the ordering of many ROIs would otherwise delay the gather)
+    mobula_hip::SideStream side(stream, p.R > kSideStreamRois);
     roialign::roi_order_kernel<<<1, 1024, 0, side.get()>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
     const dim3 tgrid(static_cast<unsigned>((pixels + 63) / 64), static_cast<unsigned>(cblk),
                      static_cast<unsigned>(p.N));
@@ -297,8 +304,9 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     MOBULA_HIP_TRY(hipGetLastError());
     return;
   }
-  // the pre-pass (small, latency-bound kernels) runs beside the dy transposition
-  mobula_hip::SideStream side(stream);
+  // the pre-pass (small, latency-bound kernels) runs beside the dy transposition,
+  // when that is long enough to hide it
+  mobula_hip::SideStream side(stream, static_cast<long long>(sizeof(T)) * p.n_out >= kSideStreamBytes);
   if (use_tiled() && roialign::backward_blocked_supports(p.PH, p.PW, p.S) &&
       plan_tiles(p, rois, roialign::kTileRows, BB::TW, /*with_dyb=*/true, side.get(), &plan)) {
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
