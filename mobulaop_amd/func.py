@@ -37,6 +37,20 @@ def get_idcode_hash(idcode):
     return '{}_{}'.format(func_name, hashlib.md5(signature.encode('utf-8')).hexdigest()[:8])
 
 
+_DTYPES = {}
+
+
+def _dtype(ctype, is_const):
+    """The one DType instance for (ctype, constness): descriptors are immutable, and
+    sharing them lets a call's resolved symbol be looked up by the identity of its
+    argument types."""
+    key = (ctype, is_const)
+    found = _DTYPES.get(key)
+    if found is None:
+        found = _DTYPES[key] = DType(ctype, is_const=is_const)
+    return found
+
+
 class _TensorArg:
     __slots__ = ('var', 'ptype', 'view')
 
@@ -86,10 +100,18 @@ class CFuncDef:
         self.template_defaults = template_defaults or {}   # `typename B = T` -> {'B': 'T'}
         self.loader = loader
         self.loader_kwargs = loader_kwargs or {}
+        self._resolved = {}
 
     def __call__(self, arg_datas, arg_types, dev_id, glue_mod=None, using_async=False):
         ctx = 'cpu' if dev_id is None else config.GPU_BACKEND
-        cfunc = self.loader(self, arg_types, ctx, **self.loader_kwargs)
+        # the symbol of an instantiation, remembered by the (shared) type descriptors
+        key = (ctx,) + tuple(map(id, arg_types))
+        cfunc = self._resolved.get(key)
+        if cfunc is None:
+            cfunc = self.loader(self, arg_types, ctx, **self.loader_kwargs)
+            if all(_DTYPES.get((getattr(t, 'ctype', None), t.is_const)) is t or isinstance(t, CStruct)
+                   for t in arg_types):
+                self._resolved[key] = cfunc   # ids of shared descriptors never get reused
 
         keep_alive, copy_back, raw, extents = [], [], [], []
         for arg in arg_datas:
@@ -192,13 +214,13 @@ class MobulaFunc:
                     ctype.is_const = ptype.is_const
                     arg_types.append(ctype)
                 else:
-                    arg_types.append(DType(ctype, is_const=ptype.is_const))
+                    arg_types.append(_dtype(ctype, ptype.is_const))
             for i, t in enumerate(arg_types):  # template scalars: type known only now
                 if isinstance(t, UnknownCType):
                     assert t.tname in template_map, Exception(
                         'Unknown template name: {}'.format(t.tname))
                     scalar_ctype = template_map[t.tname]._type_
-                    arg_types[i] = DType(scalar_ctype, t.is_const)
+                    arg_types[i] = _dtype(scalar_ctype, t.is_const)
                     arg_datas[i] = scalar_ctype(arg_datas[i])
         except TypeError:
             raise TypeError('Unmatched parameters list of the function `{}`:\n\t{}\n\t\tvs\n\t{}'
