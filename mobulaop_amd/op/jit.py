@@ -125,6 +125,8 @@ def wrapper_source(cfunc, arg_types, source, symbol, include=None):
     else:
         # a host function: a failed CHECK / LOG(FATAL) becomes the call's error
         rtn = cfunc.rtn_type or 'void'
+        if rtn in cfunc.template_list:   # `template <typename T> MOBULA_FUNC T f(...)`
+            rtn = targs[cfunc.template_list.index(rtn)]
         lines.append('{} {}({}) {{'.format(rtn, symbol, params))
         lines.append('  try {')
         lines.append('    {}{}{}({});'.format('' if rtn == 'void' else 'return ', cfunc.func_name, inst,

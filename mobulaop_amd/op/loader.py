@@ -81,7 +81,15 @@ def parse_declaration(text):
     m = _DECL_RE.search(text)
     assert m is not None, Exception('cannot parse declaration: ' + text)
     head = m.group(1).split()
-    params = [p for p in (q.strip() for q in m.group(2).split(',')) if p]
+    # the parameter list ends at the parenthesis that closes the first one (a body
+    # on the same line may hold more)
+    inner, depth = m.group(2), 1
+    for i, ch in enumerate(inner):
+        depth += {'(': 1, ')': -1}.get(ch, 0)
+        if depth == 0:
+            inner = inner[:i]
+            break
+    params = [p for p in (q.strip() for q in inner.split(',')) if p]
     rtn_type = head[-2] if len(head) >= 2 else None
     return rtn_type, head[-1], [parse_parameter_decl(p) for p in params]
 
@@ -110,7 +118,13 @@ class OpLoader:
                 raise NameError('No function `{}` (symbol {}) in {}, current functions: {}'.format(
                     idcode, sym_name, native.LIB_PATH, native.exported_names()))
             rtn = cfunc.rtn_type
-            fn.restype = CTYPENAME2CTYPE.get(rtn, None)
+            if rtn in cfunc.template_list:   # the return type is a template parameter
+                bound = [c.ctype for d, c in zip(cfunc.arg_types, arg_types)
+                         if isinstance(d, TemplateType) and d.tname == rtn]
+                assert bound, Exception('cannot tell the return type {} of {}'.format(rtn, cfunc.func_name))
+                fn.restype = bound[0]._type_ if bound[0].__name__.startswith('LP_') else bound[0]
+            else:
+                fn.restype = CTYPENAME2CTYPE.get(rtn, None)
             _RESOLVED[key] = fn
         self.func = _RESOLVED[key]
         self.cpp_info = cpp_info

@@ -273,3 +273,120 @@ def test_build_path_configuration(axpy_ops, tmp_path):
         path = jit.compile_instantiation(decl, types, source, symbol)
         assert os.path.dirname(path) == moved and hasattr(ctypes.CDLL(path), symbol)
     assert jit._build_dir(source) == local
+
+
+# ---------------------------------------------------------------------------
+# Argument kinds of the binding on user kernels (tests/ops/Mixed), mutually
+# including files (tests/ops/Loop), rebuilds, failures, concurrent first loads.
+# The behaviours are those the reference's own loader tests exercise
+# (tests/test_func/test_func.py:44-115, tests/test_building/test_building.py,
+# tests/test_parallel/test_multiprocessing.py:21-43).
+# ---------------------------------------------------------------------------
+@pytest.fixture(scope='module')
+def mixed_ops():
+    mobula.op.load('Mixed', OPS)
+    mobula.op.load('Loop', OPS)
+    return mobula.func
+
+
+def test_host_functions_with_template_return_types_and_include_cycles(mixed_ops):
+    assert mixed_ops.loop_answer() == 1234
+    for dtype, value in ((np.float32, 5.5), (np.int32, 7), (np.float64, -0.125)):
+        src, dst = np.array([value, 1], dtype=dtype), np.zeros(2, dtype=dtype)
+        assert mixed_ops.copy_first(src, dst) == value and dst[0] == value and dst[1] == 0
+
+
+def test_mixed_kernels_compile(mixed_ops):
+    f32, i32, f64 = ctypes.c_float, ctypes.c_int, ctypes.c_double
+    _compile(mixed_ops, 'five_loops', _types(_INT, *[(_F32P, False)] * 5))
+    for scalar in (i32, f32):
+        _compile(mixed_ops, 'broadcast', _types(_INT, (scalar, True), (_F32P, False)))
+    _compile(mixed_ops, 'fill_like', _types(_INT, (f64, False), (_F64P, False)))
+    _compile(mixed_ops, 'address_of', _types(_INT, (ctypes.c_void_p, True),
+                                             (ctypes.POINTER(ctypes.c_int64), False)))
+    _compile(mixed_ops, 'product_by_atomics', _types(_INT, _INT, _INT, (_F32P, True), (_F32P, True),
+                                                     (_F32P, False)))
+    code = _compile(mixed_ops, 'ordered_steps', _types(_INT, (_I32P, False), (_I32P, False)))
+    assert 'launch_together' in code
+
+
+def test_a_changed_source_is_rebuilt_and_a_broken_one_reports_the_compiler(tmp_path):
+    op_dir = tmp_path / 'Tmp'
+    op_dir.mkdir()
+    source = op_dir / 'Tmp.cpp'
+    source.write_text('MOBULA_FUNC int tmp_value() { return 1; }\n')
+    mobula.op.load('Tmp', str(tmp_path))
+    decl = mobula.func.tmp_value.func
+    first = jit.compile_instantiation(decl, [], str(source), 'tmp_value_d41d8cd9')
+    assert ctypes.CDLL(first).tmp_value_d41d8cd9() == 1
+    assert jit.compile_instantiation(decl, [], str(source), 'tmp_value_d41d8cd9') == first   # cached
+    source.write_text('MOBULA_FUNC int tmp_value() { return 2; }\n')
+    second = jit.compile_instantiation(decl, [], str(source), 'tmp_value_d41d8cd9')
+    assert second != first and ctypes.CDLL(second).tmp_value_d41d8cd9() == 2
+    source.write_text('MOBULA_FUNC int tmp_value() { return not_declared; }\n')
+    with pytest.raises(RuntimeError, match='not_declared'):
+        jit.compile_instantiation(decl, [], str(source), 'tmp_value_d41d8cd9')
+    assert not [f for f in os.listdir(str(op_dir / 'build')) if '.tmp.' in f]   # nothing half-written stays
+
+
+_CONCURRENT_LOAD = r'''
+import ctypes, os, sys
+sys.path.insert(0, sys.argv[1])
+import mobulaop_amd as mobula
+mobula.config.BUILD_PATH = sys.argv[2]
+mobula.config.BUILD_IN_LOCAL_PATH = False
+mobula.op.load('Axpy', os.path.join(sys.argv[1], 'tests', 'ops'))
+assert mobula.func.padded_length(13, 8) == 16
+assert mobula.func.padded_length(16, 8) == 16
+print('ok')
+'''
+
+
+def test_processes_loading_the_same_operator_at_once(tmp_path):
+    """Several processes build and load one instantiation into an empty build directory at
+    the same time: each writes its own temporary file and renames it into place."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = tmp_path / 'load.py'
+    script.write_text(_CONCURRENT_LOAD)
+    procs = [subprocess.Popen([sys.executable, str(script), root, str(tmp_path / 'shared')],
+                              stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True) for _ in range(4)]
+    outs = [p.communicate(timeout=600)[0] for p in procs]
+    assert all(p.returncode == 0 for p in procs), '\n'.join(outs)
+    assert all(o.strip().endswith('ok') for o in outs)
+    built = [f for d, _, fs in os.walk(str(tmp_path / 'shared')) for f in fs if f.endswith('.so')]
+    assert len(built) == 1
+
+
+@pytest.mark.gpu
+def test_mixed_kernels_run_on_the_gpu(mixed_ops):
+    import torch
+    n = 3000
+    outs = [torch.full((m,), -1.0, device='cuda') for m in (n, n // 2, n // 3, 2 * n, 3 * n)]
+    mixed_ops.five_loops(n, *outs)
+    for out, step in zip(outs, (1, 2, 3, 2, 3)):
+        assert torch.equal(out, torch.arange(out.numel(), device='cuda', dtype=torch.float32) * step)
+    out = torch.zeros(1000, device='cuda')
+    mixed_ops.broadcast(1000, ctypes.c_int(39), out)        # S = int, T = float
+    assert float(out.min()) == 39.0 == float(out.max())
+    mixed_ops.broadcast(1000, ctypes.c_float(3.5), out)      # S = float
+    assert float(out.min()) == 3.5 == float(out.max())
+    out64 = torch.zeros(10, device='cuda', dtype=torch.float64)
+    mixed_ops.fill_like(10, 0.1, out64)                      # the scalar becomes a double
+    assert float(out64[3]) == 0.1
+    addr = torch.zeros(4, device='cuda', dtype=torch.int64)
+    mixed_ops.address_of(4, ctypes.c_void_p(123456789), addr)
+    assert addr.tolist() == [123456789] * 4
+    I = U = J = 100
+    a, b = torch.rand(I, U, device='cuda'), torch.rand(U, J, device='cuda')
+    prod = torch.zeros(I, J, device='cuda')
+    mixed_ops.product_by_atomics(U, I, J, a, b, prod)
+    want = a.double() @ b.double()
+    assert float((prod.double() - want).abs().max()) <= 1e-3
+    rounds = 10000
+    counter = torch.zeros(1, device='cuda', dtype=torch.int32)
+    steps = torch.full((rounds,), -1, device='cuda', dtype=torch.int32)
+    mixed_ops.ordered_steps(rounds, counter, steps)
+    assert int(counter[0]) == rounds
+    assert torch.equal(steps, torch.arange(rounds, device='cuda', dtype=torch.int32))
