@@ -75,98 +75,97 @@ def get_in_shape(in_data):
     return [d.shape for d in in_data]
 
 
+def _store(dst, src):
+    dst[:] = src
+
+
+def _accumulate(dst, src):
+    dst[:] += src
+
+
+_WRITERS = {'null': None, 'write': _store, 'inplace': _store, 'add': _accumulate}
+
+
 def assign(_, dst, req, src):
-    """Store `src` into `dst` according to the write request."""
-    if req == 'null':
-        return
-    if req in ('write', 'inplace'):
-        dst[:] = src
-    elif req == 'add':
-        dst[:] += src
+    """`dst` receives `src` the way the write request says (bound as a method of
+    the generated operator classes, hence the unused first parameter)."""
+    writer = _WRITERS.get(req)
+    if writer is not None:
+        writer(dst, src)
+
+
+def _required(name):
+    def missing(self):
+        raise NotImplementedError('{}.{}'.format(type(self).__name__, name))
+    return property(missing)
 
 
 class MobulaTensor:
-    """Uniform view of a framework tensor for the function binding: raw
-    pointer (plus a contiguous temporary when needed), element ctype, device."""
-    F = None
+    """What the function binding needs to know about a framework tensor; each glue
+    derives one class from this and fills in the properties:
+
+    data_ptr  raw address, or (address, contiguous temporary) for a strided tensor
+    ctype     ctypes type of one element
+    dev_id    None for host memory, else the device index
+    numel     number of elements"""
+    F = None   # the framework module (`numpy`, `torch`)
+    data_ptr, ctype, dev_id, numel = (_required(n) for n in ('data_ptr', 'ctype', 'dev_id', 'numel'))
 
     def __init__(self, tensor):
         self.tensor = tensor
 
-    @property
-    def data_ptr(self):
-        raise NotImplementedError
-
-    @property
-    def ctype(self):
-        raise NotImplementedError
-
-    @property
-    def dev_id(self):
-        raise NotImplementedError
-
-    @property
-    def numel(self):
-        raise NotImplementedError
-
 
 class MobulaOperator:
-    """Callable handle stored as `mobula.op.<Name>`.
+    """The handle stored as `mobula.op.<Name>`.
 
-    `Op(*tensors, **ctor_kwargs)` dispatches on the tensors' framework;
-    `Op[np.ndarray](**ctor_kwargs)` returns a stateful op object of that glue."""
+    `Op(*tensors, **params)` runs the operator in the framework of its tensors;
+    `Op[tensor_type](**params)` makes an operator object of that framework without
+    running it (the NumPy glue's objects have `.forward` / `.backward`)."""
 
     def __init__(self, op, name, **attrs):
-        self.op = op
-        self.name = name
-        self.attrs = attrs
+        self.op, self.name, self.attrs = op, name, attrs
+
+    def _generate(self, glue_mod, args, kwargs, **extra):
+        return backend.op_gen(glue_mod, op=self.op, name=self.name)(
+            *args, **dict(kwargs, **self.attrs, **extra))
 
     def __call__(self, *args, **kwargs):
         glue_mod = backend.get_args_glue(*args, **kwargs)
         assert glue_mod is not None, ValueError('No explict backend')
-        merged = dict(kwargs)
-        merged.update(self.attrs)
-        return backend.op_gen(glue_mod, op=self.op, name=self.name)(*args, **merged)
+        return self._generate(glue_mod, args, kwargs)
 
     def __getitem__(self, input_type):
         glue_mod = backend.get_var_type_glue(input_type)
-        assert glue_mod is not None, ValueError(
-            'The backend of {} is not found'.format(input_type))
+        assert glue_mod is not None, ValueError('The backend of {} is not found'.format(input_type))
+        return lambda *args, **kwargs: self._generate(glue_mod, args, kwargs, __input_type__=input_type)
 
-        def make(*args, **kwargs):
-            merged = dict(kwargs)
-            merged.update(self.attrs)
-            merged['__input_type__'] = input_type
-            return backend.op_gen(glue_mod, op=self.op, name=self.name)(*args, **merged)
-        return make
+
+def _publish(cls, name, attrs):
+    name = name or cls.__name__
+    if name in CUSTOM_OP_LIST:
+        warnings.warn('Duplicate operator name {}, please rename it'.format(name))
+    handle = CUSTOM_OP_LIST[name] = MobulaOperator(op=cls, name=name, **attrs)
+    if OP_MODULE_GLOBALS is not None:
+        OP_MODULE_GLOBALS[name] = handle
+    return handle
 
 
 def register(op_name=None, **attrs):
-    """`@register`, `@register('Name')` or `@register(attr=value)` on an op class."""
-    def bind(name, cls):
-        name = name or cls.__name__
-        handle = MobulaOperator(op=cls, name=name, **attrs)
-        if name in CUSTOM_OP_LIST:
-            warnings.warn('Duplicate operator name {}, please rename it'.format(name))
-        CUSTOM_OP_LIST[name] = handle
-        if OP_MODULE_GLOBALS is not None:
-            OP_MODULE_GLOBALS[name] = handle
-        return handle
-    if op_name is not None and not isinstance(op_name, str):
-        return bind(None, op_name)  # bare decorator: op_name is the class
-    return functools.partial(bind, op_name)
+    """Class decorator of operator modules: bare (`@register`), with a name
+    (`@register('Name')`) or with attributes merged into every call
+    (`@register(attr=value)`)."""
+    if isinstance(op_name, type):          # bare: the argument is the class itself
+        return _publish(op_name, None, attrs)
+    return lambda cls: _publish(cls, op_name, attrs)
 
 
-INPUT_FUNCS = dict(
-    X=property(lambda self: self.in_data),
-    Y=property(lambda self: self.out_data),
-    dX=property(lambda self: self.in_grad),
-    dY=property(lambda self: self.out_grad),
-    x=property(lambda self: self.in_data[0]),
-    y=property(lambda self: self.out_data[0]),
-    dx=property(lambda self: self.in_grad[0]),
-    dy=property(lambda self: self.out_grad[0]),
-)
+# Accessors the glues add to operator classes: X/Y/dX/dY are the lists of inputs,
+# outputs and their gradients, the lower-case names their first elements.
+_SLOTS = dict(X='in_data', Y='out_data', dX='in_grad', dY='out_grad')
+INPUT_FUNCS = {}
+for _short, _slot in _SLOTS.items():
+    INPUT_FUNCS[_short] = property(lambda self, _slot=_slot: getattr(self, _slot))
+    INPUT_FUNCS[_short.lower()] = property(lambda self, _slot=_slot: getattr(self, _slot)[0])
 
 _NP2CTYPE = {
     'int8': ctypes.c_int8, 'int16': ctypes.c_int16, 'int32': ctypes.c_int32,

@@ -22,13 +22,10 @@ def _numel(t):
 @mobula.op.register
 class Conv2D:
     def __init__(self, channels, kernel_size, strides=(1, 1), padding=(0, 0), dilation=(1, 1), groups=1):
-        self.channels = channels
-        self.kernel_size = kernel_size
-        self.strides = strides
-        self.padding = padding
-        self.dilation = dilation
-        assert groups == 1
-        self.groups = groups
+        assert groups == 1, 'grouped convolution is not provided'
+        self.channels, self.groups = channels, groups
+        self.kernel_size, self.strides = tuple(kernel_size), tuple(strides)
+        self.padding, self.dilation = tuple(padding), tuple(dilation)
 
     def _geometry(self, x_shape):
         N, C, H, W = x_shape
@@ -59,23 +56,18 @@ class Conv2D:
                                              int(dy.shape[0]), int(dy.shape[2] * dy.shape[3]), self.dX[2])
 
     def infer_shape(self, in_shape):
-        assert 2 <= len(in_shape) <= 3, \
+        """[x (N,C,H,W), weight (D,C,KH,KW), optional bias (D,)] -> y (N,D,OH,OW) with
+        O = (size + 2*pad - dilated kernel) // stride + 1 on each axis."""
+        assert len(in_shape) in (2, 3), \
             "The inputs should be feature map(NCHW layout), weight and bias(optional)"
-        assert len(in_shape[0]) == 4, "input: NCHW"
-        assert len(in_shape[1]) == 4, "weight: DCKK"
+        x, weight = in_shape[0], in_shape[1]
+        assert len(x) == 4, "input: NCHW"
+        assert len(weight) == 4, "weight: DCKK"
         assert len(in_shape) == 2 or len(in_shape[2]) == 1, "bias: D"
-        x, weight = in_shape[:2]
-        N, C, H, W = x
-        KH, KW = self.kernel_size
-
-        def out_size(size, k, pad, stride, dil):
-            k += (k - 1) * (dil - 1)
-            return (size + 2 * pad - k) // stride + 1
-        OH = out_size(H, KH, self.padding[0], self.strides[0], self.dilation[0])
-        OW = out_size(W, KW, self.padding[1], self.strides[1], self.dilation[1])
-        D = self.channels
-        assert weight[0] == D
-        assert weight[1] == C
-        assert weight[2] == KH
-        assert weight[3] == KW
-        return in_shape, [(N, D, OH, OW)]
+        expected = (self.channels, x[1]) + tuple(self.kernel_size)
+        assert tuple(weight) == expected, "weight: expected {}, got {}".format(expected, tuple(weight))
+        out = []
+        for axis in (0, 1):
+            reach = self.dilation[axis] * (self.kernel_size[axis] - 1) + 1   # extent of the dilated kernel
+            out.append((x[2 + axis] + 2 * self.padding[axis] - reach) // self.strides[axis] + 1)
+        return in_shape, [(x[0], self.channels, out[0], out[1])]
