@@ -222,7 +222,9 @@ void mobula_hip_clear_error(void);
  * everything on the caller's stream; "conv_compute": 0 (default) multiplies the
  * convolution's fp32 operands as they are, 1 rounds them to bf16 and accumulates
  * in fp32 (results about 2e-3 off), 2 splits every operand into two bf16 and
- * forms three bf16 products per multiply-add (results about 5e-6 off)).  set returns 0, or -1 for an unknown name; get
+ * forms three bf16 products per multiply-add (results about 5e-6 off);
+ * "roialign_tile_columns": 0 (default) lets the backward pass choose its tile
+ * width from the size of the map, 56 or 28 fixes it).  set returns 0, or -1 for an unknown name; get
  * returns -1 for a name never set. */
 int mobula_hip_set_option(const char* name, long long value);
 long long mobula_hip_get_option(const char* name);

@@ -1,6 +1,7 @@
 // Backward ROIAlign: tile owners accumulate in LDS, 16 bytes per lane.
 //
-// dx is cut into tiles of 16 rows x 56 columns x 32 channels, and a tile into
+// dx is cut into tiles of 16 rows x 56 columns x 32 channels (28 columns for maps
+// that would give the SIMDs too few wavefronts otherwise), and a tile into
 // bands of TH rows (TH = 1: single rows).  One workgroup owns one band, keeps
 // it in LDS as acc[row][column][channel] and is the only writer of that piece
 // of dx: no atomics anywhere and a summation order fixed by the ROI order.
@@ -27,17 +28,25 @@ namespace roialign {
 struct BwdBlocked {
   static constexpr int TH = 1;           // rows of a band = wavefronts of a workgroup
   static constexpr int BANDS = kTileRows / TH;   // bands per tile
-  static constexpr int TW = 56;          // tile columns
+  static constexpr int TW = 56;          // tile columns ...
+  static constexpr int TW_SMALL = 28;    // ... and for maps that give few tiles (see backward_tile_columns)
   static constexpr int CB = 32;          // channels per workgroup
   static constexpr int NW = TH;
   static constexpr int NT = NW * 64;
   static constexpr int CS = 36;          // floats per cell: 32 channels + 4 of padding (bank spread)
-  static constexpr int RS = TW + 2;      // cells per row: one dummy on either side
   static constexpr int G = 4;            // work entries per pipeline stage
   static constexpr int PWB = 8;          // pooled columns per turn (one per group of 8 lanes)
 };
 
 inline bool backward_blocked_supports(int PH, int PW, int S) { return lists_supported(PH, PW, S); }
+
+// Tile width for a map: narrow tiles double the number of (shorter) work lists,
+// which pays only while the wide ones would leave the SIMDs short of wavefronts
+// (measured: 2048 wavefronts 82 -> 65 us, 40000 wavefronts 222 -> 262 us).
+inline int backward_tile_columns(long long images, int H, int W, int cblk) {
+  const long long wide = images * ((H + kTileRows - 1) / kTileRows) * ((W + BwdBlocked::TW - 1) / BwdBlocked::TW);
+  return wide * kTileRows * cblk < 8192 ? BwdBlocked::TW_SMALL : BwdBlocked::TW;
+}
 
 // dy[r][c][ph][pw] -> dyb[r][cb][ph][PWp][32], zero where pw >= PW or the channel
 // does not exist.  One workgroup per (ROI, group of `per` channel blocks):
@@ -99,8 +108,8 @@ inline long long backward_blocked_grid(long long tiles, int cblk) {
 typedef int int16v __attribute__((ext_vector_type(16)));
 
 // TO is the element type of dx (float or __half; sums are formed in fp32 and
-// rounded once); channels-last tensors are fp32 only.
-template <bool NHWC, typename TO>
+// rounded once); channels-last tensors are fp32 only.  TW: tile columns.
+template <bool NHWC, typename TO, int TW>
 __global__ void __launch_bounds__(BwdBlocked::NT)
 backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
                         const WorkRange* __restrict__ ranges, const WorkEntry* __restrict__ entries,
@@ -108,7 +117,8 @@ backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
                         int W, int PH, int PW, int cblk, unsigned dyb_bytes, unsigned list_bytes,
                         int assign) {
   using K = BwdBlocked;
-  __shared__ __attribute__((aligned(16))) float acc[K::TH * K::RS * K::CS];
+  constexpr int RS = TW + 2;   // cells per row: one dummy on either side
+  __shared__ __attribute__((aligned(16))) float acc[K::TH * RS * K::CS];
 
   // Job decode.  Workgroups are dealt to the 8 XCDs round-robin, so blockIdx % 8
   // names the XCD: it takes the channel blocks b with b % 8 == xcd (their slice
@@ -136,16 +146,16 @@ backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
   const int n = static_cast<int>(tile / tg.per_image);
   const int t_in_img = static_cast<int>(tile % tg.per_image);
   const int ty = t_in_img / tg.tx, tx = t_in_img % tg.tx;
-  const int r0 = ty * kTileRows + band * K::TH, q0 = tx * K::TW;
+  const int r0 = ty * kTileRows + band * K::TH, q0 = tx * TW;
   const int c0 = cb * K::CB, nch = min(K::CB, C - c0);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // = the tile row owned
-  const int rows = min(K::TH, H - r0), cols = min(K::TW, W - q0);
+  const int rows = min(K::TH, H - r0), cols = min(TW, W - q0);
   if (wave >= rows) return;   // no barrier below: rows are independent
   const int grp = lane >> 3, quad = lane & 7;   // pooled column within a turn, channel quad
 
-  float* const row = acc + wave * (K::RS * K::CS);
-  for (int i = lane; i < K::RS * K::CS / 4; i += 64)
+  float* const row = acc + wave * (RS * K::CS);
+  for (int i = lane; i < RS * K::CS / 4; i += 64)
     reinterpret_cast<float4*>(row)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 
   const WorkRange wr = ranges[tile * kTileRows + band * K::TH + wave];
@@ -279,13 +289,17 @@ backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
   // The owner writes its row: one channel plane at a time, lanes along x.
   TO* const out = dx_any + ((static_cast<size_t>(n) * C + c0) * H + r0 + wave) * W + q0;
   const size_t plane = static_cast<size_t>(H) * W;
-  if (lane < cols) {
-    const float* const src = row + (lane + 1) * K::CS;
+  // LPC lanes per channel plane (a power of two that covers the tile's columns):
+  // 64 / LPC planes are written per step
+  constexpr int LPC = TW <= 32 ? 32 : 64, PLANES = 64 / LPC;
+  const int col = lane & (LPC - 1), first = lane / LPC;
+  if (col < cols) {
+    const float* const src = row + (col + 1) * K::CS;
     if (assign) {
-      for (int c = 0; c < nch; ++c) out[c * plane + lane] = from_float<TO>(src[c]);
+      for (int c = first; c < nch; c += PLANES) out[c * plane + col] = from_float<TO>(src[c]);
     } else {
-      for (int c = 0; c < nch; ++c)
-        out[c * plane + lane] = from_float<TO>(to_float(out[c * plane + lane]) + src[c]);
+      for (int c = first; c < nch; c += PLANES)
+        out[c * plane + col] = from_float<TO>(to_float(out[c * plane + col]) + src[c]);
     }
   }
 }

@@ -270,6 +270,15 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
 
 bool use_tiled() { return mobula_hip::option("roialign_impl", kAuto) != kNaive; }
 
+// Tile columns of the backward pass: chosen from the size of the map unless the
+// option "roialign_tile_columns" names one of the two widths (tests do).
+int tile_columns(const Problem& p) {
+  using BB = roialign::BwdBlocked;
+  const long long forced = mobula_hip::option("roialign_tile_columns", 0);
+  if (forced == BB::TW || forced == BB::TW_SMALL) return static_cast<int>(forced);
+  return roialign::backward_tile_columns(p.N, p.H, p.W, (p.C + BB::CB - 1) / BB::CB);
+}
+
 bool nhwc_backward_supported(const Problem& p) {
   return roialign::backward_blocked_supports(p.PH, p.PW, p.S) && p.C % 4 == 0 &&
          static_cast<long long>(p.R) * p.PH * p.PW * p.C * 4 < (1ll << 31);
@@ -285,9 +294,10 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
   if (p.nhwc) {
     // dy and dx are used where they lie: only the pre-pass before the tile owners
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
+    const int tw = tile_columns(p);
     if (!kFp32 || !nhwc_backward_supported(p) || reinterpret_cast<size_t>(dy) % 16 != 0 ||
         reinterpret_cast<size_t>(dx) % 16 != 0 ||
-        !plan_tiles(p, rois, roialign::kTileRows, BB::TW, /*with_dyb=*/false, stream, &plan) ||
+        !plan_tiles(p, rois, roialign::kTileRows, tw, /*with_dyb=*/false, stream, &plan) ||
         roialign::backward_blocked_grid(plan.grid.total, cblk) >= (1ll << 31)) {
       if (!failed())
         set_error("roi_align_backward_nhwc: shape C=%d pooled %dx%d sampling_ratio %d (or the type or alignment "
@@ -296,8 +306,9 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     }
     const unsigned dy_bytes = static_cast<unsigned>(sizeof(float) * p.n_out);
     mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-    roialign::backward_blocked_kernel<true, float><<<static_cast<unsigned>(
-        roialign::backward_blocked_grid(plan.grid.total, cblk)), BB::NT, 0, stream>>>(
+    const auto kernel = tw == BB::TW ? roialign::backward_blocked_kernel<true, float, BB::TW>
+                                     : roialign::backward_blocked_kernel<true, float, BB::TW_SMALL>;
+    kernel<<<static_cast<unsigned>(roialign::backward_blocked_grid(plan.grid.total, cblk)), BB::NT, 0, stream>>>(
         reinterpret_cast<const float*>(dy), reinterpret_cast<float*>(dx), plan.ranges, plan.entries, plan.lists,
         plan.grid, plan.layout, p.C, p.H, p.W, p.PH, p.PW, cblk, dy_bytes,
         static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
@@ -307,8 +318,9 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
   // the pre-pass (small, latency-bound kernels) runs beside the dy transposition,
   // when that is long enough to hide it
   mobula_hip::SideStream side(stream, static_cast<long long>(sizeof(T)) * p.n_out >= kSideStreamBytes);
+  const int tw = tile_columns(p);
   if (use_tiled() && roialign::backward_blocked_supports(p.PH, p.PW, p.S) &&
-      plan_tiles(p, rois, roialign::kTileRows, BB::TW, /*with_dyb=*/true, side.get(), &plan)) {
+      plan_tiles(p, rois, roialign::kTileRows, tw, /*with_dyb=*/true, side.get(), &plan)) {
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
     // channel blocks per workgroup of the dy transposition: what 64 KB of LDS hold, at most 4
@@ -324,7 +336,9 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
       side.join();
       {
         mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-        roialign::backward_blocked_kernel<false, T><<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
+        const auto kernel = tw == BB::TW ? roialign::backward_blocked_kernel<false, T, BB::TW>
+                                         : roialign::backward_blocked_kernel<false, T, BB::TW_SMALL>;
+        kernel<<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
             plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
             p.W, p.PH, p.PW, cblk, static_cast<unsigned>(plan.dyb_bytes),
             static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);

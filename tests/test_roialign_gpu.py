@@ -12,7 +12,7 @@ import pytest
 
 torch = pytest.importorskip('torch')
 
-from mobulaop_amd import workloads  # noqa: E402
+from mobulaop_amd import native, workloads  # noqa: E402
 from mobulaop_amd.testing import assert_parity  # noqa: E402
 from oracle import roialign as oracle  # noqa: E402
 import abi_util as abi  # noqa: E402
@@ -29,6 +29,7 @@ def _announce(request):
     print('\n[case] {}'.format(request.node.nodeid), flush=True)
     yield
     abi.set_impl('auto')
+    native.set_option('roialign_tile_columns', 0)
 
 
 @pytest.mark.parametrize('impl', IMPLS)
@@ -139,6 +140,29 @@ def test_fp16_backward(C, S):
     dx = abi.backward(abi.to_dev(dy16), abi.to_dev(rois), (N, C, H, W), scale, S, dx=abi.to_dev(base))
     assert_parity(dx.cpu().numpy().astype(np.float32),
                   (want + base.astype(np.float32)).astype(np.float16).astype(np.float32), FP16_TOL, 'accumulate')
+
+
+@pytest.mark.parametrize('columns', [56, 28])
+@pytest.mark.parametrize('cfg,down', [('cfg1', 8), ('cfg2', 16), ('cfg3', 32)])
+def test_both_tile_widths_of_the_backward(cfg, down, columns):
+    """The backward chooses 28-column tiles for small maps and 56-column ones
+    otherwise; here each width is forced on every configuration."""
+    abi.set_impl('tiled')
+    native.set_option('roialign_tile_columns', columns)
+    w = workloads.make_workload(cfg, scale_down=down)
+    scale, S = w['spatial_scale'], w['sampling_ratio']
+    rois, dy = abi.to_dev(w['rois']), abi.to_dev(w['dy'])
+    want = oracle.backward(w['dy'], w['rois'], w['data'].shape, scale, S, impl='ordered')
+    assert_parity(abi.backward(dy, rois, w['data'].shape, scale, S, assign=True).cpu().numpy(), want, BWD_TOL,
+                  'bwd assign')
+    seed = torch.ones(w['data'].shape, device='cuda')
+    assert_parity(abi.backward(dy, rois, w['data'].shape, scale, S, dx=seed).cpu().numpy(), want + 1, BWD_TOL,
+                  'bwd accumulate')
+    dy_cl = dy.permute(0, 2, 3, 1).contiguous()
+    n, c, h, wd = w['data'].shape
+    if native.roialign_channels_last_supported(True, 4, c, h, wd, w['pooled_size'], S, rois.shape[0]):
+        got = abi.backward_nhwc(dy_cl, rois, (n, h, wd, c), scale, S, assign=True).permute(0, 3, 1, 2)
+        assert_parity(got.cpu().numpy(), want, BWD_TOL, 'bwd channels-last')
 
 
 @pytest.mark.parametrize('impl', IMPLS)
