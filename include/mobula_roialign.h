@@ -115,6 +115,23 @@ void roi_align_backward_assign_7924dbc8(const int device_id, const int nthreads,
                                         const int sampling_ratio, const int num_images,
                                         unsigned short* bottom_diff, const float* bottom_rois);
 
+/* The same three with bfloat16 storage (the upper 16 bits of a binary32, passed
+ * as unsigned short; fp32 rois, fp32 arithmetic, results rounded to nearest-even). */
+void roi_align_forward_f951d439(const int device_id, const int nthreads, const unsigned short* bottom_data,
+                                const float spatial_scale, const int channels, const int height,
+                                const int width, const int pooled_height, const int pooled_width,
+                                const int sampling_ratio, const float* bottom_rois, unsigned short* top_data);
+void roi_align_backward_0c43e974(const int device_id, const int nthreads, const unsigned short* top_diff,
+                                 const float spatial_scale, const int channels, const int height,
+                                 const int width, const int pooled_height, const int pooled_width,
+                                 const int sampling_ratio, unsigned short* bottom_diff, const float* bottom_rois);
+void roi_align_backward_assign_86156afd(const int device_id, const int nthreads,
+                                        const unsigned short* top_diff, const float spatial_scale,
+                                        const int channels, const int height, const int width,
+                                        const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        unsigned short* bottom_diff, const float* bottom_rois);
+
 /* The three operations on channels-last tensors: the map as [N,H,W,C], the pooled
  * tensor as [R,PH,PW,C] (what a torch tensor in torch.channels_last format holds);
  * scalar arguments as above (channels, height, width name C, H, W).  No
@@ -133,6 +150,12 @@ void roi_align_forward_nhwc_ab78de3c(const int device_id, const int nthreads, co
                                      const int width, const int pooled_height, const int pooled_width,
                                      const int sampling_ratio, const float* bottom_rois, float* top_data);
 void roi_align_forward_nhwc_e874c59a(const int device_id, const int nthreads,
+                                     const unsigned short* bottom_data, const float spatial_scale,
+                                     const int channels, const int height, const int width,
+                                     const int pooled_height, const int pooled_width,
+                                     const int sampling_ratio, const float* bottom_rois,
+                                     unsigned short* top_data);
+void roi_align_forward_nhwc_f951d439(const int device_id, const int nthreads,   /* bfloat16 storage */
                                      const unsigned short* bottom_data, const float spatial_scale,
                                      const int channels, const int height, const int width,
                                      const int pooled_height, const int pooled_width,

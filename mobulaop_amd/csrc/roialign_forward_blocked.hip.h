@@ -151,10 +151,11 @@ struct alignas(16) RowEntry { int lo, hi; float wl, wh; };
 struct alignas(16) ColEntry { int lo, hi; float wl, wh; };
 
 // Sixteen bytes of consecutive channels as they lie in a lane's registers: four
-// fp32 or eight fp16 (kept packed; an element is widened where it is used).
+// fp32 or eight 16-bit values (kept packed; an element is widened where it is used).
 template <typename T> struct LaneData;
 template <> struct LaneData<float> { typedef float type __attribute__((ext_vector_type(4))); };
 template <> struct LaneData<__half> { typedef _Float16 type __attribute__((ext_vector_type(8))); };
+template <> struct LaneData<bfloat16> { typedef __bf16 type __attribute__((ext_vector_type(8))); };
 
 // The sixteen bytes at byte offset lane_off + row_off of a raw buffer; lane
 // offsets outside the buffer read as zero without an access.

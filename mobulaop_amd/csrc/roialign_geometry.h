@@ -71,10 +71,16 @@ __device__ __forceinline__ AxisSample axis_sample(float v, int size) {
   return s;
 }
 
+// Storage types: binary32, binary16 and bfloat16 (the upper half of a binary32);
+// arithmetic is always binary32, a result is rounded to nearest-even once.
+typedef __bf16 bfloat16;
+
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(__half v) { return __half2float(v); }
+__device__ __forceinline__ float to_float(bfloat16 v) { return static_cast<float>(v); }
 template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ __half from_float<__half>(float v) { return __float2half_rn(v); }
+template <> __device__ __forceinline__ bfloat16 from_float<bfloat16>(float v) { return static_cast<bfloat16>(v); }
 
 }  // namespace roialign

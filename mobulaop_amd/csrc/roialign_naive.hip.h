@@ -99,19 +99,21 @@ zero_words_kernel(unsigned* __restrict__ p, long long n) {
   for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0u;
 }
 
-// out[i] = in[i] (widened), and the way back, for the fp16 detour of the
+// out[i] = in[i] (widened), and the way back, for the 16-bit detour of the
 // straightforward backward kernel.
+template <typename T>
 __global__ void __launch_bounds__(256)
-widen_kernel(const __half* __restrict__ in, float* __restrict__ out, long long n) {
+widen_kernel(const T* __restrict__ in, float* __restrict__ out, long long n) {
   const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
   for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
-    out[i] = __half2float(in[i]);
+    out[i] = to_float(in[i]);
 }
+template <typename T>
 __global__ void __launch_bounds__(256)
-narrow_kernel(const float* __restrict__ in, __half* __restrict__ out, long long n) {
+narrow_kernel(const float* __restrict__ in, T* __restrict__ out, long long n) {
   const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
   for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
-    out[i] = __float2half_rn(in[i]);
+    out[i] = from_float<T>(in[i]);
 }
 
 }  // namespace roialign

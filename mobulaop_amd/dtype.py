@@ -20,6 +20,11 @@ class c_half(ctypes.c_uint16):
     added for the fp16-storage paths.  Canonical C name: `half`."""
 
 
+class c_bfloat16(ctypes.c_uint16):
+    """bfloat16 storage (the upper half of a binary32), likewise an addition.
+    Canonical C name: `bfloat16`."""
+
+
 def _sized_name(ctype):
     """C `long` types are named by their width (`int64_t`), since their ctypes
     names differ between platforms."""
@@ -37,7 +42,7 @@ def ctype_basename(ctype):
 CTYPENAME2CTYPE = dict(
     {name: getattr(ctypes, 'c_' + name) for name in
      ('bool', 'char', 'double', 'float', 'int', 'int8', 'int16', 'int32', 'int64')},
-    half=c_half, void=None)
+    half=c_half, bfloat16=c_bfloat16, void=None)
 CTYPENAME2CTYPE.update({'char*': ctypes.c_char_p, 'void*': ctypes.c_void_p, None: None})
 for _bits in (8, 16, 32, 64):   # the <cstdint> spellings
     CTYPENAME2CTYPE['int{}_t'.format(_bits)] = CTYPENAME2CTYPE.pop('int{}'.format(_bits))

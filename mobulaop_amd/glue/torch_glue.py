@@ -15,7 +15,7 @@ import torch
 
 from .common import (MobulaTensor, INPUT_FUNCS, assign, get_in_data, get_in_shape,
                      get_varnames)
-from ..dtype import c_half
+from ..dtype import c_bfloat16, c_half
 
 # int32 / float32 / float64 are the reference's (mobula/glue/torch_glue.py:6-9); the
 # other widths follow the NumPy glue
@@ -24,6 +24,7 @@ THDTYPE2CTYPE_MAP = {
     torch.float32: ctypes.c_float,
     torch.float64: ctypes.c_double,
     torch.float16: c_half,
+    torch.bfloat16: c_bfloat16,
     torch.int8: ctypes.c_int8,
     torch.int16: ctypes.c_int16,
     torch.int64: ctypes.c_int64,

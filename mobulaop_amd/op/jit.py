@@ -27,8 +27,8 @@ _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 INC_PATH = os.path.join(_PKG, 'inc')
 CSRC_PATH = os.path.join(_PKG, 'csrc')
 
-# C spelling of the element types the binding knows (`half` is storage only)
-_C_SPELLING = {'half': '__half'}
+# C spelling of the element types the binding knows (`half` and `bfloat16` are storage only)
+_C_SPELLING = {'half': '__half', 'bfloat16': '__bf16'}
 
 _loaded = {}
 

@@ -356,7 +356,7 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     sums = static_cast<float*>(mobula_hip::workspace(sizeof(float) * map));
     if (failed()) return;
     if (!assign)
-      roialign::widen_kernel<<<grid_for(map, 256), 256, 0, stream>>>(reinterpret_cast<const __half*>(dx), sums, map);
+      roialign::widen_kernel<T><<<grid_for(map, 256), 256, 0, stream>>>(dx, sums, map);
   }
   if (assign)
     roialign::zero_words_kernel<<<grid_for(map, 256), 256, 0, stream>>>(reinterpret_cast<unsigned*>(sums), map);
@@ -364,7 +364,7 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     roialign::backward_naive_kernel<T><<<grid_for(p.n_out, 256), 256, 0, stream>>>(
         p.n_out, dy, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, sums, rois, p.N);
   if (!kFp32)
-    roialign::narrow_kernel<<<grid_for(map, 256), 256, 0, stream>>>(sums, reinterpret_cast<__half*>(dx), map);
+    roialign::narrow_kernel<T><<<grid_for(map, 256), 256, 0, stream>>>(sums, dx, map);
   MOBULA_HIP_TRY(hipGetLastError());
 }
 
@@ -702,6 +702,42 @@ void roi_align_backward_assign_7924dbc8(const int device_id, const int nthreads,
                          pooled_height, pooled_width, sampling_ratio, num_images, bottom_diff, bottom_rois);
 }
 
+// The same three with bfloat16 storage.
+void roi_align_forward_f951d439(const int device_id, const int nthreads, const roialign::bfloat16* bottom_data,
+                                const float spatial_scale, const int channels, const int height,
+                                const int width, const int pooled_height, const int pooled_width,
+                                const int sampling_ratio, const float* bottom_rois,
+                                roialign::bfloat16* top_data) {
+  forward_entry<roialign::bfloat16, float>(device_id, nthreads, bottom_data, spatial_scale, channels, height,
+                                           width, pooled_height, pooled_width, sampling_ratio, bottom_rois,
+                                           top_data);
+}
+
+void roi_align_backward_0c43e974(const int device_id, const int nthreads, const roialign::bfloat16* top_diff,
+                                 const float spatial_scale, const int channels, const int height,
+                                 const int width, const int pooled_height, const int pooled_width,
+                                 const int sampling_ratio, roialign::bfloat16* bottom_diff,
+                                 const float* bottom_rois) {
+  backward_entry<roialign::bfloat16, float>(device_id, nthreads, top_diff, spatial_scale, channels, height,
+                                            width, pooled_height, pooled_width, sampling_ratio, -1, bottom_diff,
+                                            bottom_rois);
+}
+
+void roi_align_backward_assign_86156afd(const int device_id, const int nthreads,
+                                        const roialign::bfloat16* top_diff, const float spatial_scale,
+                                        const int channels, const int height, const int width,
+                                        const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        roialign::bfloat16* bottom_diff, const float* bottom_rois) {
+  if (num_images < 0) {
+    set_error("roi_align_backward_assign: num_images=%d", num_images);
+    return;
+  }
+  backward_entry<roialign::bfloat16, float>(device_id, nthreads, top_diff, spatial_scale, channels, height,
+                                            width, pooled_height, pooled_width, sampling_ratio, num_images,
+                                            bottom_diff, bottom_rois);
+}
+
 // Channels-last variants (extensions): device pointers only.
 #define MOBULA_NHWC_ENTRY(call)                                                            \
   if (device_id < 0) {                                                                     \
@@ -730,6 +766,17 @@ void roi_align_forward_nhwc_e874c59a(const int device_id, const int nthreads, co
   MOBULA_NHWC_ENTRY(roi_align_forward_nhwc_kernel<__half>(nthreads, bottom_data, spatial_scale, channels, height,
                                                           width, pooled_height, pooled_width, sampling_ratio,
                                                           bottom_rois, top_data))
+}
+
+void roi_align_forward_nhwc_f951d439(const int device_id, const int nthreads,
+                                     const roialign::bfloat16* bottom_data, const float spatial_scale,
+                                     const int channels, const int height, const int width,
+                                     const int pooled_height, const int pooled_width, const int sampling_ratio,
+                                     const float* bottom_rois, roialign::bfloat16* top_data) {
+  MOBULA_NHWC_ENTRY(roi_align_forward_nhwc_kernel<roialign::bfloat16>(nthreads, bottom_data, spatial_scale,
+                                                                      channels, height, width, pooled_height,
+                                                                      pooled_width, sampling_ratio, bottom_rois,
+                                                                      top_data))
 }
 
 void roi_align_backward_nhwc_f318a24e(const int device_id, const int nthreads, const float* top_diff,
@@ -785,6 +832,7 @@ static mobula_hip::ExportRegistrar roialign_exports(
     "roi_align_forward_ab78de3c roi_align_backward_f318a24e roi_align_backward_assign_a8793cbe "
     "roi_align_forward_6b9e6c9b roi_align_backward_2b6c6dfa roi_align_backward_assign_4620f85e "
     "roi_align_forward_e874c59a roi_align_backward_23175303 roi_align_backward_assign_7924dbc8 "
-    "roi_align_forward_nhwc_ab78de3c roi_align_forward_nhwc_e874c59a "
+    "roi_align_forward_f951d439 roi_align_backward_0c43e974 roi_align_backward_assign_86156afd "
+    "roi_align_forward_nhwc_ab78de3c roi_align_forward_nhwc_e874c59a roi_align_forward_nhwc_f951d439 "
     "roi_align_backward_nhwc_f318a24e roi_align_backward_nhwc_assign_a8793cbe "
     "mobula_hip_roialign_nhwc_supported");

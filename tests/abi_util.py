@@ -9,6 +9,12 @@ from mobulaop_amd import native
 
 IMPL = {'auto': 0, 'tiled': 1, 'naive': 2}
 
+# symbol suffixes of the storage types that take fp32 boxes: forward / forward_nhwc,
+# backward, backward_assign
+_SUFFIX = {torch.float32: ('ab78de3c', 'f318a24e', 'a8793cbe'),
+           torch.float16: ('e874c59a', '23175303', '7924dbc8'),
+           torch.bfloat16: ('f951d439', '0c43e974', '86156afd')}
+
 
 def _ptr(t):
     assert t.is_contiguous()
@@ -52,7 +58,7 @@ def forward(x, rois, pooled, scale, S, declare_extents=True, stream=None, dev=0)
                                        *_geom(scale, C, H, W, PH, PW, S, ctypes.c_double), _ptr(rois), _ptr(y))
         _end(lib)
         return y
-    fn = lib.roi_align_forward_ab78de3c if x.dtype == torch.float32 else lib.roi_align_forward_e874c59a
+    fn = getattr(lib, 'roi_align_forward_' + _SUFFIX[x.dtype][0])
     fn(ctypes.c_int(dev), ctypes.c_int(y.numel()), _ptr(x), *_geom(scale, C, H, W, PH, PW, S),
        _ptr(rois), _ptr(y))
     _end(lib)
@@ -67,7 +73,6 @@ def backward(dy, rois, shape, scale, S, dx=None, assign=False, declare_extents=T
         dx = (torch.full(shape, float('nan'), dtype=dy.dtype, device=dy.device) if assign
               else torch.zeros(shape, dtype=dy.dtype, device=dy.device))
     lib = native.library()
-    half = dy.dtype == torch.float16
     if dy.dtype == torch.float64:
         assert rois.dtype == torch.float64
         geom = _geom(scale, C, H, W, PH, PW, S, ctypes.c_double)
@@ -86,13 +91,13 @@ def backward(dy, rois, shape, scale, S, dx=None, assign=False, declare_extents=T
     if assign:
         ext = [-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()]
         _begin(ext if declare_extents else [], stream)
-        (lib.roi_align_backward_assign_7924dbc8 if half else lib.roi_align_backward_assign_a8793cbe)(
+        getattr(lib, 'roi_align_backward_assign_' + _SUFFIX[dy.dtype][2])(
             ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
             ctypes.c_int(N), _ptr(dx), _ptr(rois))
     else:
         ext = [-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()]
         _begin(ext if declare_extents else [], stream)
-        (lib.roi_align_backward_23175303 if half else lib.roi_align_backward_f318a24e)(
+        getattr(lib, 'roi_align_backward_' + _SUFFIX[dy.dtype][1])(
             ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
             _ptr(dx), _ptr(rois))
     _end(lib)
@@ -107,7 +112,7 @@ def forward_nhwc(x, rois, pooled, scale, S, dev=0, stream=None):
     y = torch.empty((R, PH, PW, C), dtype=x.dtype, device=x.device)
     ext = [-1, x.numel(), -1, -1, -1, -1, -1, -1, -1, rois.numel(), y.numel()]
     lib = _begin(ext, stream)
-    fn = lib.roi_align_forward_nhwc_ab78de3c if x.dtype == torch.float32 else lib.roi_align_forward_nhwc_e874c59a
+    fn = getattr(lib, 'roi_align_forward_nhwc_' + _SUFFIX[x.dtype][0])
     fn(ctypes.c_int(dev), ctypes.c_int(y.numel()), _ptr(x), *_geom(scale, C, H, W, PH, PW, S),
        _ptr(rois), _ptr(y))
     _end(lib)

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_symbol_names_follow_the_reference_scheme(mobula):
     from mobulaop_amd.func import get_func_idcode, get_idcode_hash
-    from mobulaop_amd.dtype import c_half
+    from mobulaop_amd.dtype import c_bfloat16, c_half
     # (function, element type T, box type B, symbol); the float and double names are
     # the reference's own (mobula/func.py:13-50 over ROIAlign.cpp:10-16, 79-83)
     cases = [('roi_align_forward', ctypes.c_float, ctypes.c_float, 'roi_align_forward_ab78de3c'),
@@ -42,7 +42,9 @@ def test_symbol_names_follow_the_reference_scheme(mobula):
              ('roi_align_backward', ctypes.c_double, ctypes.c_double, 'roi_align_backward_2b6c6dfa'),
              ('roi_align_backward_assign', ctypes.c_float, ctypes.c_float,
               'roi_align_backward_assign_a8793cbe'),
-             ('roi_align_forward', c_half, ctypes.c_float, 'roi_align_forward_e874c59a')]
+             ('roi_align_forward', c_half, ctypes.c_float, 'roi_align_forward_e874c59a'),
+             ('roi_align_forward', c_bfloat16, ctypes.c_float, 'roi_align_forward_f951d439'),
+             ('roi_align_backward_assign', c_bfloat16, ctypes.c_float, 'roi_align_backward_assign_86156afd')]
     for fname, elem, box, want in cases:
         decl = getattr(mobula.func, fname).func
         bound = {'T': elem, 'B': box}

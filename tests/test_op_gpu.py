@@ -151,24 +151,30 @@ def test_channels_last_tensors_take_the_channels_last_path(mobula):
     assert float((xa.grad - xb.grad).abs().max()) <= 1e-4 * float(xa.grad.abs().max())
 
 
-def test_half_precision_training_step(mobula):
-    # fp16 map and gradients through the operator: both passes run in the library
+@pytest.mark.parametrize('low,tol', [(torch.float16, 2e-3), (torch.bfloat16, 8e-3)])
+def test_half_precision_training_step(mobula, low, tol):
+    # 16-bit map and gradients through the operator: both passes run in the library
+    # (bfloat16 carries 8 significant bits: 4e-3 per rounding)
     torch.manual_seed(6)
     x32 = torch.randn(2, 64, 20, 24, device='cuda')
     rois = torch.tensor([[0, 1, 2, 60, 50], [1, 10, 10, 90, 70], [1, -5, 3, 20, 100]], device='cuda',
                         dtype=torch.float32)
     kw = dict(pooled_size=(7, 7), spatial_scale=0.25, sampling_ratio=2)
-    xh = x32.half().requires_grad_(True)
+    xh = x32.to(low).requires_grad_(True)
     yh = mobula.op.ROIAlign(xh, rois, **kw)
-    assert yh.dtype == torch.float16
+    assert yh.dtype == low
     dy = torch.randn_like(yh)
     yh.backward(dy)
-    assert xh.grad.dtype == torch.float16
-    xf = x32.half().float().requires_grad_(True)
+    assert xh.grad.dtype == low
+    xf = x32.to(low).float().requires_grad_(True)
     yf = mobula.op.ROIAlign(xf, rois, **kw)
     yf.backward(dy.float())
-    assert float((yh.detach().float() - yf.detach()).abs().max()) <= 2e-3 * float(yf.detach().abs().max())
-    assert float((xh.grad.float() - xf.grad).abs().max()) <= 2e-3 * float(xf.grad.abs().max())
+    assert float((yh.detach().float() - yf.detach()).abs().max()) <= tol * float(yf.detach().abs().max())
+    assert float((xh.grad.float() - xf.grad).abs().max()) <= tol * float(xf.grad.abs().max())
+    # channels-last 16-bit maps: the forward reads them where they lie
+    xc = x32.to(low).contiguous(memory_format=torch.channels_last)
+    yc = mobula.op.ROIAlign(xc, rois, **kw)
+    assert float((yc.float() - yf.detach()).abs().max()) <= tol * float(yf.detach().abs().max())
 
 
 def test_double_tensors_through_the_operator(mobula):

@@ -120,6 +120,47 @@ def test_fp16_channel_blocks(C, S):
     assert_parity(y.astype(np.float32), want.astype(np.float16).astype(np.float32), FP16_TOL, 'fp16')
 
 
+BF16_TOL = 4e-3   # a bfloat16 result carries 8 significant bits: half a unit in the last place is 2e-3
+
+
+def _round_bf16(a):
+    """float32 array -> the nearest bfloat16 values, as float32 (round to nearest even)."""
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).float().numpy()
+
+
+@pytest.mark.parametrize('S', [2, 0])
+@pytest.mark.parametrize('C', [72, 64, 20])
+def test_bfloat16_storage(C, S):
+    """bfloat16 maps and gradients (fp32 boxes, fp32 arithmetic): the checker's fp32 result on
+    the bfloat16-rounded operands, rounded to bfloat16.  NCHW and channels-last; C = 20 and the
+    S = 0 backward go through the straightforward kernels."""
+    abi.set_impl('auto')
+    rng = np.random.default_rng(500 * C + S)
+    N, H, W, R, pooled, scale = 2, 30, 44, 50, (7, 7), 0.25
+    xb = _round_bf16(rng.standard_normal((N, C, H, W)))
+    dyb = _round_bf16(rng.standard_normal((R, C) + pooled))
+    c = np.stack([rng.uniform(0, W / scale, R), rng.uniform(0, H / scale, R)], 1)
+    wh = np.stack([rng.uniform(2, W / scale, R), rng.uniform(2, H / scale, R)], 1)
+    rois = np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+    x = abi.to_dev(xb).to(torch.bfloat16)
+    dy = abi.to_dev(dyb).to(torch.bfloat16)
+    r = abi.to_dev(rois)
+    want_y = _round_bf16(oracle.forward(xb, rois, pooled, scale, S))
+    y = abi.forward(x, r, pooled, scale, S)
+    assert y.dtype == torch.bfloat16
+    assert_parity(y.float().cpu().numpy(), want_y, BF16_TOL, 'bf16 fwd')
+    if C % 8 == 0:
+        y_cl = abi.forward_nhwc(x.permute(0, 2, 3, 1).contiguous(), r, pooled, scale, S)
+        assert_parity(y_cl.permute(0, 3, 1, 2).float().cpu().numpy(), want_y, BF16_TOL, 'bf16 fwd channels-last')
+    want_dx = oracle.backward(dyb, rois, (N, C, H, W), scale, S, impl='ordered')
+    dx = abi.backward(dy, r, (N, C, H, W), scale, S, assign=True)
+    assert dx.dtype == torch.bfloat16
+    assert_parity(dx.float().cpu().numpy(), _round_bf16(want_dx), BF16_TOL, 'bf16 bwd assign')
+    base = _round_bf16(rng.standard_normal((N, C, H, W)))
+    dx = abi.backward(dy, r, (N, C, H, W), scale, S, dx=abi.to_dev(base).to(torch.bfloat16))
+    assert_parity(dx.float().cpu().numpy(), _round_bf16(want_dx + base), BF16_TOL, 'bf16 bwd accumulate')
+
+
 @pytest.mark.parametrize('S', [2, 0])
 @pytest.mark.parametrize('C', [72, 20])
 def test_fp16_backward(C, S):
