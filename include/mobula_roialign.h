@@ -170,8 +170,32 @@ void roi_align_backward_nhwc_assign_a8793cbe(const int device_id, const int nthr
                                              const int width, const int pooled_height, const int pooled_width,
                                              const int sampling_ratio, const int num_images, float* bottom_diff,
                                              const float* bottom_rois);
+/* The channels-last backward with 16-bit tensors: binary16 (23175303 / 7924dbc8) and
+ * bfloat16 (0c43e974 / 86156afd); dy and dx have the same type, sums are fp32. */
+void roi_align_backward_nhwc_23175303(const int device_id, const int nthreads, const unsigned short* top_diff,
+                                      const float spatial_scale, const int channels, const int height,
+                                      const int width, const int pooled_height, const int pooled_width,
+                                      const int sampling_ratio, unsigned short* bottom_diff,
+                                      const float* bottom_rois);
+void roi_align_backward_nhwc_assign_7924dbc8(const int device_id, const int nthreads,
+                                             const unsigned short* top_diff, const float spatial_scale,
+                                             const int channels, const int height, const int width,
+                                             const int pooled_height, const int pooled_width,
+                                             const int sampling_ratio, const int num_images,
+                                             unsigned short* bottom_diff, const float* bottom_rois);
+void roi_align_backward_nhwc_0c43e974(const int device_id, const int nthreads, const unsigned short* top_diff,
+                                      const float spatial_scale, const int channels, const int height,
+                                      const int width, const int pooled_height, const int pooled_width,
+                                      const int sampling_ratio, unsigned short* bottom_diff,
+                                      const float* bottom_rois);
+void roi_align_backward_nhwc_assign_86156afd(const int device_id, const int nthreads,
+                                             const unsigned short* top_diff, const float spatial_scale,
+                                             const int channels, const int height, const int width,
+                                             const int pooled_height, const int pooled_width,
+                                             const int sampling_ratio, const int num_images,
+                                             unsigned short* bottom_diff, const float* bottom_rois);
 /* 1 if the channels-last entry points take the shape, else 0.  backward != 0 asks
- * about the two backward entry points; elem_bytes is 4 (fp32) or 2 (fp16). */
+ * about the backward entry points; elem_bytes is 4 (fp32) or 2 (fp16, bfloat16). */
 int mobula_hip_roialign_nhwc_supported(int backward, int elem_bytes, int channels, int height, int width,
                                        int pooled_height, int pooled_width, int sampling_ratio,
                                        long long num_rois);

@@ -107,11 +107,25 @@ inline long long backward_blocked_grid(long long tiles, int cblk) {
 
 typedef int int16v __attribute__((ext_vector_type(16)));
 
-// TO is the element type of dx (float or __half; sums are formed in fp32 and
-// rounded once); channels-last tensors are fp32 only.  TW: tile columns.
+// Element i (0..3) of the four consecutive values a lane loaded: four dwords of
+// fp32, or two dwords holding four 16-bit values.
+template <typename TI>
+__device__ __forceinline__ float lane_value(const unsigned __attribute__((ext_vector_type(4)))& d, int i) {
+  if constexpr (sizeof(TI) == 4) {
+    return __uint_as_float(d[i]);
+  } else {
+    const unsigned short bits = static_cast<unsigned short>(d[i >> 1] >> (16 * (i & 1)));
+    return to_float(__builtin_bit_cast(TI, bits));
+  }
+}
+
+// TO is the element type of dx (float, __half or bfloat16; sums are formed in fp32 and
+// rounded once).  TW: tile columns.
+// dy_any: the blocked fp32 copy dyb, or for channels-last tensors the caller's
+// dy[R][PH][PW][C] itself, of dx's element type.
 template <bool NHWC, typename TO, int TW>
 __global__ void __launch_bounds__(BwdBlocked::NT)
-backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
+backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any,
                         const WorkRange* __restrict__ ranges, const WorkEntry* __restrict__ entries,
                         const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll, int C, int H,
                         int W, int PH, int PW, int cblk, unsigned dyb_bytes, unsigned list_bytes,
@@ -166,13 +180,14 @@ backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
 
   // dyb and the sample lists as raw buffers: a scalar byte offset per entry
   // plus a fixed lane offset
-  // (NHWC: dyb is the caller's dy[R][PH][PW][C] itself)
-  const unsigned dy_pw = (NHWC ? C : K::CB) * sizeof(float);
+  typedef typename std::conditional<NHWC, TO, float>::type TI;   // element type of what dy_any points to
+  constexpr unsigned E = sizeof(TI);
+  const unsigned dy_pw = (NHWC ? C : K::CB) * E;
   const unsigned dy_ph = static_cast<unsigned>(NHWC ? PW : PWp) * dy_pw;
   const unsigned dy_roi = NHWC ? dy_ph * PH : dy_ph * PH * cblk;
   const unsigned list_roi = static_cast<unsigned>(ll.roi_stride) * sizeof(AxisUnit);
   const __amdgpu_buffer_rsrc_t dy_buf = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float*>(dyb), 0, static_cast<int>(dyb_bytes), 0x00020000);
+      const_cast<void*>(dy_any), 0, static_cast<int>(dyb_bytes), 0x00020000);
   const __amdgpu_buffer_rsrc_t list_buf = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<AxisUnit*>(lists), 0, static_cast<int>(list_bytes), 0x00020000);
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -183,12 +198,12 @@ backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
   // samples of the next are in flight (always eight loads per group, so the
   // wait before a group counts exactly the loads of the group after it).
   for (int pwb = 0; pwb < PW; pwb += K::PWB) {
-    const unsigned dy_fixed = (NHWC ? cb * K::CB * sizeof(float) : cb * dy_ph * PH) + pwb * dy_pw;
+    const unsigned dy_fixed = (NHWC ? cb * K::CB * E : cb * dy_ph * PH) + pwb * dy_pw;
     const unsigned list_fixed = static_cast<unsigned>(
         (static_cast<long long>(ll.ty) * ll.row_stride + static_cast<long long>(tx) * ll.col_stride + pwb) *
         sizeof(AxisUnit));
     // a lane whose pooled column or channels do not exist loads from outside the buffer (zero, no access)
-    const int dy_lane = pwb + grp < PW && quad * 4 < nch ? static_cast<int>(grp * dy_pw) + quad * 16
+    const int dy_lane = pwb + grp < PW && quad * 4 < nch ? static_cast<int>(grp * dy_pw + quad * 4 * E)
                                                          : static_cast<int>(0x80000000u);
     // The 16-byte column sample of the lane's pooled column comes as one dword per
     // lane (lane & 3 picks it; a 4-byte load costs the texture path half of a
@@ -198,7 +213,13 @@ backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
         const unsigned roi = e[4 * j], ph = e[4 * j + 1];
-        d[j] = __builtin_amdgcn_raw_buffer_load_b128(dy_buf, dy_lane, roi * dy_roi + ph * dy_ph + dy_fixed, 0);
+        if (E == 4) {
+          d[j] = __builtin_amdgcn_raw_buffer_load_b128(dy_buf, dy_lane, roi * dy_roi + ph * dy_ph + dy_fixed, 0);
+        } else {   // four 16-bit values: eight bytes
+          typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+          const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(dy_buf, dy_lane, roi * dy_roi + ph * dy_ph + dy_fixed, 0);
+          d[j] = u32x4{w.x, w.y, 0u, 0u};
+        }
         u[j] = __builtin_amdgcn_raw_buffer_load_b32(list_buf, list_lane, roi * list_roi + list_fixed, 0);
       }
     };
@@ -222,7 +243,7 @@ backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
         const int fl = e[4 * j + 3];
         const float keep = (fl & 1) ? 1.0f : 0.0f;   // first tap of a ROI restarts the sum
 #pragma unroll
-        for (int i = 0; i < 4; ++i) g[i] = fmaf(__uint_as_float(d[j][i]), wy, keep * g[i]);
+        for (int i = 0; i < 4; ++i) g[i] = fmaf(lane_value<TI>(d[j], i), wy, keep * g[i]);
         if ((fl & 2) != 0) {
           // last tap of this ROI on this row: spread g over the column samples
           // dword k of the quad's four: quad_perm [k, k, k, k]
@@ -266,22 +287,25 @@ backward_blocked_kernel(const float* __restrict__ dyb, TO* __restrict__ dx_any,
     }
   }
 
-  if (NHWC && std::is_same<TO, float>::value) {
-    float* const dx = reinterpret_cast<float*>(dx_any);
-    // dx[n][row][col][C]: a pixel's channels of this block are 128 contiguous bytes;
+  if (NHWC) {
+    // dx[n][row][col][C]: a pixel's channels of this block are contiguous;
     // eight pixels per step, a lane moves its four channels
-    float* const px0 = dx + ((static_cast<size_t>(n) * H + r0 + wave) * W + q0) * C + c0 + quad * 4;
+    struct alignas(4 * sizeof(TO)) Four { TO v[4]; };
+    TO* const px0 = dx_any + ((static_cast<size_t>(n) * H + r0 + wave) * W + q0) * C + c0 + quad * 4;
     if (quad * 4 < nch) {
       for (int col = grp; col < cols; col += 8) {
         const float4 v = *reinterpret_cast<const float4*>(row + (col + 1) * K::CS + quad * 4);
-        float4* const dst = reinterpret_cast<float4*>(px0 + static_cast<size_t>(col) * C);
+        Four* const dst = reinterpret_cast<Four*>(px0 + static_cast<size_t>(col) * C);
+        Four o;
         if (assign) {
-          *dst = v;
+          o.v[0] = from_float<TO>(v.x); o.v[1] = from_float<TO>(v.y);
+          o.v[2] = from_float<TO>(v.z); o.v[3] = from_float<TO>(v.w);
         } else {
-          float4 o = *dst;
-          o.x += v.x; o.y += v.y; o.z += v.z; o.w += v.w;
-          *dst = o;
+          o = *dst;
+          o.v[0] = from_float<TO>(to_float(o.v[0]) + v.x); o.v[1] = from_float<TO>(to_float(o.v[1]) + v.y);
+          o.v[2] = from_float<TO>(to_float(o.v[2]) + v.z); o.v[3] = from_float<TO>(to_float(o.v[3]) + v.w);
         }
+        *dst = o;
       }
     }
     return;

@@ -295,7 +295,7 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     // dy and dx are used where they lie: only the pre-pass before the tile owners
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const int tw = tile_columns(p);
-    if (!kFp32 || !nhwc_backward_supported(p) || reinterpret_cast<size_t>(dy) % 16 != 0 ||
+    if (!nhwc_backward_supported(p) || reinterpret_cast<size_t>(dy) % 16 != 0 ||
         reinterpret_cast<size_t>(dx) % 16 != 0 ||
         !plan_tiles(p, rois, roialign::kTileRows, tw, /*with_dyb=*/false, stream, &plan) ||
         roialign::backward_blocked_grid(plan.grid.total, cblk) >= (1ll << 31)) {
@@ -304,12 +304,12 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
                   "of the tensors) is not taken by the channels-last path", p.C, p.PH, p.PW, p.S);
       return;
     }
-    const unsigned dy_bytes = static_cast<unsigned>(sizeof(float) * p.n_out);
+    const unsigned dy_bytes = static_cast<unsigned>(sizeof(T) * p.n_out);
     mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-    const auto kernel = tw == BB::TW ? roialign::backward_blocked_kernel<true, float, BB::TW>
-                                     : roialign::backward_blocked_kernel<true, float, BB::TW_SMALL>;
+    const auto kernel = tw == BB::TW ? roialign::backward_blocked_kernel<true, T, BB::TW>
+                                     : roialign::backward_blocked_kernel<true, T, BB::TW_SMALL>;
     kernel<<<static_cast<unsigned>(roialign::backward_blocked_grid(plan.grid.total, cblk)), BB::NT, 0, stream>>>(
-        reinterpret_cast<const float*>(dy), reinterpret_cast<float*>(dx), plan.ranges, plan.entries, plan.lists,
+        dy, dx, plan.ranges, plan.entries, plan.lists,
         plan.grid, plan.layout, p.C, p.H, p.W, p.PH, p.PW, cblk, dy_bytes,
         static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
     MOBULA_HIP_TRY(hipGetLastError());
@@ -788,6 +788,28 @@ void roi_align_backward_nhwc_f318a24e(const int device_id, const int nthreads, c
                                                           bottom_diff, bottom_rois))
 }
 
+#define MOBULA_NHWC_BACKWARD_16(suffix, assign_suffix, type)                                                   \
+  void roi_align_backward_nhwc_##suffix(const int device_id, const int nthreads, const type* top_diff,         \
+                                        const float spatial_scale, const int channels, const int height,      \
+                                        const int width, const int pooled_height, const int pooled_width,     \
+                                        const int sampling_ratio, type* bottom_diff, const float* bottom_rois) { \
+    MOBULA_NHWC_ENTRY(roi_align_backward_nhwc_kernel<type>(nthreads, top_diff, spatial_scale, channels, height, \
+                                                           width, pooled_height, pooled_width, sampling_ratio, \
+                                                           bottom_diff, bottom_rois))                          \
+  }                                                                                                            \
+  void roi_align_backward_nhwc_assign_##assign_suffix(                                                         \
+      const int device_id, const int nthreads, const type* top_diff, const float spatial_scale,                \
+      const int channels, const int height, const int width, const int pooled_height, const int pooled_width,  \
+      const int sampling_ratio, const int num_images, type* bottom_diff, const float* bottom_rois) {           \
+    MOBULA_NHWC_ENTRY(roi_align_backward_nhwc_assign_kernel<type>(nthreads, top_diff, spatial_scale, channels, \
+                                                                  height, width, pooled_height, pooled_width,  \
+                                                                  sampling_ratio, num_images, bottom_diff,     \
+                                                                  bottom_rois))                                \
+  }
+MOBULA_NHWC_BACKWARD_16(23175303, 7924dbc8, __half)
+MOBULA_NHWC_BACKWARD_16(0c43e974, 86156afd, roialign::bfloat16)
+#undef MOBULA_NHWC_BACKWARD_16
+
 void roi_align_backward_nhwc_assign_a8793cbe(const int device_id, const int nthreads, const float* top_diff,
                                              const float spatial_scale, const int channels, const int height,
                                              const int width, const int pooled_height, const int pooled_width,
@@ -801,7 +823,7 @@ void roi_align_backward_nhwc_assign_a8793cbe(const int device_id, const int nthr
 #undef MOBULA_NHWC_ENTRY
 
 // 1 if the channels-last entry points take the shape, else 0.  backward != 0 asks
-// about the two backward entry points (fp32 only), elem_bytes is 4 (fp32) or 2 (fp16).
+// about the backward entry points, elem_bytes is 4 (fp32) or 2 (fp16, bfloat16).
 int mobula_hip_roialign_nhwc_supported(int backward, int elem_bytes, int channels, int height, int width,
                                        int pooled_height, int pooled_width, int sampling_ratio,
                                        long long num_rois) {
@@ -811,7 +833,7 @@ int mobula_hip_roialign_nhwc_supported(int backward, int elem_bytes, int channel
   Problem p;
   p.R = static_cast<int>(num_rois); p.C = channels; p.H = height; p.W = width;
   p.PH = pooled_height; p.PW = pooled_width; p.S = sampling_ratio;
-  if (backward) return elem_bytes == 4 && nhwc_backward_supported(p) ? 1 : 0;
+  if (backward) return (elem_bytes == 4 || elem_bytes == 2) && nhwc_backward_supported(p) ? 1 : 0;
   if (elem_bytes == 4) return nhwc_forward_supported<float>(p) ? 1 : 0;
   if (elem_bytes == 2) return nhwc_forward_supported<__half>(p) ? 1 : 0;
   return 0;
@@ -835,4 +857,6 @@ static mobula_hip::ExportRegistrar roialign_exports(
     "roi_align_forward_f951d439 roi_align_backward_0c43e974 roi_align_backward_assign_86156afd "
     "roi_align_forward_nhwc_ab78de3c roi_align_forward_nhwc_e874c59a roi_align_forward_nhwc_f951d439 "
     "roi_align_backward_nhwc_f318a24e roi_align_backward_nhwc_assign_a8793cbe "
+    "roi_align_backward_nhwc_23175303 roi_align_backward_nhwc_assign_7924dbc8 "
+    "roi_align_backward_nhwc_0c43e974 roi_align_backward_nhwc_assign_86156afd "
     "mobula_hip_roialign_nhwc_supported");

@@ -120,7 +120,7 @@ def forward_nhwc(x, rois, pooled, scale, S, dev=0, stream=None):
 
 
 def backward_nhwc(dy, rois, shape, scale, S, dx=None, assign=False, dev=0, stream=None):
-    """dy: cuda fp32 [R,PH,PW,C]; shape = (N,H,W,C) of dx."""
+    """dy: cuda [R,PH,PW,C] (fp32, fp16 or bfloat16); shape = (N,H,W,C) of dx, which has dy's type."""
     N, H, W, C = shape
     PH, PW = dy.shape[1], dy.shape[2]
     if dx is None:
@@ -129,12 +129,12 @@ def backward_nhwc(dy, rois, shape, scale, S, dx=None, assign=False, dev=0, strea
     lib = native.library()
     if assign:
         _begin([-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()], stream)
-        lib.roi_align_backward_nhwc_assign_a8793cbe(
+        getattr(lib, 'roi_align_backward_nhwc_assign_' + _SUFFIX[dy.dtype][2])(
             ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
             ctypes.c_int(N), _ptr(dx), _ptr(rois))
     else:
         _begin([-1, dy.numel(), -1, -1, -1, -1, -1, -1, -1, dx.numel(), rois.numel()], stream)
-        lib.roi_align_backward_nhwc_f318a24e(
+        getattr(lib, 'roi_align_backward_nhwc_' + _SUFFIX[dy.dtype][1])(
             ctypes.c_int(dev), ctypes.c_int(dy.numel()), _ptr(dy), *_geom(scale, C, H, W, PH, PW, S),
             _ptr(dx), _ptr(rois))
     _end(lib)

@@ -173,8 +173,12 @@ def test_half_precision_training_step(mobula, low, tol):
     assert float((xh.grad.float() - xf.grad).abs().max()) <= tol * float(xf.grad.abs().max())
     # channels-last 16-bit maps: the forward reads them where they lie
     xc = x32.to(low).contiguous(memory_format=torch.channels_last)
+    xc.requires_grad_(True)
     yc = mobula.op.ROIAlign(xc, rois, **kw)
-    assert float((yc.float() - yf.detach()).abs().max()) <= tol * float(yf.detach().abs().max())
+    assert float((yc.detach().float() - yf.detach()).abs().max()) <= tol * float(yf.detach().abs().max())
+    yc.backward(dy.contiguous(memory_format=torch.channels_last))
+    assert xc.grad.dtype == low and xc.grad.is_contiguous(memory_format=torch.channels_last)
+    assert float((xc.grad.float() - xf.grad).abs().max()) <= tol * float(xf.grad.abs().max())
 
 
 def test_double_tensors_through_the_operator(mobula):

@@ -159,6 +159,21 @@ def test_bfloat16_storage(C, S):
     base = _round_bf16(rng.standard_normal((N, C, H, W)))
     dx = abi.backward(dy, r, (N, C, H, W), scale, S, dx=abi.to_dev(base).to(torch.bfloat16))
     assert_parity(dx.float().cpu().numpy(), _round_bf16(want_dx + base), BF16_TOL, 'bf16 bwd accumulate')
+    if native.roialign_channels_last_supported(True, 2, C, H, W, pooled, S, R):
+        # channels-last gradients of both 16-bit types, overwriting and accumulating
+        for low, rnd, tol in ((torch.bfloat16, _round_bf16, BF16_TOL),
+                              (torch.float16, lambda a: a.astype(np.float16).astype(np.float32), FP16_TOL)):
+            dy_cl = abi.to_dev(dyb).to(low).permute(0, 2, 3, 1).contiguous()
+            want = oracle.backward(dy_cl.permute(0, 3, 1, 2).float().cpu().numpy(), rois, (N, C, H, W), scale, S,
+                                   impl='ordered')
+            got = abi.backward_nhwc(dy_cl, r, (N, H, W, C), scale, S, assign=True)
+            assert got.dtype == low
+            assert_parity(got.permute(0, 3, 1, 2).float().cpu().numpy(), rnd(want), tol, 'channels-last bwd assign')
+            seed = abi.to_dev(base).to(low).permute(0, 2, 3, 1).contiguous()
+            want_acc = want + seed.permute(0, 3, 1, 2).float().cpu().numpy()
+            got = abi.backward_nhwc(dy_cl, r, (N, H, W, C), scale, S, dx=seed)
+            assert_parity(got.permute(0, 3, 1, 2).float().cpu().numpy(), rnd(want_acc), tol,
+                          'channels-last bwd accumulate')
 
 
 @pytest.mark.parametrize('S', [2, 0])
