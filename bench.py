@@ -34,9 +34,11 @@ MEASURED_TRAFFIC = {
 }
 
 
-def cpu_baseline(w, budget_s=25.0):
+def cpu_baseline(w, budget_s=25.0, gpu_result=None):
     """Reference kernels on the host cores: forward+backward ROIs/s on a
-    bounded sample (the first ROIs of the same workload, full channel count)."""
+    bounded sample (the first ROIs of the same workload, full channel count).
+    `gpu_result(n)` returns what the library computes for the same n ROIs; the
+    largest differences between the two go into the report."""
     import numpy as np
     from oracle import roialign as oracle
     kind = 'reference' if oracle.ref_available('omp') else 'port'
@@ -51,9 +53,8 @@ def cpu_baseline(w, budget_s=25.0):
         rois = w['rois'][:n]
         dy = w['dy'][:n] if w['dy'] is not None else None
         t0 = time.perf_counter()
-        oracle.forward(x, rois, pooled, scale, S, impl=impl)
-        if dy is not None:
-            oracle.backward(dy, rois, x.shape, scale, S, impl=impl)
+        y_cpu = oracle.forward(x, rois, pooled, scale, S, impl=impl)
+        dx_cpu = oracle.backward(dy, rois, x.shape, scale, S, impl=impl) if dy is not None else None
         dt = time.perf_counter() - t0
         spent += dt
         best = (n, dt)
@@ -62,9 +63,21 @@ def cpu_baseline(w, budget_s=25.0):
             break
         n = min(R, n * 4)
     n, dt = best
-    return {'value': n / dt, 'unit': 'ROIs/s', 'cores': oracle.num_threads(), 'kind': kind,
-            'sample': 'first {} of {} ROIs of {} ({}), one pass, {:.2f} s'.format(
-                n, R, w['name'], 'fwd+bwd' if w['dy'] is not None else 'fwd only', dt)}
+    out = {'value': n / dt, 'unit': 'ROIs/s', 'cores': oracle.num_threads(), 'kind': kind,
+           'sample': 'first {} of {} ROIs of {} ({}), one pass, {:.2f} s'.format(
+               n, R, w['name'], 'fwd+bwd' if w['dy'] is not None else 'fwd only', dt)}
+    if gpu_result is not None:
+        # the same sample through the library: max |gpu - cpu| / max |cpu| per pass
+        def rel(a, b):
+            a, b = a.astype(np.float32), b.astype(np.float32)
+            return float(np.abs(a - b).max() / max(float(np.abs(b).max()), 1e-30))
+        y_gpu, dx_gpu = gpu_result(n)
+        if w['data'].dtype.itemsize == 2:   # 16-bit storage: the checker's result is rounded the same way
+            y_cpu = y_cpu.astype(w['data'].dtype)
+        out['gpu_vs_cpu'] = {'forward_max_rel': rel(y_gpu, y_cpu)}
+        if dx_cpu is not None:
+            out['gpu_vs_cpu']['backward_max_rel'] = rel(dx_gpu, dx_cpu)
+    return out
 
 
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
@@ -348,7 +361,17 @@ def main():
     if op_ms is not None:
         out['passes']['operator_fwd_bwd'] = {'ms': op_ms, 'rois_per_s': R / (op_ms * 1e-3)}
     if not args.no_cpu_baseline:
-        out['cpu_baseline'] = cpu_baseline(w)
+        def gpu_result(n):
+            # NCHW results for the first n ROIs, whatever layout the timed loop used
+            x_nchw = x.permute(0, 3, 1, 2).contiguous() if nhwc else x
+            part = rois[:n].contiguous()
+            y_n = abi.forward(x_nchw, part, pooled, scale, S)
+            dx_n = None
+            if has_bwd:
+                dy_nchw = (dy.permute(0, 3, 1, 2) if nhwc else dy)[:n].contiguous()
+                dx_n = abi.backward(dy_nchw, part, x_nchw.shape, scale, S, assign=True).cpu().numpy()
+            return y_n.cpu().numpy(), dx_n
+        out['cpu_baseline'] = cpu_baseline(w, gpu_result=gpu_result)
     print(json.dumps(out))
 
 
