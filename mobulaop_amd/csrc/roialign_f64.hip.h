@@ -41,9 +41,35 @@ struct AxisSample64 {
   bool valid;
 };
 
+__device__ __forceinline__ double sample_coord64(double start, int p, double bin, int i, int grid) {
+  return start + p * bin + (static_cast<double>(i) + 0.5) * bin / static_cast<double>(grid);
+}
+
+// [*first, *last): the samples of pooled index p that can be valid; see
+// valid_sample_range in roialign_geometry.h (same rule, binary64).
+__device__ __forceinline__ void valid_sample_range64(double start, int p, double bin, int grid, int size,
+                                                     int* first, int* last) {
+  *first = 0;
+  *last = grid;
+  if (grid <= 64) return;
+  int lo = 0, hi = grid;
+  while (lo < hi) {
+    const int mid = lo + (hi - lo) / 2;
+    if (sample_coord64(start, p, bin, mid, grid) < -1.0) lo = mid + 1; else hi = mid;
+  }
+  *first = lo;
+  hi = grid;
+  while (lo < hi) {
+    const int mid = lo + (hi - lo) / 2;
+    if (sample_coord64(start, p, bin, mid, grid) > size) hi = mid; else lo = mid + 1;
+  }
+  *last = lo;
+  if (*first < *last && isnan(sample_coord64(start, p, bin, *first, grid))) *last = *first + 1;
+}
+
 __device__ __forceinline__ AxisSample64 axis_sample64(double start, int p, double bin, int i,
                                                       int grid, int size) {
-  double v = start + p * bin + (static_cast<double>(i) + 0.5) * bin / static_cast<double>(grid);
+  double v = sample_coord64(start, p, bin, i, grid);
   AxisSample64 s;
   s.valid = !(v < -1.0 || v > size);
   if (v <= 0) v = 0;
@@ -78,9 +104,12 @@ roialign_f64_kernel(long long n_out, const double* __restrict__ in, double scale
     const long long plane = (static_cast<long long>(image_ok ? g.batch : 0) * C + c) * H * W;
     const double top = MODE == 1 ? in[idx] : 0.0;
     double acc = 0.0;
-    for (int iy = 0; image_ok && iy < g.grid_h; ++iy) {
+    int y0, y1, x0, x1;   // samples outside add nothing
+    valid_sample_range64(g.start_h, ph, g.bin_h, g.grid_h, H, &y0, &y1);
+    valid_sample_range64(g.start_w, pw, g.bin_w, g.grid_w, W, &x0, &x1);
+    for (int iy = y0; image_ok && iy < y1; ++iy) {
       const AxisSample64 sy = axis_sample64(g.start_h, ph, g.bin_h, iy, g.grid_h, H);
-      for (int ix = 0; ix < g.grid_w; ++ix) {
+      for (int ix = x0; ix < x1; ++ix) {
         const AxisSample64 sx = axis_sample64(g.start_w, pw, g.bin_w, ix, g.grid_w, W);
         if (!(sy.valid && sx.valid)) continue;
         const double w1 = sy.h * sx.h, w2 = sy.h * sx.l, w3 = sy.l * sx.h, w4 = sy.l * sx.l;

@@ -122,6 +122,9 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   const int batch = uni_i(g.batch);
   const bool image_ok = batch >= 0 && batch < num_images;
   const int gh = uni_i(g.grid_h), gw = uni_i(g.grid_w);
+  // A box far larger than the map (or infinite) has up to 2^31 sample points per
+  // bin, nearly all outside the map: forward_large_grid_kernel does those boxes.
+  if (gh > kSearchedGrid || gw > kSearchedGrid) return;
   const float count = uni_f(g.count);
   MergedEntry (*const rowm)[M::LCAP] = rowm_s[wave];
   MergedEntry (*const colm)[M::LCAP] = colm_s[wave];

@@ -46,6 +46,40 @@ __device__ __forceinline__ float sample_coord(float start, int p, float bin, int
   return (start + a) + b;
 }
 
+// The samples i of pooled index p whose coordinate lies in [-1, size] -- the only
+// ones that contribute (opzoo/ROIAlign/bilinear.h:15-18) -- as a range
+// [*first, *last) of [0, grid).  The coordinate never decreases with i (every
+// step of sample_coord is monotonic under rounding), so the range is found by
+// bisection with that very function: the cut falls exactly where the
+// reference's test does.  Grids of ordinary size are not searched (all of
+// [0, grid) is returned); the point is to bound the work for boxes far larger
+// than the map, or infinite, whose adaptive grid has up to 2^31 points per bin
+// of which only about `size` can be valid.
+constexpr int kSearchedGrid = 64;
+
+__device__ __forceinline__ void valid_sample_range(float start, int p, float bin, int grid, int size,
+                                                   int* first, int* last) {
+  *first = 0;
+  *last = grid;
+  if (grid <= kSearchedGrid) return;
+  int lo = 0, hi = grid;
+  while (lo < hi) {   // first sample that is not left of -1
+    const int mid = lo + (hi - lo) / 2;
+    if (sample_coord(start, p, bin, mid, grid) < -1.0f) lo = mid + 1; else hi = mid;
+  }
+  *first = lo;
+  hi = grid;
+  while (lo < hi) {   // first sample right of `size`
+    const int mid = lo + (hi - lo) / 2;
+    if (sample_coord(start, p, bin, mid, grid) > static_cast<float>(size)) hi = mid; else lo = mid + 1;
+  }
+  *last = lo;
+  // A box with infinite corners can give coordinates that are not numbers; they
+  // pass the reference's test, every one of them makes the result NaN, and one
+  // does so as well as 2^31.
+  if (*first < *last && isnan(sample_coord(start, p, bin, *first, grid))) *last = *first + 1;
+}
+
 struct AxisSample {
   int low, high;  // the two neighbouring rows (or columns)
   float l, h;     // weight of `high` and of `low`

@@ -25,9 +25,12 @@ forward_naive_kernel(long long n_out, const T* __restrict__ x, float scale, int 
     float acc = 0.0f;
     if (g.batch >= 0 && g.batch < num_images) {
       const T* plane = x + (static_cast<long long>(g.batch) * C + c) * H * W;
-      for (int iy = 0; iy < g.grid_h; ++iy) {
+      int y0, y1, x0, x1;   // samples outside add nothing
+      valid_sample_range(g.start_h, ph, g.bin_h, g.grid_h, H, &y0, &y1);
+      valid_sample_range(g.start_w, pw, g.bin_w, g.grid_w, W, &x0, &x1);
+      for (int iy = y0; iy < y1; ++iy) {
         const AxisSample sy = axis_sample(sample_coord(g.start_h, ph, g.bin_h, iy, g.grid_h), H);
-        for (int ix = 0; ix < g.grid_w; ++ix) {
+        for (int ix = x0; ix < x1; ++ix) {
           const AxisSample sx = axis_sample(sample_coord(g.start_w, pw, g.bin_w, ix, g.grid_w), W);
           float val = 0.0f;
           if (sy.valid && sx.valid) {
@@ -43,6 +46,49 @@ forward_naive_kernel(long long n_out, const T* __restrict__ x, float scale, int 
       }
     }
     y[idx] = from_float<T>(acc / g.count);
+  }
+}
+
+// The boxes forward_merged_kernel leaves out: those whose sampling grid has more
+// than kSearchedGrid points per bin along an axis.  One wavefront per ROI (it
+// returns at once for every other box); its lanes share out the ROI's outputs
+// and visit only the samples that can be valid.  NHWC: map [N][H][W][C] and
+// pooled tensor [R][PH][PW][C].
+template <typename T, bool NHWC>
+__global__ void __launch_bounds__(64)
+forward_large_grid_kernel(const T* __restrict__ x, float scale, int C, int H, int W, int PH, int PW, int S,
+                          const float* __restrict__ rois, T* __restrict__ y, long long num_images) {
+  const long long r = blockIdx.x;
+  const RoiGeom g = roi_geometry(rois + r * 5, scale, PH, PW, S);
+  if (g.grid_h <= kSearchedGrid && g.grid_w <= kSearchedGrid) return;
+  const bool image_ok = g.batch >= 0 && g.batch < num_images;
+  const int bins = PH * PW;
+  for (int o = threadIdx.x; o < C * bins; o += 64) {
+    // consecutive lanes take consecutive addresses of y in either layout
+    const int c = NHWC ? o % C : o / bins, bin = NHWC ? o / C : o % bins;
+    const int ph = bin / PW, pw = bin - ph * PW;
+    float acc = 0.0f;
+    if (image_ok) {
+      int y0, y1, x0, x1;
+      valid_sample_range(g.start_h, ph, g.bin_h, g.grid_h, H, &y0, &y1);
+      valid_sample_range(g.start_w, pw, g.bin_w, g.grid_w, W, &x0, &x1);
+      const long long image = static_cast<long long>(g.batch) * C * H * W;
+      auto at = [&](int row, int col) {
+        return to_float(x[NHWC ? image + (static_cast<long long>(row) * W + col) * C + c
+                               : image + (static_cast<long long>(c) * H + row) * W + col]);
+      };
+      for (int iy = y0; iy < y1; ++iy) {
+        const AxisSample sy = axis_sample(sample_coord(g.start_h, ph, g.bin_h, iy, g.grid_h), H);
+        for (int ix = x0; ix < x1; ++ix) {
+          const AxisSample sx = axis_sample(sample_coord(g.start_w, pw, g.bin_w, ix, g.grid_w), W);
+          if (!(sy.valid && sx.valid)) continue;
+          const float w1 = sy.h * sx.h, w2 = sy.h * sx.l, w3 = sy.l * sx.h, w4 = sy.l * sx.l;
+          acc += w1 * at(sy.low, sx.low) + w2 * at(sy.low, sx.high) + w3 * at(sy.high, sx.low) +
+                 w4 * at(sy.high, sx.high);
+        }
+      }
+    }
+    y[r * C * bins + o] = from_float<T>(acc / g.count);
   }
 }
 
@@ -64,10 +110,13 @@ backward_naive_kernel(long long n_out, const TI* __restrict__ dy, float scale, i
     if (g.batch < 0 || g.batch >= num_images) continue;
     float* plane = dx + (static_cast<long long>(g.batch) * C + c) * H * W;
     const float top = to_float(dy[idx]);
-    for (int iy = 0; iy < g.grid_h; ++iy) {
+    int y0, y1, x0, x1;   // samples outside add nothing
+    valid_sample_range(g.start_h, ph, g.bin_h, g.grid_h, H, &y0, &y1);
+    valid_sample_range(g.start_w, pw, g.bin_w, g.grid_w, W, &x0, &x1);
+    for (int iy = y0; iy < y1; ++iy) {
       const AxisSample sy = axis_sample(sample_coord(g.start_h, ph, g.bin_h, iy, g.grid_h), H);
       if (!sy.valid) continue;
-      for (int ix = 0; ix < g.grid_w; ++ix) {
+      for (int ix = x0; ix < x1; ++ix) {
         const AxisSample sx = axis_sample(sample_coord(g.start_w, pw, g.bin_w, ix, g.grid_w), W);
         if (!sx.valid) continue;
         const float w1 = sy.h * sx.h, w2 = sy.h * sx.l, w3 = sy.l * sx.h, w4 = sy.l * sx.l;

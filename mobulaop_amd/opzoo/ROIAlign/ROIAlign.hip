@@ -149,9 +149,15 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
       roialign::forward_blocked_kernel<T, true><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
           x, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, p.PH, p.R);
     } else {
-      mobula_hip::KernelTimer timer("forward_merged_kernel", stream);
-      roialign::forward_merged_kernel<T, true><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
-          x, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, p.PH, p.R);
+      {
+        mobula_hip::KernelTimer timer("forward_merged_kernel", stream);
+        roialign::forward_merged_kernel<T, true><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+            x, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, p.PH, p.R);
+      }
+      // the boxes that kernel leaves out (sampling grids of more than 64 points per axis)
+      if (p.S <= 0 || p.S > roialign::kSearchedGrid)
+        roialign::forward_large_grid_kernel<T, true><<<static_cast<unsigned>(p.R), 64, 0, stream>>>(
+          x, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, rois, y, p.N);
     }
     MOBULA_HIP_TRY(hipGetLastError());
     return;
@@ -184,9 +190,15 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
           xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
     } else {
       // every pixel of a bin is loaded once
-      mobula_hip::KernelTimer timer("forward_merged_kernel", stream);
-      roialign::forward_merged_kernel<T, false><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
-          xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
+      {
+        mobula_hip::KernelTimer timer("forward_merged_kernel", stream);
+        roialign::forward_merged_kernel<T, false><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+            xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
+      }
+      // the boxes that kernel leaves out (sampling grids of more than 64 points per axis), from the map itself
+      if (p.S <= 0 || p.S > roialign::kSearchedGrid)
+        roialign::forward_large_grid_kernel<T, false><<<static_cast<unsigned>(p.R), 64, 0, stream>>>(
+          x, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, rois, y, p.N);
     }
     MOBULA_HIP_TRY(hipGetLastError());
     return;

@@ -407,6 +407,61 @@ def test_empty_roi_list_and_out_of_range_batch(impl):
 
 
 @pytest.mark.parametrize('impl', IMPLS)
+def test_boxes_far_larger_than_the_map(impl):
+    """An adaptive grid has ceil(box / pooled) points per bin and axis: 1143 here, of which
+    a dozen fall on the map.  The kernels visit only the samples that can be valid (found
+    by bisection with the reference's own coordinate formula), so the results must still be
+    the reference's."""
+    abi.set_impl(impl)
+    rng = np.random.default_rng(21)
+    xh = rng.standard_normal((2, 8, 12, 16)).astype(np.float32)
+    rh = np.array([[0, -3000, -2000, 5000, 4000], [1, -500, 3, 40, 9], [0, 2, -900, 11, 700],
+                   [1, 1, 1, 14, 10]], dtype=np.float32)
+    pooled = (3, 2)
+    x, rois = abi.to_dev(xh), abi.to_dev(rh)
+    y = abi.forward(x, rois, pooled, 1.0, 0).cpu().numpy()
+    assert_parity(y, oracle.forward(xh, rh, pooled, 1.0, 0), FWD_TOL, 'fwd')
+    dyh = rng.standard_normal(y.shape).astype(np.float32)
+    dx = abi.backward(abi.to_dev(dyh), rois, x.shape, 1.0, 0, assign=True).cpu().numpy()
+    assert_parity(dx, oracle.backward(dyh, rh, xh.shape, 1.0, 0, impl='ordered'), BWD_TOL, 'bwd')
+    x64, r64 = abi.to_dev(xh.astype(np.float64)), abi.to_dev(rh.astype(np.float64))
+    np.testing.assert_array_equal(abi.forward(x64, r64, pooled, 1.0, 0).cpu().numpy(),
+                                  oracle.forward_f64(xh, rh, pooled, 1.0, 0))
+
+
+@pytest.mark.parametrize('impl', IMPLS)
+def test_non_finite_boxes_end_and_stay_inside_the_map(impl):
+    """Boxes with infinite or NaN corners: the kernels must return (an infinite box has an
+    adaptive grid of 2^31 points per bin) and must not leave their buffers.  A box whose
+    samples are all outside gives zeros; coordinates that are not numbers give NaN in that
+    box's own outputs and, in the backward, in its own image.  Such boxes sit on image 1
+    here; image 0 must come out as if they were not there."""
+    abi.set_impl(impl)
+    rng = np.random.default_rng(11)
+    xh = rng.standard_normal((2, 8, 20, 24)).astype(np.float32)
+    inf, nan = np.inf, np.nan
+    rh = np.array([[0, 4, 4, 60, 50],          # ordinary
+                   [0, 5, inf, 9, inf],        # below the map: no valid sample
+                   [inf, 1, 1, 9, 9],          # no such image
+                   [0, 10, 12, 44, 70],        # ordinary
+                   [nan, 1, 1, 9, 9],          # batch index NaN: becomes image 0 on the GPU, an ordinary box
+                   [1, -inf, 3, 20, 30], [1, 2, 2, inf, 40], [1, nan, 3, 20, 30], [1, 3, 3, nan, nan],
+                   [1, -inf, -inf, inf, inf]], dtype=np.float32)
+    ordinary = [0, 3]
+    x, rois = abi.to_dev(xh), abi.to_dev(rh)
+    as_zero_batch = rh[[0, 3, 4]].copy()
+    as_zero_batch[:, 0] = 0
+    for S in (2, 0):
+        y = abi.forward(x, rois, (7, 7), 0.25, S).cpu().numpy()
+        assert_parity(y[ordinary], oracle.forward(xh, rh[ordinary], (7, 7), 0.25, S), FWD_TOL, 'ordinary boxes')
+        assert np.abs(y[[1, 2]]).max() == 0
+        dyh = rng.standard_normal(y.shape).astype(np.float32)
+        dx = abi.backward(abi.to_dev(dyh), rois, x.shape, 0.25, S, assign=True).cpu().numpy()
+        want = oracle.backward(dyh[[0, 3, 4]], as_zero_batch, x.shape, 0.25, S, impl='ordered')
+        assert_parity(dx[0], want[0], BWD_TOL, 'image 0')
+
+
+@pytest.mark.parametrize('impl', IMPLS)
 def test_without_declared_extents(impl):
     # plain C callers do not say how many images there are: N comes from the rois
     abi.set_impl(impl)
