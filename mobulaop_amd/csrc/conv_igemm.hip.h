@@ -236,7 +236,7 @@ struct BackwardWeightOps {
   __device__ void fetch_a(int m, const Step& e, int, int ak, float (&out)[8]) const {
     const int ohw = g.OH * g.OW;
     int img = e.img, r = e.r + ak;
-    if (r >= ohw) { r -= ohw; ++img; }
+    while (r >= ohw) { r -= ohw; ++img; }   // (an output map of fewer than eight pixels: several images on)
     const size_t at = (static_cast<size_t>(img) * g.D + m) * ohw + r;
     if (m < M && ak + 8 <= e.left && r + 8 <= ohw && (at & 3) == 0) {
       const float4 lo = *reinterpret_cast<const float4*>(dy + at), hi = *reinterpret_cast<const float4*>(dy + at + 4);
@@ -261,7 +261,7 @@ struct BackwardWeightOps {
     const int ohw = g.OH * g.OW, image = g.C * g.H * g.W;
     int img = e.img, r = e.r + bk, oh0 = e.oh, ow0 = e.ow + bk;   // scalar: the step and bk are uniform
     while (ow0 >= g.OW) { ow0 -= g.OW; ++oh0; }
-    if (r >= ohw) { r -= ohw; oh0 -= g.OH; ++img; }
+    while (r >= ohw) { r -= ohw; oh0 -= g.OH; ++img; }
     if (g.stride_w == 1 && ow0 + 8 <= g.OW && bk + 8 <= e.left) {
       // eight pixels of one output row: one row check, loads from one address
       const __amdgpu_buffer_rsrc_t src = buffer_of(x + static_cast<size_t>(img) * image, image * 4u);

@@ -87,6 +87,8 @@ SHAPES = [
     (2, 64, 28, 28, 160, (3, 3), (1, 1), (1, 1), (1, 1)),   # several tiles in every dimension
     (4, 32, 30, 30, 140, (5, 5), (2, 2), (2, 2), (1, 1)),
     (5, 16, 14, 14, 24, (1, 1), (0, 0), (1, 1), (1, 1)),    # pointwise
+    (4, 38, 4, 3, 166, (1, 3), (2, 0), (2, 1), (1, 1)),     # 4 x 1 outputs: a step of the weight gradient spans images
+    (9, 5, 2, 2, 7, (2, 2), (0, 0), (1, 1), (1, 1)),        # one output pixel per image
 ]
 
 
