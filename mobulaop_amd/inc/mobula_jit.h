@@ -159,6 +159,37 @@ class KernelRunner {
 };
 }  // namespace mobula
 
+// Device memory helpers for host functions of an operator source (reference:
+// context/hip_ctx.h:116-148).  A failure is recorded as the call's error; the
+// pointer is then null.
+namespace mobula {
+template <typename T>
+T* new_array(size_t size) {
+  void* p = nullptr;
+  MOBULA_HIP_TRY(hipMalloc(&p, sizeof(T) * (size > 0 ? size : 1)));
+  return mobula_hip::failed() ? nullptr : static_cast<T*>(p);
+}
+template <typename T>
+void del_array(T* p) {
+  if (p != nullptr) MOBULA_HIP_TRY(hipFree(p));
+}
+template <typename T>
+T* MemcpyHostToDev(T* dst, const T* src, size_t size) {
+  MOBULA_HIP_TRY(hipMemcpy(dst, src, size, hipMemcpyHostToDevice));
+  return dst;
+}
+template <typename T>
+T* MemcpyDevToHost(T* dst, const T* src, size_t size) {
+  MOBULA_HIP_TRY(hipMemcpy(dst, src, size, hipMemcpyDeviceToHost));
+  return dst;
+}
+template <typename T>
+T* MemcpyDevToDev(T* dst, const T* src, size_t size) {
+  MOBULA_HIP_TRY(hipMemcpy(dst, src, size, hipMemcpyDeviceToDevice));
+  return dst;
+}
+}  // namespace mobula
+
 #define KERNEL_RUN(a) (mobula::KernelRunner<decltype(&(a))>(&(a)))
 #define KERNEL_RUN_STREAM(a, strm) (mobula::KernelRunner<decltype(&(a))>(&(a), strm))
 #define KERNEL_RUN_BEGIN(device_id) \

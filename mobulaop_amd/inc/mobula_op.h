@@ -14,7 +14,6 @@
 // take consecutive iterations.  The first parameter of a kernel is the number
 // of iterations it is launched for (the reference's convention).
 //
-//
 // Kernels that synchronise their threads (Reduce, __syncthreads, or their own
 // use of get_num_threads / get_thread_num) are launched as ONE workgroup of
 // 1024 threads, so that "all threads of the launch" and "all threads a barrier
@@ -27,8 +26,8 @@
 // binding raises (the reference exits the process); in kernel code they
 // compile to nothing.  KERNEL_RUN for host functions is in mobula_jit.h.
 //
-// Not provided: the reference's host-side helpers (blas_gemm, new_array, ...);
-// sources that need them do not build.
+// Not provided: the reference's host BLAS helper (blas_gemm); sources that need
+// it do not build.  new_array / del_array / Memcpy* are in mobula_jit.h.
 #pragma once
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>

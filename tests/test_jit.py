@@ -196,6 +196,7 @@ def test_structures_and_host_functions(more_ops, capfd):
         more_ops.positive_or_fail(-2)
     assert more_ops.positive_or_fail(5) == 5                           # and the library is usable afterwards
     _compile(more_ops, 'fill_with_sevens', _types(_INT, (_F32P, False)))
+    _compile(more_ops, 'round_trip_plus_one', _types(_INT, (_F32P, True), (_F32P, False)))
 
 
 @pytest.mark.gpu
@@ -256,6 +257,11 @@ def test_structures_and_host_launches_on_the_gpu(more_ops):
     with pytest.raises(RuntimeError, match='host memory'):
         more_ops.fill_with_sevens(8, np.zeros(8, dtype=np.float32))
     more_ops.fill_with_sevens(out.numel(), out)
+    # device memory helpers inside a host function: host arrays in, host arrays out
+    src = np.arange(1000, dtype=np.float32)
+    dst = np.zeros_like(src)
+    assert more_ops.round_trip_plus_one(1000, src, dst) == 1000
+    np.testing.assert_array_equal(dst, src + 1)
 
 
 def test_build_path_configuration(axpy_ops, tmp_path):
