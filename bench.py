@@ -235,13 +235,20 @@ def main():
         step()
     torch.cuda.synchronize()
 
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    # the throughput loop: K steps back to back, nothing else in the stream
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
-        step(evs[k])
+        step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+
+    # per-pass times: the same steps again with an event before, between and after the passes
+    # (the event records cost the stream a few microseconds each, hence a loop of their own)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    for k in range(args.steps):
+        step(evs[k])
+    torch.cuda.synchronize()
 
     # Per-kernel time of the dominant kernel of each pass: the library brackets it
     # with HIP events on the launch stream (option "kernel_timing"); measured in
