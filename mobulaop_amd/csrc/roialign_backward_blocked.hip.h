@@ -212,12 +212,13 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
     auto issue = [&](const int16v& e, u32x4 (&d)[K::G], unsigned (&u)[K::G]) {
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
-        const unsigned roi = e[4 * j], ph = e[4 * j + 1];
+        // the item's lists, the dy of the ROI it belongs to
+        const unsigned roi = e[4 * j], ph = e[4 * j + 1], owner = static_cast<unsigned>(e[4 * j + 3]) >> 2;
         if (E == 4) {
-          d[j] = __builtin_amdgcn_raw_buffer_load_b128(dy_buf, dy_lane, roi * dy_roi + ph * dy_ph + dy_fixed, 0);
+          d[j] = __builtin_amdgcn_raw_buffer_load_b128(dy_buf, dy_lane, owner * dy_roi + ph * dy_ph + dy_fixed, 0);
         } else {   // four 16-bit values: eight bytes
           typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-          const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(dy_buf, dy_lane, roi * dy_roi + ph * dy_ph + dy_fixed, 0);
+          const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(dy_buf, dy_lane, owner * dy_roi + ph * dy_ph + dy_fixed, 0);
           d[j] = u32x4{w.x, w.y, 0u, 0u};
         }
         u[j] = __builtin_amdgcn_raw_buffer_load_b32(list_buf, list_lane, roi * list_roi + list_fixed, 0);

@@ -21,7 +21,12 @@
 //                           by tile row, then by sample order
 //   col list  of (roi, tx): one 16-byte ColPair per pooled column (padded to a
 //                           multiple of 8 columns): its one or two sample columns
-// Only fixed sampling grids with S <= 2 use this path.
+// The lists hold one or two sample points per bin and axis.  A larger sampling
+// grid (a ratio above 2, or the adaptive ceil(bin size)) is cut into pieces of
+// 2 x 2 points: every piece is a list item of its own, with the box, the row
+// taps and the column pairs of its own points, and the tile owners add the
+// pieces up like so many ROIs that share one dy (the gradient is a sum over
+// sample points).  `piece_offsets_kernel` numbers the pieces.
 // Sample coordinates come from roialign_geometry.h (reference operation order).
 #pragma once
 #include "roialign_tiles.hip.h"
@@ -46,7 +51,7 @@ constexpr int kColStrideShift = 8;
 constexpr int kColStrideMask = 7;
 
 constexpr int kRowSlots = 32;   // PH * S <= 32 sample rows per ROI
-constexpr int kMaxListPW = 16;  // PW <= 16, S <= 2
+constexpr int kMaxListPW = 16;  // PW <= 16, one or two sample points per bin
 constexpr int kTileRows = 16;   // rows of a tile (fixed by the row-tap index)
 
 struct RowTap { int ph; float wy; };
@@ -73,8 +78,50 @@ inline ListLayout make_list_layout(const TileGrid& tg, int PW) {
   return l;
 }
 
+inline bool lists_in_pieces(int S) { return S != 1 && S != 2; }
 inline bool lists_supported(int PH, int PW, int S) {
-  return S >= 1 && S <= 2 && PH * S <= kRowSlots && PW <= kMaxListPW;
+  return PH * (S == 1 ? 1 : 2) <= kRowSlots && PW <= kMaxListPW;
+}
+
+// offsets[r] = number of the first piece of ROI r, offsets[R] = their total;
+// info[0] = the total, info[1] = 1 if some ROI's grid has more than
+// kSearchedGrid points along an axis (such ROIs are not cut up: the caller
+// takes another path).  One workgroup of 1024 threads.
+__global__ void __launch_bounds__(1024)
+piece_offsets_kernel(const float* __restrict__ rois, int R, float scale, int PH, int PW, int S,
+                     int* __restrict__ offsets, int* __restrict__ info) {
+  __shared__ int part[1024];
+  __shared__ int too_big;
+  const int t = threadIdx.x, share = (R + 1023) / 1024;
+  const int first = min(R, t * share), last = min(R, first + share);
+  if (t == 0) too_big = 0;
+  __syncthreads();
+  auto pieces_of = [&](int r) {
+    const RoiGeom g = roi_geometry(rois + static_cast<long long>(r) * 5, scale, PH, PW, S);
+    if (g.grid_h > kSearchedGrid || g.grid_w > kSearchedGrid || g.grid_h < 1 || g.grid_w < 1) {
+      too_big = 1;
+      return 0;
+    }
+    return ((g.grid_h + 1) / 2) * ((g.grid_w + 1) / 2);
+  };
+  int sum = 0;
+  for (int r = first; r < last; ++r) sum += pieces_of(r);
+  part[t] = sum;
+  __syncthreads();
+  if (t == 0) {   // exclusive prefix over the threads
+    int run = 0;
+    for (int i = 0; i < 1024; ++i) { const int c = part[i]; part[i] = run; run += c; }
+    offsets[R] = run;
+    info[0] = run;
+  }
+  __syncthreads();
+  int at = part[t];
+  for (int r = first; r < last; ++r) {
+    offsets[r] = at;
+    at += pieces_of(r);
+  }
+  __syncthreads();
+  if (t == 0) info[1] = too_big;
 }
 
 __device__ __forceinline__ AxisUnit clip_unit(int bin, const AxisSample& a, int t0, int tsize,
@@ -96,21 +143,40 @@ __device__ __forceinline__ AxisUnit clip_unit(int bin, const AxisSample& a, int 
 // The wavefront also finds the ROI's box (the pixels any valid sample touches),
 // and stores it as tile ranges for build_tile_work_kernel.
 __global__ void __launch_bounds__(256)
-build_lists_kernel(const float* __restrict__ rois, int R, float scale, int PH, int PW, int S, int H,
-                   int W, long long num_images, TileGrid tg, ListLayout ll,
+build_lists_kernel(const float* __restrict__ rois, int items, int R, float scale, int PH, int PW, int S_given,
+                   int H, int W, long long num_images, TileGrid tg, ListLayout ll,
                    TileBox* __restrict__ boxes, int* __restrict__ cursors,
-                   AxisUnit* __restrict__ lists) {
+                   AxisUnit* __restrict__ lists, const int* __restrict__ piece_offsets) {
   // the two bump pointers of build_tile_work_kernel, which runs after this one
   if (blockIdx.x == 0 && threadIdx.x < 2) cursors[threadIdx.x] = 0;
-  const int roi = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-  if (roi >= R) return;
+  // item: a ROI, or (piece_offsets given) one 2 x 2 piece of a ROI's sampling grid
+  const int item = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  if (item >= items) return;
   const int lane = threadIdx.x & 63;
-  const RoiGeom g = roi_geometry(rois + static_cast<long long>(roi) * 5, scale, PH, PW, S);
+  int roi = item;
+  if (piece_offsets != nullptr) {   // the ROI whose pieces include this one
+    int lo = 0, hi = R;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) / 2;
+      if (piece_offsets[mid] <= item) lo = mid; else hi = mid;
+    }
+    roi = lo;
+  }
+  const RoiGeom g = roi_geometry(rois + static_cast<long long>(roi) * 5, scale, PH, PW, S_given);
+  // S points per bin and axis in this item, the first of them point (y_first, x_first) of the grid
+  const int S = piece_offsets != nullptr ? 2 : S_given;
+  int y_first = 0, x_first = 0;
+  if (piece_offsets != nullptr) {
+    const int local = item - piece_offsets[roi], across = (g.grid_w + 1) / 2;
+    y_first = 2 * (local / across);
+    x_first = 2 * (local % across);
+  }
   // one row sample and one column sample per lane
-  AxisSample ay = axis_sample(sample_coord(g.start_h, lane / S, g.bin_h, lane % S, S), H);
-  ay.valid = ay.valid && lane < PH * S;
-  AxisSample ax = axis_sample(sample_coord(g.start_w, lane / S, g.bin_w, lane % S, S), W);
-  ax.valid = ax.valid && lane < PW * S;
+  const int iy = y_first + lane % S, ix_of_lane = x_first + lane % S;
+  AxisSample ay = axis_sample(sample_coord(g.start_h, lane / S, g.bin_h, iy, g.grid_h), H);
+  ay.valid = ay.valid && lane < PH * S && iy < g.grid_h;
+  AxisSample ax = axis_sample(sample_coord(g.start_w, lane / S, g.bin_w, ix_of_lane, g.grid_w), W);
+  ax.valid = ax.valid && lane < PW * S && ix_of_lane < g.grid_w;
   struct { int row_lo, row_hi, col_lo, col_hi; float start_h, start_w, bin_h, bin_w, count; } rec;
   rec.start_h = g.start_h; rec.start_w = g.start_w; rec.bin_h = g.bin_h; rec.bin_w = g.bin_w;
   rec.count = g.count;
@@ -127,10 +193,10 @@ build_lists_kernel(const float* __restrict__ rois, int R, float scale, int PH, i
     rec.col_lo = any ? clo : 0; rec.col_hi = any ? chi : -1;
     const int ty0 = rec.row_lo / tg.th, ty1 = any ? rec.row_hi / tg.th : -1;
     const int tx0 = rec.col_lo / tg.tw, tx1 = any ? rec.col_hi / tg.tw : -1;
-    if (lane == 0) boxes[roi] = TileBox{any ? g.batch : -1, ty0 | (ty1 << 16), tx0 | (tx1 << 16), 0};
+    if (lane == 0) boxes[item] = TileBox{any ? g.batch : -1, ty0 | (ty1 << 16), tx0 | (tx1 << 16), roi};
     if (!any) return;
   }
-  AxisUnit* const base = lists + static_cast<long long>(roi) * ll.roi_stride;
+  AxisUnit* const base = lists + static_cast<long long>(item) * ll.roi_stride;
   const float inv_count = 1.0f / rec.count;
   {
     const int ph = lane / S;
@@ -198,10 +264,11 @@ build_lists_kernel(const float* __restrict__ rois, int R, float scale, int PH, i
 // on one tile row, in ROI order, so that the owner of that row streams through
 // them without looking anything up.
 struct alignas(16) WorkEntry {
-  int roi;
+  int roi;     // the list item (its column pairs are read from its lists)
   int ph;
   float wy;
-  int flags;   // bit 0: continues the previous entry's ROI; bit 1: last entry of its ROI
+  int flags;   // bit 0: continues the previous entry's item; bit 1: last entry of its item;
+               // bits 2..: the ROI whose dy the entry reads (the item itself, or the ROI it is a piece of)
 };
 struct WorkRange { int begin; int count; };
 
@@ -291,10 +358,11 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
   for (int r = 0; r < row; ++r) out += row_total[r];
   if (lane == 0) ranges[tile * kTileRows + row] = WorkRange{out, padded};
   for (int base = begin; base < end; base += 64) {
-    int c = 0, roi = 0;
+    int c = 0, roi = 0, owner = 0;
     const RowTap* taps = nullptr;
     if (base + lane < end) {
       roi = tile_rois[base + lane];
+      owner = boxes[roi].roi << 2;
       const RowTapTable* tb = table_of(roi);
       const unsigned idx = tb->index[row];
       c = idx >> 8;
@@ -307,11 +375,14 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
     }
     WorkEntry* dst = entries + out + incl - c;
     for (int q = 0; q < c; ++q)
-      dst[q] = WorkEntry{roi, taps[q].ph, taps[q].wy, (q > 0 ? 1 : 0) | (q == c - 1 ? 2 : 0)};
+      dst[q] = WorkEntry{roi, taps[q].ph, taps[q].wy, (q > 0 ? 1 : 0) | (q == c - 1 ? 2 : 0) | owner};
     out += __shfl(incl, 63);
   }
   // padding: taps of weight zero that continue the last ROI and never end it
-  if (lane < reserved - total) entries[out + lane] = WorkEntry{tile_rois[end - 1], 0, 0.0f, 1};
+  if (lane < reserved - total) {
+    const int item = tile_rois[end - 1];
+    entries[out + lane] = WorkEntry{item, 0, 0.0f, 1 | (boxes[item].roi << 2)};
+  }
 }
 
 }  // namespace roialign

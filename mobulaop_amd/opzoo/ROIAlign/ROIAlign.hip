@@ -229,25 +229,44 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // on error); the caller then uses the straightforward kernels.
 bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_dyb,
                 hipStream_t stream, TilePlan* plan) {
+  // List items: the ROIs, or for sampling grids of more than 2 x 2 points their
+  // 2 x 2 pieces.  An adaptive grid depends on the boxes, so the number of
+  // pieces has to come back from the device (one blocking copy).
+  const bool pieces = roialign::lists_in_pieces(p.S);
+  long long items = p.R;
+  if (p.S > roialign::kSearchedGrid) return false;   // (such grids are not cut up)
+  if (pieces && p.S > 2) items = static_cast<long long>(p.R) * ((p.S + 1) / 2) * ((p.S + 1) / 2);
+  if (pieces && p.S <= 0) {
+    int* const scratch = static_cast<int*>(mobula_hip::workspace(sizeof(int) * (p.R + 3)));
+    if (failed()) return false;
+    roialign::piece_offsets_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.PH, p.PW, p.S, scratch,
+                                                           scratch + p.R + 1);
+    int info[2] = {0, 1};
+    MOBULA_HIP_TRY(hipMemcpyAsync(info, scratch + p.R + 1, sizeof(info), hipMemcpyDeviceToHost, stream));
+    MOBULA_HIP_TRY(hipStreamSynchronize(stream));
+    if (failed() || info[1] != 0) return false;   // a grid of more than 64 points per axis: not cut up
+    items = info[0];
+  }
+  if (items > (1ll << 22)) return false;
   roialign::TileGrid& g = plan->grid;
   g.th = th; g.tw = tw;
   g.ty = (p.H + th - 1) / th;
   g.tx = (p.W + tw - 1) / tw;
   g.per_image = g.ty * g.tx;
   g.total = static_cast<long long>(g.per_image) * p.N;
-  const long long list_cap = static_cast<long long>(p.R) * g.per_image;  // every ROI in every tile
+  const long long list_cap = items * g.per_image;  // every item in every tile
   if (g.total <= 0 || g.total > (1ll << 24) || list_cap > (1ll << 27)) return false;
-  const size_t b_recs = align_up(sizeof(roialign::TileBox) * std::max(p.R, 1), 256);
+  const size_t b_recs = align_up(sizeof(roialign::TileBox) * std::max<long long>(items, 1), 256);
   const size_t b_cnt = 256;   // the two bump pointers
   const size_t b_list = align_up(sizeof(int) * std::max<long long>(list_cap, 1), 256);
   plan->layout = roialign::make_list_layout(g, p.PW);
-  const long long n_units = plan->layout.roi_stride * p.R;
+  const long long n_units = plan->layout.roi_stride * items;
   if (n_units > (1ll << 25)) return false;   // 512 MiB of sample lists: not worth it
   const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256) + 256;  // blocks are read whole
   const int cblk = (p.C + 31) / 32;
   const size_t b_dyt = with_dyb ? align_up(sizeof(float) * 32 * plan->layout.col_stride * p.R * p.PH * cblk, 256) : 0;
   // work lists: every tap of every ROI once per tile column it spans
-  const long long n_entries = static_cast<long long>(p.R) * 2 * p.PH * std::max(p.S, 1) * g.tx +
+  const long long n_entries = items * 2 * p.PH * (p.S == 1 ? 1 : 2) * g.tx +
                               11 * roialign::kTileRows * g.total;
   if (n_entries > (1ll << 27)) return false;
   // the consumer addresses both with 32-bit byte offsets
@@ -255,8 +274,9 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   plan->dyb_bytes = b_dyt; plan->list_bytes = b_units;
   const size_t b_ranges = align_up(sizeof(roialign::WorkRange) * g.total * roialign::kTileRows, 256);
   const size_t b_entries = align_up(sizeof(roialign::WorkEntry) * n_entries, 256) + 512;
+  const size_t b_offsets = pieces ? align_up(sizeof(int) * (p.R + 3), 256) : 0;
   char* base = static_cast<char*>(mobula_hip::workspace(b_recs + b_cnt + b_list + b_units + b_dyt +
-                                                        b_ranges + b_entries + 256));
+                                                        b_ranges + b_entries + b_offsets + 256));
   if (failed()) return false;
   plan->boxes = reinterpret_cast<roialign::TileBox*>(base);
   plan->cursors = reinterpret_cast<int*>(base + b_recs);
@@ -269,12 +289,19 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   cur += b_ranges;
   plan->entries = reinterpret_cast<roialign::WorkEntry*>(cur);
   cur += b_entries;
-  // two kernels: per-ROI tables (which also resets the bump pointers), then per-tile lists
-  roialign::build_lists_kernel<<<std::max(1, (p.R * 64 + 255) / 256), 256, 0, stream>>>(
-      rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->layout, plan->boxes,
-      plan->cursors, plan->lists);
+  int* offsets = nullptr;
+  if (pieces) {   // (again, for an adaptive grid: the buffer of the first pass may have moved)
+    offsets = reinterpret_cast<int*>(cur);
+    roialign::piece_offsets_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.PH, p.PW, p.S, offsets,
+                                                           offsets + p.R + 1);
+  }
+  // two kernels: per-item tables (which also resets the bump pointers), then per-tile lists
+  const int n_items = static_cast<int>(items);
+  roialign::build_lists_kernel<<<static_cast<unsigned>(std::max(1ll, (items * 64 + 255) / 256)), 256, 0, stream>>>(
+      rois, n_items, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->layout, plan->boxes,
+      plan->cursors, plan->lists, offsets);
   roialign::build_tile_work_kernel<<<static_cast<unsigned>(g.total), roialign::kTileRows * 64, 0, stream>>>(
-      plan->boxes, p.R, plan->tile_rois, plan->lists, g, plan->layout, plan->cursors, plan->ranges,
+      plan->boxes, n_items, plan->tile_rois, plan->lists, g, plan->layout, plan->cursors, plan->ranges,
       plan->entries);
   MOBULA_HIP_TRY(hipGetLastError());
   return !failed();
@@ -291,8 +318,11 @@ int tile_columns(const Problem& p) {
   return roialign::backward_tile_columns(p.N, p.H, p.W, (p.C + BB::CB - 1) / BB::CB);
 }
 
+// Fixed sampling grids only: whether an adaptive one fits the tiled backward
+// depends on the boxes, and this path has no other kernel to fall back on.
 bool nhwc_backward_supported(const Problem& p) {
-  return roialign::backward_blocked_supports(p.PH, p.PW, p.S) && p.C % 4 == 0 &&
+  return roialign::backward_blocked_supports(p.PH, p.PW, p.S) && p.S >= 1 && p.S <= roialign::kSearchedGrid &&
+         p.C % 4 == 0 &&
          static_cast<long long>(p.R) * p.PH * p.PW * p.C * 4 < (1ll << 31);
 }
 

@@ -221,6 +221,38 @@ def test_both_tile_widths_of_the_backward(cfg, down, columns):
         assert_parity(got.cpu().numpy(), want, BWD_TOL, 'bwd channels-last')
 
 
+@pytest.mark.parametrize('columns', [56, 28])
+@pytest.mark.parametrize('S', [0, 3, 4, 5, 7, 65])
+def test_tiled_backward_with_larger_sampling_grids(S, columns):
+    """Sampling grids other than 1 or 2 points per bin are cut into 2 x 2 pieces
+    for the tiled backward (odd grids leave half-filled pieces; S = 0 gives every
+    ROI its own grid; 65 is beyond what is cut up and takes the plain kernel).
+    Boxes: tiny, ordinary, wider than the map, partly off the map."""
+    abi.set_impl('tiled')
+    native.set_option('roialign_tile_columns', columns)
+    rng = np.random.default_rng(40 + S)
+    N, C, H, W, PH, PW, scale = 2, 32, 37, 53, 7, 6, 0.25
+    R = 96 if S < 65 else 6
+    x1 = rng.uniform(-30, W / scale, R); y1 = rng.uniform(-30, H / scale, R)
+    bw = rng.choice([0.5, 8, 40, 150, 400], R) * rng.uniform(0.5, 1.5, R)
+    bh = rng.choice([0.5, 8, 40, 150, 400], R) * rng.uniform(0.5, 1.5, R)
+    rois = np.stack([rng.integers(0, N, R), x1, y1, x1 + bw, y1 + bh], 1).astype(np.float32)
+    dy = rng.standard_normal((R, C, PH, PW)).astype(np.float32)
+    want = oracle.backward(dy, rois, (N, C, H, W), scale, S, impl='ordered')
+    d_dy, d_rois = abi.to_dev(dy), abi.to_dev(rois)
+    first = abi.backward(d_dy, d_rois, (N, C, H, W), scale, S, assign=True)
+    assert_parity(first.cpu().numpy(), want, BWD_TOL, 'bwd assign')
+    if S < 65:   # (the plain kernel adds with atomics, in any order)
+        again = abi.backward(d_dy, d_rois, (N, C, H, W), scale, S, assign=True)
+        assert torch.equal(first, again), 'the tiled backward is deterministic'
+    seed = torch.full((N, C, H, W), 2.0, device='cuda')
+    assert_parity(abi.backward(d_dy, d_rois, (N, C, H, W), scale, S, dx=seed).cpu().numpy(), want + 2, BWD_TOL,
+                  'bwd accumulate')
+    if native.roialign_channels_last_supported(True, 4, C, H, W, (PH, PW), S, R):
+        got = abi.backward_nhwc(d_dy.permute(0, 2, 3, 1).contiguous(), d_rois, (N, H, W, C), scale, S, assign=True)
+        assert_parity(got.permute(0, 3, 1, 2).cpu().numpy(), want, BWD_TOL, 'bwd channels-last')
+
+
 @pytest.mark.parametrize('impl', IMPLS)
 @pytest.mark.parametrize('shape', [
     # N, C, H, W, R, pooled, scale, S
@@ -302,7 +334,11 @@ def test_channels_last_rejects_what_it_does_not_take():
     rois = torch.tensor([[0, 1, 1, 6, 6]], device='cuda', dtype=torch.float32)
     with pytest.raises(RuntimeError, match='channels-last'):
         abi.forward_nhwc(x, rois, (2, 2), 1.0, 2)
-    dy = torch.zeros(1, 7, 7, 8, device='cuda')          # adaptive grid: not taken by the backward
+    dy = torch.zeros(1, 7, 17, 8, device='cuda')         # 17 pooled columns: more than the backward's lists hold
+    with pytest.raises(RuntimeError, match='channels-last'):
+        abi.backward_nhwc(dy, rois, (1, 8, 8, 8), 1.0, 2)
+    dy = torch.zeros(1, 2, 2, 8, device='cuda')          # adaptive grid: whether it fits depends on the boxes
+    assert not native.roialign_channels_last_supported(True, 4, 8, 8, 8, (2, 2), 0, 1)
     with pytest.raises(RuntimeError, match='channels-last'):
         abi.backward_nhwc(dy, rois, (1, 8, 8, 8), 1.0, 0)
     # the library is usable afterwards
