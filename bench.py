@@ -63,9 +63,20 @@ def cpu_baseline(w, budget_s=25.0, gpu_result=None):
             break
         n = min(R, n * 4)
     n, dt = best
+    # the CPU gets its best of a few more passes over the final sample (warm caches, settled threads)
+    passes = 1
+    while passes < 8 and spent + dt < min(budget_s, 12.0):
+        t0 = time.perf_counter()
+        oracle.forward(x, rois, pooled, scale, S, impl=impl)
+        if dy is not None:
+            oracle.backward(dy, rois, x.shape, scale, S, impl=impl)
+        again = time.perf_counter() - t0
+        spent += again
+        dt = min(dt, again)
+        passes += 1
     out = {'value': n / dt, 'unit': 'ROIs/s', 'cores': oracle.num_threads(), 'kind': kind,
-           'sample': 'first {} of {} ROIs of {} ({}), one pass, {:.2f} s'.format(
-               n, R, w['name'], 'fwd+bwd' if w['dy'] is not None else 'fwd only', dt)}
+           'sample': 'first {} of {} ROIs of {} ({}), best of {} passes, {:.2f} s each'.format(
+               n, R, w['name'], 'fwd+bwd' if w['dy'] is not None else 'fwd only', passes, dt)}
     if gpu_result is not None:
         # the same sample through the library: max |gpu - cpu| / max |cpu| per pass
         def rel(a, b):
