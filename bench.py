@@ -310,6 +310,33 @@ def main():
         torch.cuda.synchronize()
         op_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # The same step recorded once in a HIP graph and replayed: what a caller gets who captures
+    # the calls (all kernels run on every replay; the links between the two streams of a
+    # call become edges of the graph).  Not for the adaptive backward, which reads a count
+    # back from the device inside the call.
+    graph_ms = None
+    if not has_bwd or S > 0:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            inner = torch.cuda.current_stream().cuda_stream
+            y_graph = run_forward(x, rois, pooled, scale, S, stream=inner)
+            if has_bwd:
+                run_backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=inner)
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        y_eager = step()
+        torch.cuda.synchronize()
+        assert torch.equal(y_graph, y_eager), 'graph replay and direct calls differ'
+        del graph, y_graph, y_eager
+
     # Backward twice from the same inputs: the largest difference between the two
     # results (the reference's atomics give a different summation order each run).
     repeat_diff = None
@@ -378,6 +405,8 @@ def main():
         out['backward_run_to_run_max_abs'] = repeat_diff
     if op_ms is not None:
         out['passes']['operator_fwd_bwd'] = {'ms': op_ms, 'rois_per_s': R / (op_ms * 1e-3)}
+    if graph_ms is not None:
+        out['passes']['graph_replay'] = {'ms': graph_ms, 'rois_per_s': R / (graph_ms * 1e-3)}
     if not args.no_cpu_baseline:
         def gpu_result(n):
             # NCHW results for the first n ROIs, whatever layout the timed loop used

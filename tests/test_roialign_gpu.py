@@ -424,6 +424,46 @@ def test_asynchronous_calls_on_two_streams_and_two_threads():
         assert_parity(dx.cpu().numpy(), cases[k][5], BWD_TOL, 'bwd')
 
 
+@pytest.mark.parametrize('layout', ['nchw', 'nhwc'])
+def test_calls_recorded_in_a_graph_replay_bit_for_bit(layout):
+    """After one ordinary call (which sizes the workspace) a forward and a
+    backward on a capturing stream are recorded, not run; every replay, with
+    ordinary calls and synchronisations in between, gives the bits of a direct
+    call.  (The backward forks to a second stream and joins it inside the call.)"""
+    w = workloads.make_workload('cfg2')   # full size: dy is large enough for the backward to fork
+    scale, S, pooled = w['spatial_scale'], w['sampling_ratio'], w['pooled_size']
+    nhwc = layout == 'nhwc'
+    x = abi.to_dev(w['data'].transpose(0, 2, 3, 1) if nhwc else w['data'])
+    dy = abi.to_dev(w['dy'].transpose(0, 2, 3, 1) if nhwc else w['dy'])
+    rois = abi.to_dev(w['rois'])
+    fwd, bwd = (abi.forward_nhwc, abi.backward_nhwc) if nhwc else (abi.forward, abi.backward)
+    dx = torch.empty_like(x)
+    stream = torch.cuda.Stream()
+
+    def direct():
+        with torch.cuda.stream(stream):
+            y = fwd(x, rois, pooled, scale, S, stream=stream.cuda_stream)
+            bwd(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream.cuda_stream)
+        stream.synchronize()
+        return y.clone(), dx.clone()
+
+    y_want, dx_want = direct()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        inner = torch.cuda.current_stream().cuda_stream
+        y_graph = fwd(x, rois, pooled, scale, S, stream=inner)
+        bwd(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=inner)
+    for replay in range(4):
+        dx.fill_(7.0); y_graph.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_graph, y_want), 'forward, replay %d' % replay
+        assert torch.equal(dx, dx_want), 'backward, replay %d' % replay
+        y_now, dx_now = direct()            # ordinary calls between the replays
+        assert torch.equal(y_now, y_want) and torch.equal(dx_now, dx_want)
+
+
 @pytest.mark.parametrize('impl', IMPLS)
 def test_empty_roi_list_and_out_of_range_batch(impl):
     abi.set_impl(impl)
