@@ -204,8 +204,8 @@ def main():
                     help='cfg5 only: how the convolution forms its products')
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit('bench.py: this build measures one GPU only (the path shards by image with no '
-                 'exchange; see DESIGN.md); run with --gpus 1')
+        sys.exit('bench.py: this build measures one GPU only (the path would shard by image, each GPU '
+                 'taking the ROIs of its images, with no exchange between them); run with --gpus 1')
 
     if args.workload == 'cfg5':
         return bench_conv(args)
