@@ -285,6 +285,16 @@ double mobula_hip_last_kernel_ms(const char** name);
 
 int mobula_hip_device_count(void);
 
+/* The calls keep one grow-only scratch buffer per calling thread and device for
+ * their intermediate tables (no counterpart in the reference, whose kernels use
+ * none).  workspace_bytes: its current size for the calling thread on the
+ * current device.  release_workspace: gives it back to the device (waits for the
+ * work that still uses it) and returns the bytes freed; the next call allocates
+ * afresh.  A HIP graph recorded from calls of this thread refers to the buffer
+ * and must not be replayed after a release. */
+long long mobula_hip_workspace_bytes(void);
+long long mobula_hip_release_workspace(void);
+
 /* 1 if a kernel may dereference p (device, pinned or managed memory), else 0. */
 int mobula_hip_device_can_read(const void* p);
 

@@ -41,6 +41,8 @@ long long arg_extent(int index);
 // between asynchronous calls is ordered behind its previous call; every entry
 // point ends with finish_call(), which keeps the book for that.
 void* workspace(size_t bytes);
+long long release_workspace();   // frees the calling thread's buffer on the current device
+long long workspace_bytes();
 
 long long option(const char* name, long long fallback);
 

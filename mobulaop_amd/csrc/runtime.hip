@@ -83,6 +83,25 @@ void* workspace(size_t bytes) {
   return s->ptr;
 }
 
+// Frees the calling thread's scratch buffer on the current device (hipFree waits
+// for the work that still uses it); returns the bytes given back.
+long long release_workspace() {
+  Scratch* const s = scratch_of_current_device();
+  if (s == nullptr || s->ptr == nullptr) return 0;
+  const long long bytes = static_cast<long long>(s->bytes);
+  MOBULA_HIP_TRY(hipFree(s->ptr));
+  s->ptr = nullptr;
+  s->bytes = 0;
+  s->busy = false;
+  s->last = nullptr;
+  return failed() ? 0 : bytes;
+}
+
+long long workspace_bytes() {
+  Scratch* const s = scratch_of_current_device();
+  return s == nullptr ? 0 : static_cast<long long>(s->bytes);
+}
+
 long long option(const char* name, long long fallback) {
   std::lock_guard<std::mutex> lock(g_mutex);
   auto it = g_options.find(name);
@@ -297,6 +316,9 @@ double mobula_hip_last_kernel_ms(const char** name) {
     return -1.0;
   return ms;
 }
+
+long long mobula_hip_workspace_bytes(void) { return mobula_hip::workspace_bytes(); }
+long long mobula_hip_release_workspace(void) { return mobula_hip::release_workspace(); }
 
 // 1 if a kernel may dereference p: device memory, or host memory the device
 // reaches (pinned, managed); 0 for ordinary host memory and for null.

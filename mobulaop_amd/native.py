@@ -105,6 +105,21 @@ def device_can_read(address):
     return bool(fn(ctypes.c_void_p(address)))
 
 
+def workspace_bytes():
+    """Size of the calling thread's scratch buffer on the current device."""
+    fn = library().mobula_hip_workspace_bytes
+    fn.restype = ctypes.c_longlong
+    return int(fn())
+
+
+def release_workspace():
+    """Give the calling thread's scratch buffer back to the device; returns the
+    bytes freed.  The next call allocates what it needs."""
+    fn = library().mobula_hip_release_workspace
+    fn.restype = ctypes.c_longlong
+    return int(fn())
+
+
 def begin_call(stream, extents):
     lib = library()
     if stream is None:

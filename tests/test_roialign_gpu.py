@@ -464,6 +464,24 @@ def test_calls_recorded_in_a_graph_replay_bit_for_bit(layout):
         assert torch.equal(y_now, y_want) and torch.equal(dx_now, dx_want)
 
 
+def test_workspace_can_be_given_back():
+    """The scratch buffer grows with the largest call of the thread; a caller
+    may release it between phases, and the next call allocates afresh."""
+    w = workloads.make_workload('cfg1', scale_down=4)
+    scale, S, pooled = w['spatial_scale'], w['sampling_ratio'], w['pooled_size']
+    x, rois, dy = abi.to_dev(w['data']), abi.to_dev(w['rois']), abi.to_dev(w['dy'])
+    abi.set_impl('tiled')
+    y = abi.forward(x, rois, pooled, scale, S)
+    dx = abi.backward(dy, rois, x.shape, scale, S, assign=True)
+    held = native.workspace_bytes()
+    assert held > 0
+    assert native.release_workspace() == held
+    assert native.workspace_bytes() == 0 and native.release_workspace() == 0
+    assert torch.equal(abi.forward(x, rois, pooled, scale, S), y)
+    assert torch.equal(abi.backward(dy, rois, x.shape, scale, S, assign=True), dx)
+    assert native.workspace_bytes() > 0
+
+
 @pytest.mark.parametrize('impl', IMPLS)
 def test_empty_roi_list_and_out_of_range_batch(impl):
     abi.set_impl(impl)
