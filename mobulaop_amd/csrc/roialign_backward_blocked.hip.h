@@ -242,9 +242,13 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
       for (int j = 0; j < K::G; ++j) {
         const float wy = __int_as_float(e[4 * j + 2]);
         const int fl = e[4 * j + 3];
-        const float keep = (fl & 1) ? 1.0f : 0.0f;   // first tap of a ROI restarts the sum
+        if ((fl & 1) != 0) {   // (the same for the whole wavefront)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) g[i] = fmaf(lane_value<TI>(d[j], i), wy, keep * g[i]);
+          for (int i = 0; i < 4; ++i) g[i] = fmaf(lane_value<TI>(d[j], i), wy, g[i]);
+        } else {               // first tap of an item: the sum starts afresh, whatever the last one held
+#pragma unroll
+          for (int i = 0; i < 4; ++i) g[i] = lane_value<TI>(d[j], i) * wy;
+        }
         if ((fl & 2) != 0) {
           // last tap of this ROI on this row: spread g over the column samples
           // dword k of the quad's four: quad_perm [k, k, k, k]

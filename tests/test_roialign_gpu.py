@@ -464,6 +464,26 @@ def test_calls_recorded_in_a_graph_replay_bit_for_bit(layout):
         assert torch.equal(y_now, y_want) and torch.equal(dx_now, dx_want)
 
 
+@pytest.mark.parametrize('impl', IMPLS)
+def test_non_finite_gradient_of_one_roi_stays_in_its_cells(impl):
+    """dy of ROI 0 is infinite; ROI 1 lies in the same tile rows but touches
+    other cells: its part of dx is what it would be without ROI 0."""
+    abi.set_impl(impl)
+    rng = np.random.default_rng(5)
+    N, C, H, W, pooled, scale, S = 1, 8, 16, 56, (3, 3), 1.0, 2
+    rois = np.array([[0, 1.3, 2.2, 9.1, 12.7], [0, 30.4, 1.5, 41.2, 13.3]], np.float32)
+    dy = rng.standard_normal((2, C) + pooled).astype(np.float32)
+    alone = dy.copy(); alone[0] = 0.0
+    want = oracle.backward(alone, rois, (N, C, H, W), scale, S, impl='ordered')
+    dy[0] = np.inf
+    for S_ in (S, 0, 3):
+        want = oracle.backward(alone, rois, (N, C, H, W), scale, S_, impl='ordered')
+        got = abi.backward(abi.to_dev(dy), abi.to_dev(rois), (N, C, H, W), scale, S_, assign=True).cpu().numpy()
+        assert np.isfinite(got[..., 28:]).all(), 'S=%d' % S_
+        assert_parity(got[..., 28:], want[..., 28:], BWD_TOL, 'cells of ROI 1, S=%d' % S_)
+        assert not np.isfinite(got[..., :12]).all()
+
+
 def test_workspace_can_be_given_back():
     """The scratch buffer grows with the largest call of the thread; a caller
     may release it between phases, and the next call allocates afresh."""
