@@ -197,6 +197,9 @@ def main():
     ap.add_argument('--workload', default='cfg2', choices=['cfg1', 'cfg2', 'cfg3', 'cfg4', 'cfg5'])
     ap.add_argument('--impl', default='auto', choices=['auto', 'tiled', 'naive'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--sampling-ratio', type=int, default=None,
+                    help='replace the sampling ratio of the workload (0: adaptive grid); the configuration '
+                         'string of the report says so')
     ap.add_argument('--layout', default='nchw', choices=['nchw', 'nhwc'],
                     help='nhwc: channels-last tensors through the channels-last entry points (an extension; '
                          'the reference interface, and the default here, is nchw)')
@@ -216,6 +219,9 @@ def main():
     assert torch.cuda.is_available(), 'bench.py needs a GPU'
 
     w = workloads.make_workload(args.workload)
+    if args.sampling_ratio is not None:
+        w['sampling_ratio'] = args.sampling_ratio
+        w['name'] += ' with sampling_ratio replaced'
     pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
     nhwc = args.layout == 'nhwc'
     x = abi.to_dev(w['data'].transpose(0, 2, 3, 1) if nhwc else w['data'])
