@@ -290,8 +290,9 @@ int mobula_hip_device_count(void);
  * none).  workspace_bytes: its current size for the calling thread on the
  * current device.  release_workspace: gives it back to the device (waits for the
  * work that still uses it) and returns the bytes freed; the next call allocates
- * afresh.  A HIP graph recorded from calls of this thread refers to the buffer
- * and must not be replayed after a release. */
+ * afresh.  A HIP graph recorded from calls of this thread refers to the buffer:
+ * it must not be replayed after a release, and its replays are not ordered
+ * against the thread's calls on other streams (the caller orders those). */
 long long mobula_hip_workspace_bytes(void);
 long long mobula_hip_release_workspace(void);
 
