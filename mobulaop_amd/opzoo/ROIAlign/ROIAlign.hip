@@ -29,6 +29,9 @@ enum Impl { kAuto = 0, kTiled = 1, kNaive = 2 };
 // them the hand-over costs more than the overlap gains).
 constexpr int kSideStreamRois = 4096;
 constexpr long long kSideStreamBytes = 64ll << 20;
+// Maps up to this size are gathered in the caller's ROI order: each of the eight
+// L2 caches (4 MB) then holds its eighth of the map's channel blocks whole.
+constexpr size_t kSortedAboveBytes = 24u << 20;
 
 struct Problem {
   long long n_out;  // R*C*PH*PW
@@ -140,9 +143,12 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
                 "is not taken by the channels-last path", p.C, p.H, p.W, p.PH, p.PW);
       return;
     }
-    int* const order = static_cast<int*>(mobula_hip::workspace(sizeof(int) * p.R));
-    if (failed()) return;
-    roialign::roi_order_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
+    int* order = nullptr;   // (a map that stays in the L2 caches is read in the caller's ROI order)
+    if (sizeof(T) * p.N * pixels * p.C > kSortedAboveBytes) {
+      order = static_cast<int*>(mobula_hip::workspace(sizeof(int) * p.R));
+      if (failed()) return;
+      roialign::roi_order_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
+    }
     const long long grid = roialign::blocked_grid_nhwc(p.R, cblk);
     if (small_grid) {
       mobula_hip::KernelTimer timer("forward_blocked_kernel", stream);
@@ -168,12 +174,15 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
     char* const ws = static_cast<char*>(mobula_hip::workspace(xt_bytes + sizeof(int) * p.R));
     if (failed()) return;
     T* const xt = reinterpret_cast<T*>(ws);
-    int* const order = reinterpret_cast<int*>(ws + xt_bytes);
+    // ROIs are visited in spatial order when the map is larger than the L2 caches
+    // hold; a small map is read in the caller's order and the ordering kernel is left out
+    int* const order = xt_bytes > kSortedAboveBytes ? reinterpret_cast<int*>(ws + xt_bytes) : nullptr;
     // the ROI ordering (one small workgroup) runs beside the transposition
     // (handing work to a second stream and waiting for it costs 10-15 us: only
     // worth it when the ordering of many ROIs would otherwise delay the gather)
-    mobula_hip::SideStream side(stream, p.R > kSideStreamRois);
-    roialign::roi_order_kernel<<<1, 1024, 0, side.get()>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
+    mobula_hip::SideStream side(stream, order != nullptr && p.R > kSideStreamRois);
+    if (order != nullptr)
+      roialign::roi_order_kernel<<<1, 1024, 0, side.get()>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
     const dim3 tgrid(static_cast<unsigned>((pixels + 63) / 64), static_cast<unsigned>(cblk),
                      static_cast<unsigned>(p.N));
     const bool vec = pixels % 4 == 0 && reinterpret_cast<size_t>(x) % (4 * sizeof(T)) == 0;
