@@ -53,16 +53,17 @@ inline int backward_tile_columns(long long images, int H, int W, int cblk) {
 // the input words of the group are contiguous and so are its output words.
 // LDS holds the input as it is; the transposition happens in the reads.
 // T is the element type of dy (float or __half); dyb is fp32 either way.
+// `block`: index among the workgroups (of 256 threads) that transpose.
 template <typename T>
-__global__ void __launch_bounds__(256)
-transpose_dy_blocked_kernel(const T* __restrict__ dy, float* __restrict__ dyb, int C, int PH,
-                            int PW, int PWp, int cblk, int per) {
+__device__ __forceinline__ void transpose_dy_blocked_body(unsigned block, const T* __restrict__ dy,
+                                                          float* __restrict__ dyb, int C, int PH, int PW,
+                                                          int PWp, int cblk, int per) {
   constexpr int CB = BwdBlocked::CB;
   constexpr int VEC = 16 / sizeof(T);   // elements per 16-byte word
   extern __shared__ __attribute__((aligned(16))) unsigned char tbuf_bytes[];   // [per * 32][PH * PW] of T
   T* const tbuf = reinterpret_cast<T*>(tbuf_bytes);
   const int groups = (cblk + per - 1) / per;
-  const int r = blockIdx.x / groups, grp = blockIdx.x % groups;
+  const int r = block / groups, grp = block % groups;
   const int cb0 = grp * per, nblk = min(per, cblk - cb0);
   const int c0 = cb0 * CB, nch = min(nblk * CB, C - c0);
   const int bins = PH * PW;
@@ -93,6 +94,28 @@ transpose_dy_blocked_kernel(const T* __restrict__ dy, float* __restrict__ dyb, i
     }
     *reinterpret_cast<float4*>(dst + static_cast<size_t>(q) * 4) = v;
   }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+transpose_dy_blocked_kernel(const T* __restrict__ dy, float* __restrict__ dyb, int C, int PH,
+                            int PW, int PWp, int cblk, int per) {
+  transpose_dy_blocked_body<T>(blockIdx.x, dy, dyb, C, PH, PW, PWp, cblk, per);
+}
+
+// Both in one launch, for inputs too small to be worth a second stream: the
+// first list_blocks workgroups build the lists (few, and each a chain of
+// dependent steps: they start first), the others transpose dy.  The two do not
+// depend on each other; small kernels one after the other cost more in
+// dependencies than in work.  Dynamic LDS as for transpose_dy_blocked_kernel.
+template <typename T>
+__global__ void __launch_bounds__(256)
+lists_and_dy_kernel(ListsArgs lists, unsigned list_blocks, const T* __restrict__ dy, float* __restrict__ dyb,
+                    int PWp, int cblk, int per, int C) {
+  if (blockIdx.x < list_blocks)
+    build_lists_body(blockIdx.x, lists);
+  else
+    transpose_dy_blocked_body<T>(blockIdx.x - list_blocks, dy, dyb, C, lists.PH, lists.PW, PWp, cblk, per);
 }
 
 // Number of workgroups for `tiles` tiles and cblk channel blocks (job decode at

@@ -142,15 +142,36 @@ __device__ __forceinline__ AxisUnit clip_unit(int bin, const AxisSample& a, int 
 // against every tile row of the ROI's box; likewise for sample columns.
 // The wavefront also finds the ROI's box (the pixels any valid sample touches),
 // and stores it as tile ranges for build_tile_work_kernel.
-__global__ void __launch_bounds__(256)
-build_lists_kernel(const float* __restrict__ rois, int items, int R, float scale, int PH, int PW, int S_given,
-                   int H, int W, long long num_images, TileGrid tg, ListLayout ll,
-                   TileBox* __restrict__ boxes, int* __restrict__ cursors,
-                   AxisUnit* __restrict__ lists, const int* __restrict__ piece_offsets) {
+// `block`: index among the workgroups (of 256 threads) that build lists.
+struct ListsArgs {
+  const float* rois;
+  int items, R;
+  float scale;
+  int PH, PW, S_given, H, W;
+  long long num_images;
+  TileGrid tg;
+  ListLayout ll;
+  TileBox* boxes;
+  int* cursors;
+  AxisUnit* lists;
+  const int* piece_offsets;
+};
+
+__device__ __forceinline__ void build_lists_body(unsigned block, const ListsArgs& a) {
+  const float* __restrict__ rois = a.rois;
+  const int items = a.items, R = a.R, PH = a.PH, PW = a.PW, S_given = a.S_given, H = a.H, W = a.W;
+  const float scale = a.scale;
+  const long long num_images = a.num_images;
+  const TileGrid tg = a.tg;
+  const ListLayout ll = a.ll;
+  TileBox* __restrict__ boxes = a.boxes;
+  int* __restrict__ cursors = a.cursors;
+  AxisUnit* __restrict__ lists = a.lists;
+  const int* __restrict__ piece_offsets = a.piece_offsets;
   // the two bump pointers of build_tile_work_kernel, which runs after this one
-  if (blockIdx.x == 0 && threadIdx.x < 2) cursors[threadIdx.x] = 0;
+  if (block == 0 && threadIdx.x < 2) cursors[threadIdx.x] = 0;
   // item: a ROI, or (piece_offsets given) one 2 x 2 piece of a ROI's sampling grid
-  const int item = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int item = static_cast<int>((block * 256u + threadIdx.x) >> 6);
   if (item >= items) return;
   const int lane = threadIdx.x & 63;
   int roi = item;
@@ -258,6 +279,8 @@ build_lists_kernel(const float* __restrict__ rois, int items, int R, float scale
     }
   }
 }
+
+__global__ void __launch_bounds__(256) build_lists_kernel(ListsArgs a) { build_lists_body(blockIdx.x, a); }
 
 
 // One wavefront's share of a tile: the (ROI, pooled row, weight) taps that land

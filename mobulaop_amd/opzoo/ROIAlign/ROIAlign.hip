@@ -219,6 +219,7 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
 
 // Scratch layout of the tile pre-pass, carved out of the device workspace.
 struct TilePlan {
+  bool dy_transposed = false;   // the pre-pass also wrote dyb (plan_tiles was given dy)
   roialign::TileGrid grid;
   roialign::TileBox* boxes;
   int* cursors;                // bump pointers: [0] ROI lists, [1] work lists
@@ -236,8 +237,24 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // Runs the pre-pass (ROI boxes and sample tables, per-tile ROI and work lists) for tiles of th x tw
 // pixels.  Returns false if the problem is too large for the list buffers (or
 // on error); the caller then uses the straightforward kernels.
+// How transpose_dy_blocked_kernel is launched for a problem: channel blocks per
+// workgroup (what 64 KB of LDS hold, at most 4; 0: not at all), workgroups, LDS bytes.
+struct DyLaunch { int per; long long blocks; size_t lds; };
+template <typename T>
+DyLaunch dy_launch(const Problem& p) {
+  using BB = roialign::BwdBlocked;
+  const int cblk = (p.C + BB::CB - 1) / BB::CB;
+  const size_t blk_bytes = sizeof(T) * BB::CB * p.PH * p.PW;
+  const int per = static_cast<int>(std::min<size_t>(4, (64 * 1024) / blk_bytes));
+  const long long blocks = per > 0 ? static_cast<long long>(p.R) * ((cblk + per - 1) / per) : 0;
+  return DyLaunch{per, blocks, per * blk_bytes};
+}
+
+// fuse_dy (optional): dy of the call; its transposition into plan->dyb then shares
+// the launch of the list builder (plan->dy_transposed says whether it did).
+template <typename T>
 bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_dyb,
-                hipStream_t stream, TilePlan* plan) {
+                hipStream_t stream, TilePlan* plan, const T* fuse_dy = nullptr) {
   // List items: the ROIs, or for sampling grids of more than 2 x 2 points their
   // 2 x 2 pieces.  An adaptive grid depends on the boxes, so the number of
   // pieces has to come back from the device (one blocking copy).
@@ -306,9 +323,17 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   }
   // two kernels: per-item tables (which also resets the bump pointers), then per-tile lists
   const int n_items = static_cast<int>(items);
-  roialign::build_lists_kernel<<<static_cast<unsigned>(std::max(1ll, (items * 64 + 255) / 256)), 256, 0, stream>>>(
-      rois, n_items, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->layout, plan->boxes,
-      plan->cursors, plan->lists, offsets);
+  const roialign::ListsArgs la{rois, n_items, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->layout,
+                               plan->boxes, plan->cursors, plan->lists, offsets};
+  const long long list_blocks = std::max(1ll, (items * 64 + 255) / 256);
+  const DyLaunch dl = dy_launch<T>(p);
+  if (fuse_dy != nullptr && with_dyb && dl.per > 0 && dl.blocks > 0 && dl.blocks + list_blocks < (1ll << 31)) {
+    roialign::lists_and_dy_kernel<T><<<static_cast<unsigned>(dl.blocks + list_blocks), 256, dl.lds, stream>>>(
+        la, static_cast<unsigned>(list_blocks), fuse_dy, plan->dyb, plan->layout.col_stride, cblk, dl.per, p.C);
+    plan->dy_transposed = true;
+  } else {
+    roialign::build_lists_kernel<<<static_cast<unsigned>(list_blocks), 256, 0, stream>>>(la);
+  }
   roialign::build_tile_work_kernel<<<static_cast<unsigned>(g.total), roialign::kTileRows * 64, 0, stream>>>(
       plan->boxes, n_items, plan->tile_rois, plan->lists, g, plan->layout, plan->cursors, plan->ranges,
       plan->entries);
@@ -348,7 +373,7 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     const int tw = tile_columns(p);
     if (!nhwc_backward_supported(p) || reinterpret_cast<size_t>(dy) % 16 != 0 ||
         reinterpret_cast<size_t>(dx) % 16 != 0 ||
-        !plan_tiles(p, rois, roialign::kTileRows, tw, /*with_dyb=*/false, stream, &plan) ||
+        !plan_tiles<T>(p, rois, roialign::kTileRows, tw, /*with_dyb=*/false, stream, &plan) ||
         roialign::backward_blocked_grid(plan.grid.total, cblk) >= (1ll << 31)) {
       if (!failed())
         set_error("roi_align_backward_nhwc: shape C=%d pooled %dx%d sampling_ratio %d (or the type or alignment "
@@ -368,22 +393,22 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
   }
   // the pre-pass (small, latency-bound kernels) runs beside the dy transposition,
   // when that is long enough to hide it
-  mobula_hip::SideStream side(stream, static_cast<long long>(sizeof(T)) * p.n_out >= kSideStreamBytes);
+  // (without a second stream the transposition shares the launch of the list builder instead)
+  const bool forked = static_cast<long long>(sizeof(T)) * p.n_out >= kSideStreamBytes &&
+                      mobula_hip::option("side_stream", 1) != 0;
+  mobula_hip::SideStream side(stream, forked);
   const int tw = tile_columns(p);
   if (use_tiled() && roialign::backward_blocked_supports(p.PH, p.PW, p.S) &&
-      plan_tiles(p, rois, roialign::kTileRows, tw, /*with_dyb=*/true, side.get(), &plan)) {
+      plan_tiles<T>(p, rois, roialign::kTileRows, tw, /*with_dyb=*/true, side.get(), &plan,
+                    side.get() == stream ? dy : nullptr)) {
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
-    // channel blocks per workgroup of the dy transposition: what 64 KB of LDS hold, at most 4
-    const size_t dy_blk_bytes = sizeof(T) * BB::CB * p.PH * p.PW;
-    const int dy_per = static_cast<int>(std::min<size_t>(4, (64 * 1024) / dy_blk_bytes));
-    const long long dy_blocks = dy_per > 0 ? static_cast<long long>(p.R) * ((cblk + dy_per - 1) / dy_per) : 0;
-    if (grid < (1ll << 31) && dy_blocks < (1ll << 31) && dy_per > 0) {
+    const DyLaunch dl = dy_launch<T>(p);
+    if (grid < (1ll << 31) && dl.blocks < (1ll << 31) && dl.per > 0) {
       const int pwp = plan.layout.col_stride;
-      if (p.R > 0)
-        roialign::transpose_dy_blocked_kernel<T><<<static_cast<unsigned>(dy_blocks), 256,
-                                                   dy_per * dy_blk_bytes, stream>>>(
-            dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dy_per);
+      if (p.R > 0 && !plan.dy_transposed)
+        roialign::transpose_dy_blocked_kernel<T><<<static_cast<unsigned>(dl.blocks), 256, dl.lds, stream>>>(
+            dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dl.per);
       side.join();
       {
         mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
