@@ -282,9 +282,11 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
           const float l0 = __int_as_float(__builtin_amdgcn_mov_dpp(uj, 0xaa, 0xf, 0xf, true));
           const float l1 = __int_as_float(__builtin_amdgcn_mov_dpp(uj, 0xff, 0xf, 0xf, true));
           const int turns = 1 << ((__builtin_amdgcn_readfirstlane(cf) >> kColStrideShift) & kColStrideMask);
+          // A sample with a corner in the tile adds to both its cells: a corner
+          // outside the tile has its cell among the dummies, one of weight zero adds zero.
           auto add_both = [&] {
-            if ((cf & 3) != 0) add_sample(pos0, (cf & 1) ? 1.0f - l0 : 0.0f, (cf & 2) ? l0 : 0.0f);
-            if ((cf & 12) != 0) add_sample(pos1, (cf & 4) ? 1.0f - l1 : 0.0f, (cf & 8) ? l1 : 0.0f);
+            if ((cf & 3) != 0) add_sample(pos0, 1.0f - l0, l0);
+            if ((cf & 12) != 0) add_sample(pos1, 1.0f - l1, l1);
           };
           if (turns == 1) {
             add_both();
