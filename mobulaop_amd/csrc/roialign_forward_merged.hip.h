@@ -113,7 +113,7 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
     slot = part * range + wi;
   }
   if (slot >= R) return;
-  const int roi = order != nullptr ? uni_i(order[slot]) : static_cast<int>(slot);   // no order: as listed
+  const int roi = uni_i(order != nullptr ? order[slot] : static_cast<int>(slot));   // no order: as listed
   const int c0 = cb * CB, nch = min(CB, C - c0);
   const int grp = lane >> 3, quad = lane & 7;
   const bool quad_on = CPL * quad < nch;
