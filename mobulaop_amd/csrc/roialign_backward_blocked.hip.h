@@ -74,8 +74,9 @@ __device__ __forceinline__ void transpose_dy_blocked_body(unsigned block, const 
   const int n_in = nch * bins;
   if ((reinterpret_cast<size_t>(src) & 15) == 0) {
     const int nvec = n_in / VEC;
-    for (int i = threadIdx.x; i < nvec; i += 256)
-      reinterpret_cast<float4*>(tbuf)[i] = reinterpret_cast<const float4*>(src)[i];
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    for (int i = threadIdx.x; i < nvec; i += 256)   // dy is read once: no need to keep it in the caches
+      reinterpret_cast<f32x4*>(tbuf)[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src) + i);
     for (int i = VEC * nvec + threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
   } else {
     for (int i = threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];

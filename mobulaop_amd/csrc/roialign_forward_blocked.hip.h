@@ -62,7 +62,17 @@ transpose_to_blocked_kernel(const T* __restrict__ in, T* __restrict__ out, int C
       V4 v;
 #pragma unroll
       for (int i = 0; i < 4; ++i) v.v[i] = from_float<T>(0.0f);
-      if (c < C && p < P) v = *reinterpret_cast<const V4*>(src + static_cast<size_t>(c) * P + p);
+      if (c < C && p < P) {   // the map is read once here: no need to keep it in the caches
+        if constexpr (sizeof(T) == 4) {
+          typedef float f32x4 __attribute__((ext_vector_type(4)));
+          const f32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + static_cast<size_t>(c) * P + p));
+          v = __builtin_bit_cast(V4, raw);
+        } else {
+          typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+          const u32x2 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + static_cast<size_t>(c) * P + p));
+          v = __builtin_bit_cast(V4, raw);
+        }
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) tile[r + 16 * k][4 * q + i] = v.v[i];
     }
