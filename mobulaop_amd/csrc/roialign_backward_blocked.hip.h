@@ -96,7 +96,8 @@ __device__ __forceinline__ void transpose_dy_blocked_body(unsigned block, const 
       if (c + 2 < nch) v.z = to_float(in[2 * bins]);
       if (c + 3 < nch) v.w = to_float(in[3 * bins]);
     }
-    *reinterpret_cast<float4*>(dst + static_cast<size_t>(q) * 4) = v;
+    typedef float f32x4s __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(f32x4s{v.x, v.y, v.z, v.w}, reinterpret_cast<f32x4s*>(dst + static_cast<size_t>(q) * 4));
   }
 }
 
