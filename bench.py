@@ -20,7 +20,6 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, 'tests'))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
@@ -215,7 +214,7 @@ def main():
 
     import torch
     from mobulaop_amd import workloads
-    import abi_util as abi
+    from mobulaop_amd import abi
     assert torch.cuda.is_available(), 'bench.py needs a GPU'
 
     w = workloads.make_workload(args.workload)

@@ -135,7 +135,10 @@ template <typename B>
 __global__ void max_batch_kernel(const B* __restrict__ rois, int R, int* __restrict__ out) {
   int m = 0;
   for (int r = blockIdx.x * blockDim.x + threadIdx.x; r < R; r += gridDim.x * blockDim.x)
-    m = max(m, static_cast<int>(rois[r * 5]) + 1);
+{
+    const B b = rois[static_cast<long long>(r) * 5];   // (an index that is negative, huge or not a number names no image)
+    if (b >= static_cast<B>(0) && b < static_cast<B>(2147483520.0)) m = max(m, static_cast<int>(b) + 1);
+  }
   for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off));
   if ((threadIdx.x & 63) == 0) atomicMax(out, m);
 }

@@ -74,8 +74,14 @@ class HostStaging {
   std::vector<Item> items_;
 };
 
-// Synchronises if the call is synchronous and clears the per-call extents.
+// Every entry point starts a call with begin_call() -- the error text of the
+// thread's previous call is dropped, so an error is reported for the call that
+// caused it and never makes a later one return early -- and ends it with
+// finish_call(), which synchronises if the call is synchronous and clears the
+// per-call extents.
+void begin_call();
 void finish_call();
+struct CallBegin { CallBegin() { begin_call(); } };   // begin_call() as a first member / first local
 
 // A second stream of the current device on which independent helper kernels of
 // a call run beside the work on the caller's stream:
@@ -109,7 +115,7 @@ struct ExportRegistrar {
 // reports the elapsed time of the calling thread's last bracket.
 class KernelTimer {
  public:
-  KernelTimer(const char* name, hipStream_t stream);
+  KernelTimer(const char* name, hipStream_t stream, bool wanted = true);   // !wanted: no bracket
   ~KernelTimer();
 
  private:

@@ -221,8 +221,8 @@ TimerState& timer_state() {
 }
 }  // namespace
 
-KernelTimer::KernelTimer(const char* name, hipStream_t stream)
-    : stream_(stream), on_(option("kernel_timing", 0) != 0) {
+KernelTimer::KernelTimer(const char* name, hipStream_t stream, bool wanted)
+    : stream_(stream), on_(wanted && option("kernel_timing", 0) != 0) {
   if (!on_) return;
   TimerState& t = timer_state();
   if (t.start == nullptr) {
@@ -242,6 +242,8 @@ KernelTimer::~KernelTimer() {
   TimerState& t = timer_state();
   t.pending = hipEventRecord(t.stop, stream_) == hipSuccess;
 }
+
+void begin_call() { call_state().error.clear(); }
 
 void finish_call() {
   CallState& st = call_state();

@@ -93,6 +93,7 @@ class KernelCall {
   }
 
  private:
+  mobula_hip::CallBegin begin_;   // (first member: the previous call's error goes before anything can fail)
   const char* name_;
   bool host_;
   bool copies_ = false;

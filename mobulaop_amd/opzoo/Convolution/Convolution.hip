@@ -370,6 +370,7 @@ MOBULA_KERNEL conv2d_backward_bias_kernel(const int n, const T* dy, const int ac
 // ---------------------------------------------------------------------------
 namespace {
 bool on_device(const char* what, int device_id) {
+  mobula_hip::begin_call();
   if (device_id >= 0) return true;
   set_error("%s: host buffers are not supported, pass device tensors", what);
   mobula_hip::finish_call();

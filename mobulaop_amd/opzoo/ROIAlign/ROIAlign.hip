@@ -463,10 +463,17 @@ void backward_device(const Problem& p, const double* dy, const double* rois, dou
   MOBULA_HIP_TRY(hipGetLastError());
 }
 
+// Number of images a host ROI list implies: the largest batch index + 1.  Indices
+// that cannot name an image of a map with 32-bit offsets (negative, not a number,
+// beyond `limit`) are left out; the kernels skip such ROIs as well.
 template <typename B>
-long long host_images(const B* rois, int R) {
+long long host_images(const B* rois, int R, long long limit) {
   long long n = 0;
-  for (int r = 0; r < R; ++r) n = std::max<long long>(n, static_cast<long long>(rois[5 * r]) + 1);
+  for (int r = 0; r < R; ++r) {
+    const B b = rois[5 * r];
+    if (!(b >= static_cast<B>(0)) || !(b < static_cast<B>(limit))) continue;
+    n = std::max<long long>(n, static_cast<long long>(b) + 1);
+  }
   return n;
 }
 
@@ -611,6 +618,7 @@ int staging_device() { return static_cast<int>(mobula_hip::option("host_staging_
 template <typename T, typename B>
 void forward_entry(int device_id, int nthreads, const T* x, B scale, int C, int H, int W,
                    int PH, int PW, int S, const B* rois, T* y) {
+  mobula_hip::begin_call();
   if (device_id >= 0) {
     mobula_hip::DeviceScope scope(device_id);
     if (scope.ok()) roi_align_forward_kernel<T, B>(nthreads, x, scale, C, H, W, PH, PW, S, rois, y);
@@ -625,7 +633,7 @@ void forward_entry(int device_id, int nthreads, const T* x, B scale, int C, int 
   Problem p;
   if (scope.ok() && describe(&p, "roi_align_forward", nthreads, static_cast<float>(scale), C, H, W, PH,
                              PW, S, 1, 9, 10, -1)) {
-    if (p.N < 0) p.N = host_images(rois, p.R);
+    if (p.N < 0) p.N = host_images(rois, p.R, (1ll << 31) / (static_cast<long long>(C) * H * W));
     st.extents.assign(11, -1);
     st.extents[1] = p.N * C * H * W;
     mobula_hip::HostStaging stage;
@@ -634,6 +642,7 @@ void forward_entry(int device_id, int nthreads, const T* x, B scale, int C, int 
     T* dy = static_cast<T*>(stage.inout(y, sizeof(T) * p.n_out, /*upload=*/false));
     if (!failed()) roi_align_forward_kernel<T, B>(nthreads, dx, scale, C, H, W, PH, PW, S, dr, dy);
     if (!failed()) stage.flush(nullptr);
+    mobula_hip::finish_call();   // (on the staging device, before the caller's stream comes back)
   }
   st.stream = saved_stream;
   st.extents.clear();
@@ -642,6 +651,7 @@ void forward_entry(int device_id, int nthreads, const T* x, B scale, int C, int 
 template <typename T, typename B>
 void backward_entry(int device_id, int nthreads, const T* dy, B scale, int C, int H, int W,
                     int PH, int PW, int S, int num_images, T* dx, const B* rois) {
+  mobula_hip::begin_call();
   const bool assign = num_images >= 0;
   if (device_id >= 0) {
     mobula_hip::DeviceScope scope(device_id);
@@ -663,7 +673,7 @@ void backward_entry(int device_id, int nthreads, const T* dy, B scale, int C, in
   const int e_map = assign ? 10 : 9, e_rois = assign ? 11 : 10;
   if (scope.ok() && describe(&p, "roi_align_backward", nthreads, static_cast<float>(scale), C, H, W, PH,
                              PW, S, e_map, e_rois, 1, assign ? num_images : -1)) {
-    if (p.N < 0) p.N = host_images(rois, p.R);
+    if (p.N < 0) p.N = host_images(rois, p.R, (1ll << 31) / (static_cast<long long>(C) * H * W));
     mobula_hip::HostStaging stage;
     const T* ddy = static_cast<const T*>(stage.in(dy, sizeof(T) * p.n_out));
     const B* dr = static_cast<const B*>(stage.in(rois, sizeof(B) * 5 * p.R));
@@ -678,6 +688,7 @@ void backward_entry(int device_id, int nthreads, const T* dy, B scale, int C, in
         roi_align_backward_kernel<T, B>(nthreads, ddy, scale, C, H, W, PH, PW, S, ddx, dr);
     }
     if (!failed()) stage.flush(nullptr);
+    mobula_hip::finish_call();
   }
   st.stream = saved_stream;
   st.extents.clear();
@@ -731,8 +742,10 @@ void roi_align_backward_assign_4620f85e(const int device_id, const int nthreads,
                                         const int width, const int pooled_height, const int pooled_width,
                                         const int sampling_ratio, const int num_images,
                                         double* bottom_diff, const double* bottom_rois) {
+  mobula_hip::begin_call();
   if (num_images < 0) {
     set_error("roi_align_backward_assign: num_images=%d", num_images);
+    mobula_hip::finish_call();
     return;
   }
   backward_entry<double, double>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
@@ -747,8 +760,10 @@ void roi_align_backward_assign_a8793cbe(const int device_id, const int nthreads,
                                         const int pooled_height, const int pooled_width,
                                         const int sampling_ratio, const int num_images,
                                         float* bottom_diff, const float* bottom_rois) {
+  mobula_hip::begin_call();
   if (num_images < 0) {
     set_error("roi_align_backward_assign: num_images=%d", num_images);
+    mobula_hip::finish_call();
     return;
   }
   backward_entry<float, float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
@@ -770,8 +785,10 @@ void roi_align_backward_assign_7924dbc8(const int device_id, const int nthreads,
                                         const int width, const int pooled_height, const int pooled_width,
                                         const int sampling_ratio, const int num_images,
                                         __half* bottom_diff, const float* bottom_rois) {
+  mobula_hip::begin_call();
   if (num_images < 0) {
     set_error("roi_align_backward_assign: num_images=%d", num_images);
+    mobula_hip::finish_call();
     return;
   }
   backward_entry<__half, float>(device_id, nthreads, top_diff, spatial_scale, channels, height, width,
@@ -805,8 +822,10 @@ void roi_align_backward_assign_86156afd(const int device_id, const int nthreads,
                                         const int pooled_height, const int pooled_width,
                                         const int sampling_ratio, const int num_images,
                                         roialign::bfloat16* bottom_diff, const float* bottom_rois) {
+  mobula_hip::begin_call();
   if (num_images < 0) {
     set_error("roi_align_backward_assign: num_images=%d", num_images);
+    mobula_hip::finish_call();
     return;
   }
   backward_entry<roialign::bfloat16, float>(device_id, nthreads, top_diff, spatial_scale, channels, height,
@@ -816,8 +835,10 @@ void roi_align_backward_assign_86156afd(const int device_id, const int nthreads,
 
 // Channels-last variants (extensions): device pointers only.
 #define MOBULA_NHWC_ENTRY(call)                                                            \
+  mobula_hip::begin_call();                                                                \
   if (device_id < 0) {                                                                     \
     set_error("the channels-last entry points take device memory only");                   \
+    mobula_hip::finish_call();                                                             \
     return;                                                                                \
   }                                                                                        \
   {                                                                                        \

@@ -61,9 +61,11 @@ def parity_report(a, b):
                 linf_rel=float(err.max() / scale) if scale > 0 else float(err.max() if err.size else 0.0))
 
 
-def assert_parity(a, b, tol, what=''):
-    """Gate: every element within tol*|b| + tol*max|b| of the expected value
-    (reference metric with an absolute floor of tol*max|b|)."""
+def assert_parity(a, b, tol, what='', floor=None):
+    """Gate on both parity figures: (i) elementwise |a-b| <= tol * max(|b|, floor), the
+    reference's relative metric (mobula/testing.py:102-115) with an absolute floor
+    for elements near zero -- by default the tensor's scale max|b| --, and (ii)
+    ||a-b||_inf <= tol * ||b||_inf."""
     a64 = to_numpy(a).astype(np.float64)
     b64 = to_numpy(b).astype(np.float64)
     assert a64.shape == b64.shape, 'Unmatched Shape: {} vs {}'.format(a64.shape, b64.shape)
@@ -71,9 +73,12 @@ def assert_parity(a, b, tol, what=''):
         return
     assert np.isfinite(a64).all(), '{}: non-finite values'.format(what)
     err = np.abs(a64 - b64)
-    bound = tol * np.abs(b64) + tol * np.abs(b64).max()
+    scale = np.abs(b64).max()
+    bound = tol * np.maximum(np.abs(b64), scale if floor is None else floor)
     bad = err > bound
     if bad.any():
         idx = np.unravel_index(int(np.argmax(err - bound)), err.shape)
         raise AssertionError('{}: {} of {} elements outside tol={}; worst at {}: got {!r} want {!r}'
                              .format(what, int(bad.sum()), err.size, tol, idx, a64[idx], b64[idx]))
+    if err.max() > tol * scale:
+        raise AssertionError('{}: ||a-b||_inf / ||b||_inf = {:.3e} > tol={}'.format(what, err.max() / scale, tol))

@@ -186,6 +186,39 @@ def test_resnet_block_shape_properties(compute):
     assert abs(lhs - float((w.double() * dw.double()).sum())) <= bound
 
 
+@pytest.mark.parametrize('mode', ['fp32', 'bf16x3'])
+def test_full_cfg5_against_torch(mode):
+    # BASELINE configuration 5 at its full size: N=32, 256 -> 256 channels, 56 x 56, 3 x 3,
+    # stride 1, pad 1; y, dx and dw against torch's conv2d and its autograd on the CPU, 1e-3
+    N, C, H, W, D = 32, 256, 56, 56, 256
+    g = torch.Generator().manual_seed(1005)
+    xh = torch.randn(N, C, H, W, generator=g)
+    wh = torch.randn(D, C, 3, 3, generator=g) * (2.0 / (C * 9)) ** 0.5   # Kaiming-normal
+    dyh = torch.randn(N, D, H, W, generator=g)
+    xr, wr = xh.clone().requires_grad_(True), wh.clone().requires_grad_(True)
+    print('cfg5: torch conv2d on the CPU ...', flush=True)
+    yr = F.conv2d(xr, wr, padding=1)
+    yr.backward(dyh)
+    native.set_option('conv_compute', MODES[mode][0])
+    try:
+        x, w, dy = xh.cuda(), wh.cuda(), dyh.cuda()
+        geo = _ci(N, C, H, W, D, 3, 3, 1, 1, 1, 1, 1, 1)
+        y = torch.empty(N, D, H, W, device='cuda')
+        _call('conv2d_forward_c6a7aa85', ctypes.c_int(y.numel()), _ptr(x), _ptr(w), _ptr(w), ctypes.c_int(0), *geo,
+              _ptr(y))
+        _close(y, yr, 'cfg5 y ' + mode)
+        dx = torch.empty_like(x)
+        _call('conv2d_backward_data_ecf81c91', ctypes.c_int(dx.numel()), _ptr(dy), _ptr(w), ctypes.c_int(0), *geo,
+              _ptr(dx))
+        _close(dx, xr.grad, 'cfg5 dx ' + mode)
+        dw = torch.empty_like(w)
+        _call('conv2d_backward_weight_ecf81c91', ctypes.c_int(dw.numel()), _ptr(dy), _ptr(x), ctypes.c_int(0),
+              *geo, _ptr(dw))
+        _close(dw, wr.grad, 'cfg5 dw ' + mode)
+    finally:
+        native.set_option('conv_compute', 0)
+
+
 def test_bf16_mode_is_exact_on_bf16_valued_operands():
     # Mode 1 rounds both operands of every product to bf16 and accumulates in fp32: against
     # the same products of the rounded operands in fp32 only the order of the sums differs,
