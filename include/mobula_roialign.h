@@ -77,6 +77,26 @@ void roi_align_backward_assign_a8793cbe(const int device_id, const int nthreads,
                                         const int sampling_ratio, const int num_images,
                                         float* bottom_diff, const float* bottom_rois);
 
+/* The forward pass for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same result as roi_align_forward_ab78de3c
+ * (same kernels); the scratch memory those kernels need (the channel-blocked
+ * copy of the map and the ROI order) is a fixed buffer of 48 MiB that every GPU
+ * the library runs on holds until the process ends, so the call makes no
+ * allocation, no stream and no event.  num_images is the N of the [N,C,H,W]
+ * map.  Device memory only.  A problem that needs more scratch than the buffer
+ * holds (about N*C*H*W*4 + R*4 bytes) is refused with an error.  All calls on
+ * one GPU share the buffer: calls that overlap in time on one GPU race. */
+void roi_align_forward_noalloc_83212f20(const int device_id, const int nthreads,
+                                        const float* bottom_data, const float spatial_scale,
+                                        const int channels, const int height, const int width,
+                                        const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        const float* bottom_rois, float* top_data);
+/* Looks up the fixed buffer's address on device_id ahead of the first call
+ * there (which does it otherwise); returns the buffer's size in bytes, -1 on error. */
+long long mobula_hip_roialign_noalloc_init(const int device_id);
+
 /* Backward in binary64, accumulating and overwriting.  The names are what the
  * reference's scheme gives the <double> instantiations, but the reference cannot
  * build them: its atomic_add takes float only

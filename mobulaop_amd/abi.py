@@ -65,6 +65,23 @@ def forward(x, rois, pooled, scale, S, declare_extents=True, stream=None, dev=0)
     return y
 
 
+def forward_noalloc(x, rois, pooled, scale, S, y=None, stream=None, dev=0):
+    """The entry point that allocates nothing; fp32 device tensors.  y may be given
+    (a caller that cannot allocate brings its own output)."""
+    N, C, H, W = x.shape
+    PH, PW = pooled
+    R = rois.shape[0]
+    if y is None:
+        y = torch.empty((R, C, PH, PW), dtype=x.dtype, device=x.device)
+    ext = [-1, x.numel(), -1, -1, -1, -1, -1, -1, -1, -1, rois.numel(), y.numel()]
+    lib = _begin(ext, stream)
+    lib.roi_align_forward_noalloc_83212f20(ctypes.c_int(dev), ctypes.c_int(y.numel()), _ptr(x),
+                                           *_geom(scale, C, H, W, PH, PW, S), ctypes.c_int(N),
+                                           _ptr(rois), _ptr(y))
+    _end(lib)
+    return y
+
+
 def backward(dy, rois, shape, scale, S, dx=None, assign=False, declare_extents=True, stream=None,
              dev=0):
     N, C, H, W = shape

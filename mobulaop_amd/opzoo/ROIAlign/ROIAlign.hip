@@ -7,6 +7,7 @@
 // functions at the end carry the names the reference's loader derives for the
 // same instantiations (mobula/func.py:13-50, op/templates/kernel_code.cpp:1-5).
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "runtime.h"
@@ -40,6 +41,11 @@ struct Problem {
   float scale;
   double scale64 = 0.0;  // the scale as given, for the binary64 kernels
   bool nhwc = false;   // map [N,H,W,C] and pooled tensor [R,PH,PW,C] instead of [N,C,H,W] / [R,C,PH,PW]
+  // Scratch memory the caller of forward_device provides instead of the thread's
+  // workspace (the entry point that allocates nothing): no allocation, no second
+  // stream, no event is made on that path.
+  char* fixed_scratch = nullptr;
+  size_t fixed_scratch_bytes = 0;
 };
 
 // Shape checks shared by every entry point.  Returns false (with the error
@@ -110,6 +116,42 @@ long long images_from_rois(const B* d_rois, int R, hipStream_t stream) {
   return h;
 }
 
+// The fixed scratch buffer of roi_align_forward_noalloc: every GPU the library
+// runs on holds its own copy of this array at its own address.  Host code never
+// uses the array's name as an address; it asks once per device, with that
+// device current, for the device address and keeps it.
+constexpr size_t kNoAllocScratchBytes = 48u << 20;
+constexpr int kNoAllocMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char roialign_noalloc_scratch[kNoAllocScratchBytes];
+namespace {
+std::mutex g_noalloc_mutex;
+char* g_noalloc_ptr[kNoAllocMaxDevices] = {};
+
+// Device address of the current device's copy of the buffer (null and an error if it cannot be had).
+char* noalloc_scratch(size_t* bytes) {
+  *bytes = kNoAllocScratchBytes;
+  int device = -1;
+  MOBULA_HIP_TRY(hipGetDevice(&device));
+  if (failed()) return nullptr;
+  if (device < 0 || device >= kNoAllocMaxDevices) {
+    set_error("roi_align_forward_noalloc: device %d is beyond the %d the fixed buffer is kept for", device,
+              kNoAllocMaxDevices);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+  if (g_noalloc_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    MOBULA_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(roialign_noalloc_scratch)));
+    if (failed() || ptr == nullptr) {
+      if (!failed()) set_error("roi_align_forward_noalloc: the fixed buffer has no address on device %d", device);
+      return nullptr;
+    }
+    g_noalloc_ptr[device] = static_cast<char*>(ptr);
+  }
+  return g_noalloc_ptr[device];
+}
+
 int grid_for(long long n, int block) {
   return static_cast<int>(std::min<long long>((n + block - 1) / block, 256ll * 64));
 }
@@ -171,7 +213,14 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
   if (use_tiled() && fits) {
     // channel-blocked copy of the map, spatial ROI order, then the gather
     const size_t xt_bytes = (sizeof(T) * p.N * cblk * CB * pixels + 255) / 256 * 256;
-    char* const ws = static_cast<char*>(mobula_hip::workspace(xt_bytes + sizeof(int) * p.R));
+    const bool fixed = p.fixed_scratch != nullptr;
+    if (fixed && xt_bytes + sizeof(int) * p.R > p.fixed_scratch_bytes) {
+      set_error("roi_align_forward_noalloc: the problem needs %zu bytes of scratch memory, the library's fixed "
+                "buffer holds %zu (feature map too large for the entry point that allocates nothing)",
+                xt_bytes + sizeof(int) * p.R, p.fixed_scratch_bytes);
+      return;
+    }
+    char* const ws = fixed ? p.fixed_scratch : static_cast<char*>(mobula_hip::workspace(xt_bytes + sizeof(int) * p.R));
     if (failed()) return;
     T* const xt = reinterpret_cast<T*>(ws);
     // ROIs are visited in spatial order when the map is larger than the L2 caches
@@ -180,7 +229,7 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
     // the ROI ordering (one small workgroup) runs beside the transposition
     // (handing work to a second stream and waiting for it costs 10-15 us: only
     // worth it when the ordering of many ROIs would otherwise delay the gather)
-    mobula_hip::SideStream side(stream, order != nullptr && p.R > kSideStreamRois);
+    mobula_hip::SideStream side(stream, !fixed && order != nullptr && p.R > kSideStreamRois);
     if (order != nullptr)
       roialign::roi_order_kernel<<<1, 1024, 0, side.get()>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
     const dim3 tgrid(static_cast<unsigned>((pixels + 63) / 64), static_cast<unsigned>(cblk),
@@ -194,13 +243,13 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
           x, xt, p.C, static_cast<int>(pixels));
     side.join();
     if (small_grid) {
-      mobula_hip::KernelTimer timer("forward_blocked_kernel", stream);
+      mobula_hip::KernelTimer timer("forward_blocked_kernel", stream, !fixed);   // (its events are allocations)
       roialign::forward_blocked_kernel<T, false><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
           xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
     } else {
       // every pixel of a bin is loaded once
       {
-        mobula_hip::KernelTimer timer("forward_merged_kernel", stream);
+        mobula_hip::KernelTimer timer("forward_merged_kernel", stream, !fixed);
         roialign::forward_merged_kernel<T, false><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
             xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
       }
@@ -546,6 +595,35 @@ MOBULA_KERNEL roi_align_backward_assign_kernel(const int nthreads, const T* top_
   backward_device(p, top_diff, bottom_rois, bottom_diff, /*assign=*/true, call_state().stream);
 }
 
+// Not in the reference: the forward pass for callers that cannot allocate device
+// memory (code under HIP graph capture, serving loops, harnesses that forbid
+// it).  The channel-blocked copy of the map and the ROI order live in a fixed
+// buffer of the library (kNoAllocScratchBytes per GPU, held until the process
+// ends) instead of the thread's workspace: the call makes no allocation, no
+// stream and no event.  num_images is the N of the [N,C,H,W] map.  Problems
+// whose scratch need exceeds the buffer are an error.  All calls on one GPU
+// share the buffer: calls that overlap in time on one GPU race.
+template <typename T, typename B = T>
+MOBULA_KERNEL roi_align_forward_noalloc_kernel(const int nthreads, const T* bottom_data,
+                                               const B spatial_scale, const int channels,
+                                               const int height, const int width,
+                                               const int pooled_height, const int pooled_width,
+                                               const int sampling_ratio, const int num_images,
+                                               const B* bottom_rois, T* top_data) {
+  Problem p;
+  if (num_images < 0) {
+    set_error("roi_align_forward_noalloc: num_images=%d", num_images);
+    return;
+  }
+  if (!describe(&p, "roi_align_forward_noalloc", nthreads, static_cast<float>(spatial_scale), channels, height,
+                width, pooled_height, pooled_width, sampling_ratio, 1, 10, 11, num_images))
+    return;
+  p.scale64 = spatial_scale;
+  p.fixed_scratch = noalloc_scratch(&p.fixed_scratch_bytes);
+  if (failed()) return;
+  forward_device(p, bottom_data, bottom_rois, top_data, call_state().stream);
+}
+
 // Not in the reference: the same three operations on channels-last tensors, the
 // map as [N,H,W,C] and the pooled tensor as [R,PH,PW,C] (what a torch tensor in
 // torch.channels_last format holds).  The kernels read and write these where
@@ -771,6 +849,37 @@ void roi_align_backward_assign_a8793cbe(const int device_id, const int nthreads,
                         bottom_rois);
 }
 
+// The forward pass that allocates nothing (see roi_align_forward_noalloc_kernel); device memory only.
+void roi_align_forward_noalloc_83212f20(const int device_id, const int nthreads, const float* bottom_data,
+                                        const float spatial_scale, const int channels, const int height,
+                                        const int width, const int pooled_height, const int pooled_width,
+                                        const int sampling_ratio, const int num_images,
+                                        const float* bottom_rois, float* top_data) {
+  mobula_hip::begin_call();
+  if (device_id < 0) {
+    set_error("roi_align_forward_noalloc takes device memory only");
+    mobula_hip::finish_call();
+    return;
+  }
+  mobula_hip::DeviceScope scope(device_id);
+  if (scope.ok())
+    roi_align_forward_noalloc_kernel<float, float>(nthreads, bottom_data, spatial_scale, channels, height, width,
+                                                   pooled_height, pooled_width, sampling_ratio, num_images,
+                                                   bottom_rois, top_data);
+  mobula_hip::finish_call();
+}
+
+// Sets up the fixed buffer of roi_align_forward_noalloc on `device_id` ahead of
+// the first call there (the first call does it otherwise); returns its size in
+// bytes, or -1 with the error text set.
+long long mobula_hip_roialign_noalloc_init(const int device_id) {
+  mobula_hip::begin_call();
+  mobula_hip::DeviceScope scope(device_id);
+  size_t bytes = 0;
+  if (!scope.ok() || noalloc_scratch(&bytes) == nullptr) return -1;
+  return static_cast<long long>(bytes);
+}
+
 // Backward with binary16 top_diff / bottom_diff (sums in fp32, rounded once).
 void roi_align_backward_23175303(const int device_id, const int nthreads, const __half* top_diff,
                                  const float spatial_scale, const int channels, const int height,
@@ -956,4 +1065,4 @@ static mobula_hip::ExportRegistrar roialign_exports(
     "roi_align_backward_nhwc_f318a24e roi_align_backward_nhwc_assign_a8793cbe "
     "roi_align_backward_nhwc_23175303 roi_align_backward_nhwc_assign_7924dbc8 "
     "roi_align_backward_nhwc_0c43e974 roi_align_backward_nhwc_assign_86156afd "
-    "mobula_hip_roialign_nhwc_supported");
+    "mobula_hip_roialign_nhwc_supported roi_align_forward_noalloc_83212f20 mobula_hip_roialign_noalloc_init");
