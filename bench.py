@@ -23,14 +23,41 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
-# HBM bytes per launch of a kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc
-# WRITE_SIZE runs of this script (summaries under profiles/), each scaled by what
-# the same counter reads for a copy of known size.  Keyed by (workload, kernel);
-# absent entries are reported as null.
-MEASURED_TRAFFIC = {
-    ('cfg2', 'forward_blocked_kernel'): 473.4e6,    # 272.7 MB read + 200.7 MB written
-    ('cfg2', 'backward_blocked_kernel'): 575.7e6,   # 277.1 MB read + 298.6 MB written
-}
+
+
+def kernel_source_digest():
+    """Digest of the ROIAlign kernel sources: a traffic summary names the digest of the
+    sources it was measured on, and is only quoted while they are unchanged."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    files = sorted(glob.glob(os.path.join(ROOT, 'mobulaop_amd', 'csrc', 'roialign_*.h')) +
+                   [os.path.join(ROOT, 'mobulaop_amd', 'opzoo', 'ROIAlign', 'ROIAlign.hip')])
+    for f in files:
+        h.update(open(f, 'rb').read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(path, kernel):
+    """HBM bytes per launch of `kernel` from a summary under profiles/ (two rocprofv3 --pmc
+    runs of this script, FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
+    reads for a copy of known size): the `total MB` column of the NCHW table.  None when
+    the file is absent, was measured on other kernel sources, or does not list the kernel."""
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    if 'kernel sources: ' + kernel_source_digest() not in text:
+        return None
+    for line in text.split('-- channels-last')[0].splitlines():
+        parts = line.split()
+        if len(parts) >= 6 and parts[0].startswith(kernel):
+            try:
+                return float(parts[-1]) * 1e6
+            except ValueError:
+                return None
+    return None
+
 
 
 def cpu_baseline(w, budget_s=25.0, gpu_result=None):
@@ -92,6 +119,114 @@ def cpu_baseline(w, budget_s=25.0, gpu_result=None):
 
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
+
+
+def short_roialign_run(name, steps=5, warmup=2):
+    """One of the other BASELINE configurations, a few steps through the C ABI: ms per
+    step, fraction of the HBM peak on the algorithmic bytes, and the largest difference
+    from the CPU oracle on the first ROIs (relative to the largest expected value)."""
+    import numpy as np
+    import torch
+    from mobulaop_amd import abi, workloads
+    from oracle import roialign as oracle
+    w = workloads.make_workload(name)
+    pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
+    x, rois = abi.to_dev(w['data']), abi.to_dev(w['rois'])
+    has_bwd = w['dy'] is not None
+    dy = abi.to_dev(w['dy']) if has_bwd else None
+    dx = torch.empty_like(x) if has_bwd else None
+    stream = torch.cuda.current_stream().cuda_stream
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    fwd_ms = bwd_ms = 0.0
+    for k in range(warmup + steps):
+        ev[0].record()
+        abi.forward(x, rois, pooled, scale, S, stream=stream)
+        ev[1].record()
+        if has_bwd:
+            abi.backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream)
+        ev[2].record()
+        torch.cuda.synchronize()
+        if k >= warmup:
+            fwd_ms += ev[0].elapsed_time(ev[1]) / steps
+            bwd_ms += ev[1].elapsed_time(ev[2]) / steps
+    b_fwd, b_bwd = workloads.algorithmic_bytes(w)
+    nbytes = b_fwd + (b_bwd if has_bwd else 0)
+    ms = fwd_ms + bwd_ms
+    n = min(32, rois.shape[0])
+    part = rois[:n].contiguous()
+
+    def rel(a, b):
+        a, b = a.astype(np.float32), b.astype(np.float32)
+        return float(np.abs(a - b).max() / max(float(np.abs(b).max()), 1e-30))
+    want = oracle.forward(w['data'].astype(np.float32), w['rois'][:n], pooled, scale, S)
+    if w['data'].dtype.itemsize == 2:
+        want = want.astype(w['data'].dtype)
+    parity = {'forward': rel(abi.forward(x, part, pooled, scale, S).cpu().numpy(), want)}
+    if has_bwd:
+        got = abi.backward(dy[:n].contiguous(), part, x.shape, scale, S, assign=True).cpu().numpy()
+        parity['backward'] = rel(got, oracle.backward(w['dy'][:n], w['rois'][:n], w['data'].shape, scale, S,
+                                                     impl='ordered'))
+    out = {'step': 'forward + backward(assign)' if has_bwd else 'forward', 'ms_per_step': ms,
+           'forward_ms': fwd_ms, 'frac': nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+           'rois_per_s': rois.shape[0] / (ms * 1e-3), 'parity_max_rel': parity,
+           'parity_sample': 'first {} ROIs against the CPU oracle'.format(n)}
+    if has_bwd:
+        out['backward_ms'] = bwd_ms
+    return out
+
+
+def short_conv_run(steps=5, warmup=2):
+    """cfg5 with fp32 products: ms per step (forward + data gradient + weight gradient),
+    fraction of the fp32 matrix peak, parity of the first two images against torch's
+    conv2d on the CPU."""
+    import torch
+    import torch.nn.functional as F
+    from mobulaop_amd import native
+    N, C, H, W, D, K = 32, 256, 56, 56, 256, 3
+    g = torch.Generator().manual_seed(1005)
+    xh = torch.randn(N, C, H, W, generator=g)
+    wh = torch.randn(D, C, K, K, generator=g) * (2.0 / (C * K * K)) ** 0.5
+    dyh = torch.randn(N, D, H, W, generator=g)
+    x, w, dy = xh.cuda(), wh.cuda(), dyh.cuda()
+    y, dx, dw = torch.empty_like(dy), torch.empty_like(x), torch.empty_like(w)
+    lib = native.library()
+    stream = torch.cuda.current_stream().cuda_stream
+    geo = [ctypes.c_int(v) for v in (N, C, H, W, D, K, K, 1, 1, 1, 1, 1, 1)]
+    native.set_option('conv_compute', 0)
+
+    def ptr(t):
+        return ctypes.c_void_p(t.data_ptr())
+
+    def call(fn, *a):
+        native.begin_call(stream, [])
+        fn(ctypes.c_int(0), *a)
+        native.end_call(fn.__name__)
+
+    def step():
+        call(lib.conv2d_forward_c6a7aa85, ctypes.c_int(y.numel()), ptr(x), ptr(w), ptr(w), ctypes.c_int(0), *geo, ptr(y))
+        call(lib.conv2d_backward_data_ecf81c91, ctypes.c_int(dx.numel()), ptr(dy), ptr(w), ctypes.c_int(0), *geo, ptr(dx))
+        call(lib.conv2d_backward_weight_ecf81c91, ctypes.c_int(dw.numel()), ptr(dy), ptr(x), ctypes.c_int(0), *geo,
+             ptr(dw))
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    flops = 3 * 2.0 * N * D * H * W * C * K * K
+    xr = xh[:2].clone().requires_grad_(True)
+    yr = F.conv2d(xr, wh, padding=1)
+    yr.backward(dyh[:2])
+
+    def rel(a, b):
+        return float((a.cpu().double() - b.double()).abs().max() / b.double().abs().max())
+    return {'step': 'forward + data gradient + weight gradient, fp32 products', 'ms_per_step': ms,
+            'frac': flops / (ms * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 'bound': 'mfma fp32',
+            'tflops': flops / (ms * 1e-3) / 1e12,
+            'parity_max_rel': {'forward': rel(y[:2], yr.detach()), 'data_gradient': rel(dx[:2], xr.grad)},
+            'parity_sample': 'first 2 images against torch conv2d on the CPU'}
 
 
 def bench_conv(args):
@@ -204,6 +339,10 @@ def main():
                          'the reference interface, and the default here, is nchw)')
     ap.add_argument('--conv-compute', default='fp32', choices=['fp32', 'bf16', 'bf16x3'],
                     help='cfg5 only: how the convolution forms its products')
+    ap.add_argument('--traffic-file', default=os.path.join(ROOT, 'profiles', 'roialign_cfg2_hbm_traffic.txt'),
+                    help='counter summary that roofline.traffic is read from (cfg2, NCHW)')
+    ap.add_argument('--no-other-configs', action='store_true',
+                    help='leave out the short runs of the other BASELINE configurations (the "configs" object)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build measures one GPU only (the path would shard by image, each GPU '
@@ -397,8 +536,10 @@ def main():
             'step': 'forward + backward(assign)' if has_bwd else 'forward'},
         'roofline': {'bound': 'hbm', 'kernel': dom_kernel, 'achieved': gbs(dom_bytes, dom_ms),
                      'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': gbs(dom_bytes, dom_ms) / HBM_PEAK_GBS,
-                     'traffic': None if nhwc else MEASURED_TRAFFIC.get((w['name'], dom_kernel)),
-                     'algorithmic_bytes': dom_bytes, 'avg_ms': dom_ms},
+                     'traffic': None if nhwc or w['name'] != 'cfg2' else measured_traffic(args.traffic_file, dom_kernel),
+                     'algorithmic_bytes': dom_bytes, 'avg_ms': dom_ms,
+                     # the whole step (every helper kernel and gap included) on the algorithmic bytes of both passes
+                     'step_frac': total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
         'kernels_ms': kernel_ms,
         'passes': passes,
         # share of the map inside some ROI's box: the e*|x| term of the algorithmic bytes counts all of it
@@ -424,6 +565,17 @@ def main():
                 dx_n = abi.backward(dy_nchw, part, x_nchw.shape, scale, S, assign=True).cpu().numpy()
             return y_n.cpu().numpy(), dx_n
         out['cpu_baseline'] = cpu_baseline(w, gpu_result=gpu_result)
+    if args.workload == 'cfg2' and not args.no_other_configs and not nhwc and args.sampling_ratio is None:
+        # the other configurations of BASELINE.json, a few steps each (parity cases, shown
+        # for orientation; `value` above is cfg2 alone)
+        del x, dy, dx
+        torch.cuda.empty_cache()
+        out['configs'] = {'cfg2': {'step': 'forward + backward(assign)', 'ms_per_step': ms_per_step,
+                                   'frac': total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}}
+        for name in ('cfg1', 'cfg3', 'cfg4'):
+            out['configs'][name] = short_roialign_run(name)
+            torch.cuda.empty_cache()
+        out['configs']['cfg5'] = short_conv_run()
     print(json.dumps(out))
 
 
