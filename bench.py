@@ -341,6 +341,8 @@ def main():
                     help='cfg5 only: how the convolution forms its products')
     ap.add_argument('--traffic-file', default=os.path.join(ROOT, 'profiles', 'roialign_cfg2_hbm_traffic.txt'),
                     help='counter summary that roofline.traffic is read from (cfg2, NCHW)')
+    ap.add_argument('--option', action='append', default=[], metavar='NAME=VALUE',
+                    help='set a library option (mobula_hip_set_option) before the run, for experiments')
     ap.add_argument('--no-other-configs', action='store_true',
                     help='leave out the short runs of the other BASELINE configurations (the "configs" object)')
     args = ap.parse_args()
@@ -355,6 +357,10 @@ def main():
     from mobulaop_amd import workloads
     from mobulaop_amd import abi
     assert torch.cuda.is_available(), 'bench.py needs a GPU'
+    for item in args.option:
+        from mobulaop_amd import native
+        name, _, value = item.partition('=')
+        native.set_option(name, int(value))
 
     w = workloads.make_workload(args.workload)
     if args.sampling_ratio is not None:
