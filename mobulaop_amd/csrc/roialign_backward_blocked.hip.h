@@ -16,8 +16,9 @@
 // Pooled columns whose cells may coincide are taken in separate turns (the
 // pre-pass stores the spacing at which they cannot).
 //
-// dy is read from a channel-blocked copy dyb[R][C/32][PH][PWp][32] (PWp = PW
-// rounded up to 8): one 16-byte load per lane fetches a pooled row (1 KB).
+// dy is read from a channel-blocked copy dyb[C/32][R][PH][PWp][32] (PWp = PW
+// rounded up to 8): one 16-byte load per lane fetches a pooled row (1 KB); the
+// slab of a channel block is addressed with 32-bit offsets (up to 2 GiB each).
 #pragma once
 #include <type_traits>
 
@@ -51,61 +52,92 @@ inline int backward_tile_columns(long long images, int H, int W, int cblk) {
   return wide * kTileRows * cblk < 8192 ? BwdBlocked::TW_SMALL : BwdBlocked::TW;
 }
 
-// dy[r][c][ph][pw] -> dyb[r][cb][ph][PWp][32], zero where pw >= PW or the channel
+// dy[r][c][ph][pw] -> dyb[cb][r][ph][PWp][32] (R: number of ROIs), zero where pw >= PW or the channel
 // does not exist.  One workgroup per (ROI, group of `per` channel blocks):
 // the input words of the group are contiguous and so are its output words.
 // LDS holds the input as it is; the transposition happens in the reads.
 // T is the element type of dy (float or __half); dyb is fp32 either way.
 // `block`: index among the workgroups (of 256 threads) that transpose.
+// `cap`: channels LDS holds at a time.  With per >= 1 whole blocks fit (cap is not used);
+// per == 0 says that not even one block does (large pooled sizes): the workgroup then takes one
+// channel block in passes of `cap` channels (a multiple of 4).
 template <typename T>
 __device__ __forceinline__ void transpose_dy_blocked_body(unsigned block, const T* __restrict__ dy,
                                                           float* __restrict__ dyb, int C, int PH, int PW,
-                                                          int PWp, int cblk, int per) {
+                                                          int PWp, int cblk, int per, int R, int cap) {
   constexpr int CB = BwdBlocked::CB;
   constexpr int VEC = 16 / sizeof(T);   // elements per 16-byte word
-  extern __shared__ __attribute__((aligned(16))) unsigned char tbuf_bytes[];   // [per * 32][PH * PW] of T
+  extern __shared__ __attribute__((aligned(16))) unsigned char tbuf_bytes[];   // [channels][PH * PW] of T
   T* const tbuf = reinterpret_cast<T*>(tbuf_bytes);
-  const int groups = (cblk + per - 1) / per;
+  const int blocks_per_group = per > 0 ? per : 1;
+  const int groups = (cblk + blocks_per_group - 1) / blocks_per_group;
   const int r = block / groups, grp = block % groups;
-  const int cb0 = grp * per, nblk = min(per, cblk - cb0);
+  const int cb0 = grp * blocks_per_group, nblk = min(blocks_per_group, cblk - cb0);
   const int c0 = cb0 * CB, nch = min(nblk * CB, C - c0);
   const int bins = PH * PW;
-  const T* src = dy + (static_cast<size_t>(r) * C + c0) * bins;
-  const int n_in = nch * bins;
-  if ((reinterpret_cast<size_t>(src) & 15) == 0) {
-    const int nvec = n_in / VEC;
-    typedef float f32x4 __attribute__((ext_vector_type(4)));
-    for (int i = threadIdx.x; i < nvec; i += 256)   // dy is read once: no need to keep it in the caches
-      reinterpret_cast<f32x4*>(tbuf)[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src) + i);
-    for (int i = VEC * nvec + threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
-  } else {
-    for (int i = threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
-  }
-  __syncthreads();
-  float* dst = dyb + (static_cast<size_t>(r) * cblk + cb0) * PH * PWp * CB;
-  const int per_blk = PH * PWp * (CB / 4);   // 16-byte pieces of one channel block
-  for (int q = threadIdx.x; q < nblk * per_blk; q += 256) {
-    const int blk = q / per_blk, p = q - blk * per_blk;
-    const int cq = p & 7, cell = p >> 3, pw = cell % PWp, ph = cell / PWp;
-    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    if (pw < PW) {
-      const int c = blk * CB + 4 * cq;
-      const T* in = tbuf + c * bins + ph * PW + pw;
-      if (c + 0 < nch) v.x = to_float(in[0]);
-      if (c + 1 < nch) v.y = to_float(in[bins]);
-      if (c + 2 < nch) v.z = to_float(in[2 * bins]);
-      if (c + 3 < nch) v.w = to_float(in[3 * bins]);
+  const int pass_ch = per > 0 ? nch : cap;
+  typedef float f32x4s __attribute__((ext_vector_type(4)));
+  for (int pc = 0; pc < nch; pc += pass_ch) {
+    const int pn = min(pass_ch, nch - pc);
+    const T* src = dy + (static_cast<size_t>(r) * C + c0 + pc) * bins;
+    const int n_in = pn * bins;
+    if (pc > 0) __syncthreads();   // the previous pass has been read
+    if ((reinterpret_cast<size_t>(src) & 15) == 0) {
+      const int nvec = n_in / VEC;
+      typedef float f32x4 __attribute__((ext_vector_type(4)));
+      for (int i = threadIdx.x; i < nvec; i += 256)   // dy is read once: no need to keep it in the caches
+        reinterpret_cast<f32x4*>(tbuf)[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src) + i);
+      for (int i = VEC * nvec + threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
+    } else {
+      for (int i = threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
     }
-    typedef float f32x4s __attribute__((ext_vector_type(4)));
-    __builtin_nontemporal_store(f32x4s{v.x, v.y, v.z, v.w}, reinterpret_cast<f32x4s*>(dst + static_cast<size_t>(q) * 4));
+    __syncthreads();
+    const int per_blk = PH * PWp * (CB / 4);   // 16-byte pieces of one channel block
+    if (per > 0) {
+      for (int q = threadIdx.x; q < nblk * per_blk; q += 256) {
+        const int blk = q / per_blk, p = q - blk * per_blk;
+        // every channel block has a slab of its own (all ROIs): its owners address it with 32-bit offsets
+        float* const dst = dyb + (static_cast<size_t>(cb0 + blk) * R + r) * PH * PWp * CB;
+        const int cq = p & 7, cell = p >> 3, pw = cell % PWp, ph = cell / PWp;
+        float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (pw < PW) {
+          const int c = blk * CB + 4 * cq;
+          const T* in = tbuf + c * bins + ph * PW + pw;
+          if (c + 0 < nch) v.x = to_float(in[0]);
+          if (c + 1 < nch) v.y = to_float(in[bins]);
+          if (c + 2 < nch) v.z = to_float(in[2 * bins]);
+          if (c + 3 < nch) v.w = to_float(in[3 * bins]);
+        }
+        __builtin_nontemporal_store(f32x4s{v.x, v.y, v.z, v.w}, reinterpret_cast<f32x4s*>(dst + static_cast<size_t>(p) * 4));
+      }
+    } else {
+      // the channel quads pc / 4 .. of the one block: 16-byte pieces, the quads of a cell side by side;
+      // the last pass also writes the zero quads of channels that do not exist
+      float* const dst = dyb + (static_cast<size_t>(cb0) * R + r) * PH * PWp * CB;
+      const int q0 = pc / 4, nq = pc + pass_ch >= nch ? CB / 4 - q0 : pn / 4;
+      for (int q = threadIdx.x; q < nq * PH * PWp; q += 256) {
+        const int cell = q / nq, qi = q - cell * nq, pw = cell % PWp, ph = cell / PWp;
+        float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (pw < PW) {
+          const int c = 4 * qi;   // within the pass
+          const T* in = tbuf + c * bins + ph * PW + pw;
+          if (c + 0 < pn) v.x = to_float(in[0]);
+          if (c + 1 < pn) v.y = to_float(in[bins]);
+          if (c + 2 < pn) v.z = to_float(in[2 * bins]);
+          if (c + 3 < pn) v.w = to_float(in[3 * bins]);
+        }
+        __builtin_nontemporal_store(f32x4s{v.x, v.y, v.z, v.w},
+                                    reinterpret_cast<f32x4s*>(dst + (static_cast<size_t>(cell) * 8 + q0 + qi) * 4));
+      }
+    }
   }
 }
 
 template <typename T>
 __global__ void __launch_bounds__(256)
 transpose_dy_blocked_kernel(const T* __restrict__ dy, float* __restrict__ dyb, int C, int PH,
-                            int PW, int PWp, int cblk, int per) {
-  transpose_dy_blocked_body<T>(blockIdx.x, dy, dyb, C, PH, PW, PWp, cblk, per);
+                            int PW, int PWp, int cblk, int per, int R, int cap) {
+  transpose_dy_blocked_body<T>(blockIdx.x, dy, dyb, C, PH, PW, PWp, cblk, per, R, cap);
 }
 
 // Both in one launch, for inputs too small to be worth a second stream: the
@@ -120,7 +152,7 @@ lists_and_dy_kernel(ListsArgs lists, unsigned list_blocks, const T* __restrict__
   if (blockIdx.x < list_blocks)
     build_lists_body(blockIdx.x, lists);
   else
-    transpose_dy_blocked_body<T>(blockIdx.x - list_blocks, dy, dyb, C, lists.PH, lists.PW, PWp, cblk, per);
+    transpose_dy_blocked_body<T>(blockIdx.x - list_blocks, dy, dyb, C, lists.PH, lists.PW, PWp, cblk, per, lists.R, 0);
 }
 
 // Number of workgroups for `tiles` tiles and cblk channel blocks (job decode at
@@ -212,10 +244,12 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
   constexpr unsigned E = sizeof(TI);
   const unsigned dy_pw = (NHWC ? C : K::CB) * E;
   const unsigned dy_ph = static_cast<unsigned>(NHWC ? PW : PWp) * dy_pw;
-  const unsigned dy_roi = NHWC ? dy_ph * PH : dy_ph * PH * cblk;
+  const unsigned dy_roi = dy_ph * PH;
   const unsigned list_roi = static_cast<unsigned>(ll.roi_stride) * sizeof(AxisUnit);
+  // (dyb_bytes: the bytes of one channel block's slab of dyb, or of the caller's whole dy)
   const __amdgpu_buffer_rsrc_t dy_buf = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<void*>(dy_any), 0, static_cast<int>(dyb_bytes), 0x00020000);
+      const_cast<char*>(static_cast<const char*>(dy_any)) + (NHWC ? 0 : static_cast<size_t>(cb) * dyb_bytes), 0,
+      static_cast<int>(dyb_bytes), 0x00020000);
   const __amdgpu_buffer_rsrc_t list_buf = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<AxisUnit*>(lists), 0, static_cast<int>(list_bytes), 0x00020000);
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -226,7 +260,7 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
   // samples of the next are in flight (always eight loads per group, so the
   // wait before a group counts exactly the loads of the group after it).
   for (int pwb = 0; pwb < PW; pwb += K::PWB) {
-    const unsigned dy_fixed = (NHWC ? cb * K::CB * E : cb * dy_ph * PH) + pwb * dy_pw;
+    const unsigned dy_fixed = (NHWC ? cb * K::CB * E : 0u) + pwb * dy_pw;
     const unsigned list_fixed = static_cast<unsigned>(
         (static_cast<long long>(ll.ty) * ll.row_stride + static_cast<long long>(tx) * ll.col_stride + pwb) *
         sizeof(AxisUnit));

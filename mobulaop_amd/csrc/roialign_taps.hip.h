@@ -50,17 +50,19 @@ struct alignas(16) ColPair { int cells; int flags; float l0, l1; };
 constexpr int kColStrideShift = 8;
 constexpr int kColStrideMask = 7;
 
-constexpr int kRowSlots = 32;   // PH * S <= 32 sample rows per ROI
-constexpr int kMaxListPW = 16;  // PW <= 16, one or two sample points per bin
+constexpr int kRowSlots = 64;   // PH * S <= 64 sample rows per ROI (one per lane of the list builder)
+constexpr int kMaxListPW = 32;  // PW * S <= 64 sample columns, one or two sample points per bin
 constexpr int kTileRows = 16;   // rows of a tile (fixed by the row-tap index)
 
 struct RowTap { int ph; float wy; };
-// Row taps of one (roi, tile row): 32-byte index + up to 2*kRowSlots taps.
+// Row taps of one (roi, tile row): 32-byte index + two taps per sample row.  In memory a
+// table ends after the taps its shape can have (ListLayout::row_stride), not after taps[].
 struct alignas(16) RowTapTable {
   unsigned short index[kTileRows];   // start | count << 8, per tile row
   RowTap taps[2 * kRowSlots];
 };
-constexpr int kRowTableUnits = sizeof(RowTapTable) / 16;   // in 16-byte units
+// 16-byte units of a table for `slots` sample rows
+inline int row_table_units(int slots) { return 2 + slots; }
 
 struct ListLayout {
   int ty, tx;            // tiles per image
@@ -69,10 +71,10 @@ struct ListLayout {
   long long roi_stride;  // units per ROI: ty*row_stride + tx*col_stride
 };
 
-inline ListLayout make_list_layout(const TileGrid& tg, int PW) {
+inline ListLayout make_list_layout(const TileGrid& tg, int PH, int PW, int S) {
   ListLayout l;
   l.ty = tg.ty; l.tx = tg.tx;
-  l.row_stride = kRowTableUnits;
+  l.row_stride = row_table_units(PH * (S == 1 ? 1 : 2));
   l.col_stride = (PW + 7) / 8 * 8;
   l.roi_stride = static_cast<long long>(l.ty) * l.row_stride + static_cast<long long>(l.tx) * l.col_stride;
   return l;

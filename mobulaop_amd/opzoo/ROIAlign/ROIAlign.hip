@@ -276,7 +276,7 @@ struct TilePlan {
   roialign::ListLayout layout;
   roialign::AxisUnit* lists;
   float* dyb;                  // channel-blocked copy of dy (null for channels-last tensors)
-  size_t dyb_bytes, list_bytes;
+  size_t dyb_bytes, list_bytes;   // dyb_bytes: of one channel block's slab
   roialign::WorkRange* ranges; // per (tile, tile row)
   roialign::WorkEntry* entries;
 };
@@ -288,15 +288,18 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // on error); the caller then uses the straightforward kernels.
 // How transpose_dy_blocked_kernel is launched for a problem: channel blocks per
 // workgroup (what 64 KB of LDS hold, at most 4; 0: not at all), workgroups, LDS bytes.
-struct DyLaunch { int per; long long blocks; size_t lds; };
+struct DyLaunch { int per; long long blocks; size_t lds; int cap; };
 template <typename T>
 DyLaunch dy_launch(const Problem& p) {
   using BB = roialign::BwdBlocked;
   const int cblk = (p.C + BB::CB - 1) / BB::CB;
-  const size_t blk_bytes = sizeof(T) * BB::CB * p.PH * p.PW;
+  const size_t chan_bytes = sizeof(T) * p.PH * p.PW, blk_bytes = BB::CB * chan_bytes;
   const int per = static_cast<int>(std::min<size_t>(4, (64 * 1024) / blk_bytes));
-  const long long blocks = per > 0 ? static_cast<long long>(p.R) * ((cblk + per - 1) / per) : 0;
-  return DyLaunch{per, blocks, per * blk_bytes};
+  if (per > 0)
+    return DyLaunch{per, static_cast<long long>(p.R) * ((cblk + per - 1) / per), per * blk_bytes, 0};
+  // large pooled sizes: one channel block per workgroup, in passes of `cap` channels
+  const int cap = static_cast<int>((64 * 1024) / chan_bytes) & ~3;
+  return DyLaunch{0, cap >= 4 ? static_cast<long long>(p.R) * cblk : 0, cap * chan_bytes, cap};
 }
 
 // fuse_dy (optional): dy of the call; its transposition into plan->dyb then shares
@@ -334,19 +337,21 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   const size_t b_recs = align_up(sizeof(roialign::TileBox) * std::max<long long>(items, 1), 256);
   const size_t b_cnt = 256;   // the two bump pointers
   const size_t b_list = align_up(sizeof(int) * std::max<long long>(list_cap, 1), 256);
-  plan->layout = roialign::make_list_layout(g, p.PW);
+  plan->layout = roialign::make_list_layout(g, p.PH, p.PW, p.S);
   const long long n_units = plan->layout.roi_stride * items;
   if (n_units > (1ll << 25)) return false;   // 512 MiB of sample lists: not worth it
   const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256) + 256;  // blocks are read whole
   const int cblk = (p.C + 31) / 32;
-  const size_t b_dyt = with_dyb ? align_up(sizeof(float) * 32 * plan->layout.col_stride * p.R * p.PH * cblk, 256) : 0;
+  // dyb: one slab per channel block (all ROIs), 256-byte aligned
+  const size_t b_slab = with_dyb ? align_up(sizeof(float) * 32 * plan->layout.col_stride * p.R * p.PH, 256) : 0;
+  const size_t b_dyt = b_slab * cblk;
   // work lists: every tap of every ROI once per tile column it spans
   const long long n_entries = items * 2 * p.PH * (p.S == 1 ? 1 : 2) * g.tx +
                               11 * roialign::kTileRows * g.total;
   if (n_entries > (1ll << 27)) return false;
   // the consumer addresses both with 32-bit byte offsets
-  if (b_dyt >= (1ull << 31) || b_units >= (1ull << 31)) return false;
-  plan->dyb_bytes = b_dyt; plan->list_bytes = b_units;
+  if (b_slab >= (1ull << 31) || b_units >= (1ull << 31)) return false;
+  plan->dyb_bytes = b_slab; plan->list_bytes = b_units;
   const size_t b_ranges = align_up(sizeof(roialign::WorkRange) * g.total * roialign::kTileRows, 256);
   const size_t b_entries = align_up(sizeof(roialign::WorkEntry) * n_entries, 256) + 512;
   const size_t b_offsets = pieces ? align_up(sizeof(int) * (p.R + 3), 256) : 0;
@@ -453,11 +458,11 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
     const DyLaunch dl = dy_launch<T>(p);
-    if (grid < (1ll << 31) && dl.blocks < (1ll << 31) && dl.per > 0) {
+    if (grid < (1ll << 31) && dl.blocks < (1ll << 31) && (dl.per > 0 || dl.cap >= 4)) {
       const int pwp = plan.layout.col_stride;
       if (p.R > 0 && !plan.dy_transposed)
         roialign::transpose_dy_blocked_kernel<T><<<static_cast<unsigned>(dl.blocks), 256, dl.lds, stream>>>(
-            dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dl.per);
+            dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dl.per, p.R, dl.cap);
       side.join();
       {
         mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);

@@ -251,6 +251,70 @@ def test_both_tile_widths_of_the_backward(cfg, down, columns):
         assert_parity(got.cpu().numpy(), want, BWD_TOL, 'bwd channels-last')
 
 
+def _last_bracketed_kernel():
+    import ctypes
+    lib = native.library()
+    lib.mobula_hip_last_kernel_ms.restype = ctypes.c_double
+    lib.mobula_hip_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_char_p)]
+    name = ctypes.c_char_p()
+    ms = lib.mobula_hip_last_kernel_ms(ctypes.byref(name))
+    return name.value.decode() if ms >= 0 and name.value else None
+
+
+@pytest.mark.parametrize('pooled,S', [((28, 28), 2), ((32, 20), 2), ((17, 32), 1), ((9, 30), 3)])
+def test_tiled_backward_with_large_pooled_sizes(pooled, S):
+    """Up to 64 sample rows and columns per ROI (32 x 32 bins of 2 x 2 points, mask heads pool 28 x 28)
+    stay on the tile owners; every element against the oracle."""
+    abi.set_impl('tiled')
+    rng = np.random.default_rng(7000 + pooled[0] + S)
+    N, C, H, W, R, scale = 2, 40, 40, 72, 24, 0.25
+    x = rng.random((N, C, H, W), dtype=np.float32)
+    dyh = rng.standard_normal((R, C) + pooled).astype(np.float32)
+    c = np.stack([rng.uniform(0, W / scale, R), rng.uniform(0, H / scale, R)], 1)
+    wh = np.exp(rng.uniform(np.log(4), np.log(1.2 * W / scale), (R, 2)))
+    rois = np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+    native.set_option('kernel_timing', 1)
+    try:
+        dx = abi.backward(abi.to_dev(dyh), abi.to_dev(rois), x.shape, scale, S, assign=True)
+        assert _last_bracketed_kernel() == 'backward_blocked_kernel'
+    finally:
+        native.set_option('kernel_timing', 0)
+    want = oracle.backward(dyh, rois, x.shape, scale, S, impl='ordered')
+    assert_parity(dx.cpu().numpy(), want, BWD_TOL, 'bwd {} S={}'.format(pooled, S))
+    y = abi.forward(abi.to_dev(x), abi.to_dev(rois), pooled, scale, S).cpu().numpy()
+    assert_parity(y, oracle.forward(x, rois, pooled, scale, S), FWD_TOL, 'fwd {} S={}'.format(pooled, S))
+
+
+def test_tiled_backward_beyond_two_gib_of_blocked_gradient():
+    """10000 ROIs x 256 channels x 14 x 14: the channel-blocked copy of dy holds 2.3 GB (every channel block
+    a slab of its own, addressed with 32-bit offsets).  Checked against the straightforward kernel on the
+    same inputs and by the adjoint identity with the forward."""
+    g = torch.Generator(device='cuda').manual_seed(77)
+    N, C, H, W, R, pooled, scale, S = 8, 256, 128, 128, 10000, (14, 14), 0.125, 2
+    size = torch.exp(torch.rand(R, 2, device='cuda', generator=g) * np.log(16.0) + np.log(32.0))
+    centre = torch.rand(R, 2, device='cuda', generator=g) * 1024.0
+    rois = torch.cat([torch.randint(0, N, (R, 1), device='cuda', generator=g).float(), centre - size / 2,
+                      centre + size / 2], 1).contiguous()
+    dy = torch.randn((R, C) + pooled, device='cuda', generator=g)
+    x = torch.rand((N, C, H, W), device='cuda', generator=g)
+    abi.set_impl('tiled')
+    native.set_option('kernel_timing', 1)
+    try:
+        dx = abi.backward(dy, rois, x.shape, scale, S, assign=True)
+        assert _last_bracketed_kernel() == 'backward_blocked_kernel'
+    finally:
+        native.set_option('kernel_timing', 0)
+    y = abi.forward(x, rois, pooled, scale, S)
+    lhs = float((y.double() * dy.double()).sum())
+    rhs = float((x.double() * dx.double()).sum())
+    assert abs(lhs - rhs) <= 1e-6 * float((y.double().abs() * dy.double().abs()).sum())
+    del y
+    abi.set_impl('naive')
+    dx_n = abi.backward(dy, rois, x.shape, scale, S)
+    scale_ = float(dx_n.abs().max())
+    assert float((dx - dx_n).abs().max()) <= BWD_TOL * scale_
+
+
 @pytest.mark.parametrize('columns', [56, 28])
 @pytest.mark.parametrize('S', [0, 3, 4, 5, 7, 65])
 def test_tiled_backward_with_larger_sampling_grids(S, columns):
@@ -364,7 +428,7 @@ def test_channels_last_rejects_what_it_does_not_take():
     rois = torch.tensor([[0, 1, 1, 6, 6]], device='cuda', dtype=torch.float32)
     with pytest.raises(RuntimeError, match='channels-last'):
         abi.forward_nhwc(x, rois, (2, 2), 1.0, 2)
-    dy = torch.zeros(1, 7, 17, 8, device='cuda')         # 17 pooled columns: more than the backward's lists hold
+    dy = torch.zeros(1, 7, 33, 8, device='cuda')         # 33 pooled columns: more than the backward's lists hold
     with pytest.raises(RuntimeError, match='channels-last'):
         abi.backward_nhwc(dy, rois, (1, 8, 8, 8), 1.0, 2)
     dy = torch.zeros(1, 2, 2, 8, device='cuda')          # adaptive grid: whether it fits depends on the boxes
