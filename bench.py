@@ -486,6 +486,7 @@ def main():
         torch.cuda.synchronize()
         assert torch.equal(y_graph, y_eager), 'graph replay and direct calls differ'
         del graph, y_graph, y_eager
+        native.unpin_workspace()   # recording pinned the thread's workspace
 
     # Backward twice from the same inputs: the largest difference between the two
     # results (the reference's atomics give a different summation order each run).

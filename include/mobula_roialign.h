@@ -310,11 +310,14 @@ int mobula_hip_device_count(void);
  * none).  workspace_bytes: its current size for the calling thread on the
  * current device.  release_workspace: gives it back to the device (waits for the
  * work that still uses it) and returns the bytes freed; the next call allocates
- * afresh.  A HIP graph recorded from calls of this thread refers to the buffer:
- * it must not be replayed after a release, and its replays are not ordered
- * against the thread's calls on other streams (the caller orders those). */
+ * afresh.  A HIP graph recorded from calls of this thread refers to the buffer
+ * by address: a call on a capturing stream pins it, and a pinned buffer is
+ * neither released nor replaced by a larger one (such a call fails with an
+ * error instead) until unpin_workspace() says the graphs are gone.  Replays are
+ * not ordered against the thread's calls on other streams (the caller orders those). */
 long long mobula_hip_workspace_bytes(void);
 long long mobula_hip_release_workspace(void);
+void mobula_hip_unpin_workspace(void);
 
 /* 1 if a kernel may dereference p (device, pinned or managed memory), else 0. */
 int mobula_hip_device_can_read(const void* p);

@@ -42,6 +42,9 @@ long long arg_extent(int index);
 // point ends with finish_call(), which keeps the book for that.
 void* workspace(size_t bytes);
 long long release_workspace();   // frees the calling thread's buffer on the current device
+// A call recorded into a HIP graph pins the buffer (replays use its address): it is then
+// neither grown nor released (an error instead) until unpin_workspace().
+void unpin_workspace();
 long long workspace_bytes();
 
 long long option(const char* name, long long fallback);

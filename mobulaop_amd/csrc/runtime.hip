@@ -41,6 +41,8 @@ struct Scratch {
   hipStream_t last = nullptr;   // stream of the last call that used the buffer
   hipEvent_t idle = nullptr;    // recorded behind that call when it did not wait itself
   bool busy = false;            // `idle` is recorded and not known to have passed
+  bool pinned = false;          // a call was recorded into a HIP graph while using the buffer:
+                                // replays use this very address, so it is neither freed nor moved
 };
 struct ScratchOfThread {
   std::map<int, Scratch> per_device;
@@ -69,6 +71,20 @@ void* workspace(size_t bytes) {
     MOBULA_HIP_TRY(hipStreamWaitEvent(st.stream, s->idle, 0));
     if (failed()) return nullptr;
   }
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (st.stream != nullptr && hipStreamIsCapturing(st.stream, &capture) != hipSuccess) {
+    (void)hipGetLastError();
+    capture = hipStreamCaptureStatusNone;
+  }
+  const bool capturing = capture == hipStreamCaptureStatusActive;
+  if (s->bytes < bytes && (capturing || s->pinned)) {
+    set_error("the workspace of this thread (%zu bytes) is too small for the call (%zu bytes) and cannot be "
+              "replaced %s: make one ordinary call of the largest shape before recording, or call "
+              "mobula_hip_unpin_workspace() once the graphs are gone", s->bytes, bytes,
+              capturing ? "while the stream is being captured" : "because a recorded graph uses it");
+    return nullptr;
+  }
+  if (capturing) s->pinned = true;
   if (s->bytes < bytes) {
     if (s->ptr != nullptr) MOBULA_HIP_TRY(hipFree(s->ptr));  // waits for pending work
     s->ptr = nullptr;
@@ -88,6 +104,11 @@ void* workspace(size_t bytes) {
 long long release_workspace() {
   Scratch* const s = scratch_of_current_device();
   if (s == nullptr || s->ptr == nullptr) return 0;
+  if (s->pinned) {
+    set_error("the workspace of this thread is used by a recorded graph: call mobula_hip_unpin_workspace() "
+              "once the graph is gone");
+    return 0;
+  }
   const long long bytes = static_cast<long long>(s->bytes);
   MOBULA_HIP_TRY(hipFree(s->ptr));
   s->ptr = nullptr;
@@ -95,6 +116,11 @@ long long release_workspace() {
   s->busy = false;
   s->last = nullptr;
   return failed() ? 0 : bytes;
+}
+
+void unpin_workspace() {
+  Scratch* const s = scratch_of_current_device();
+  if (s != nullptr) s->pinned = false;
 }
 
 long long workspace_bytes() {
@@ -320,7 +346,12 @@ double mobula_hip_last_kernel_ms(const char** name) {
 }
 
 long long mobula_hip_workspace_bytes(void) { return mobula_hip::workspace_bytes(); }
-long long mobula_hip_release_workspace(void) { return mobula_hip::release_workspace(); }
+long long mobula_hip_release_workspace(void) {
+  mobula_hip::begin_call();
+  return mobula_hip::release_workspace();
+}
+// The calling thread's workspace on the current device is no longer used by any recorded graph.
+void mobula_hip_unpin_workspace(void) { mobula_hip::unpin_workspace(); }
 
 // 1 if a kernel may dereference p: device memory, or host memory the device
 // reaches (pinned, managed); 0 for ordinary host memory and for null.

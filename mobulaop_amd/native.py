@@ -114,10 +114,24 @@ def workspace_bytes():
 
 def release_workspace():
     """Give the calling thread's scratch buffer back to the device; returns the
-    bytes freed.  The next call allocates what it needs."""
-    fn = library().mobula_hip_release_workspace
+    bytes freed.  The next call allocates what it needs.  Refused (RuntimeError)
+    while a recorded HIP graph uses the buffer: see unpin_workspace()."""
+    lib = library()
+    fn = lib.mobula_hip_release_workspace
     fn.restype = ctypes.c_longlong
-    return int(fn())
+    freed = int(fn())
+    msg = lib.mobula_hip_last_error()
+    if msg:
+        text = msg.decode()
+        lib.mobula_hip_clear_error()
+        raise RuntimeError(text)
+    return freed
+
+
+def unpin_workspace():
+    """Tell the library that no recorded HIP graph uses the calling thread's scratch
+    buffer any more (recording a call pins it: it is then neither grown nor released)."""
+    library().mobula_hip_unpin_workspace()
 
 
 def begin_call(stream, extents):

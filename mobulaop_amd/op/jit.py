@@ -165,6 +165,34 @@ def _build_dir(source):
     return path
 
 
+_INCLUDE = re.compile(r'^[ \t]*#[ \t]*include[ \t]*"([^"]+)"', re.M)
+
+
+def source_dependencies(source):
+    """`source` and every file it includes with #include "...", recursively, looked up
+    beside the including file, then in the dialect's and the launcher's include
+    directories (what the compiler is given with -I).  The reference walks the same graph
+    before it decides to rebuild (mobula/building/build_utils.py: dependant files)."""
+    seen, stack = [], [os.path.abspath(source)]
+    while stack:
+        path = stack.pop()
+        if path in seen:
+            continue
+        seen.append(path)
+        try:
+            with open(path, 'r', errors='replace') as fin:
+                text = fin.read()
+        except OSError:
+            continue
+        for name in _INCLUDE.findall(text):
+            for base in (os.path.dirname(path), INC_PATH, CSRC_PATH):
+                cand = os.path.normpath(os.path.join(base, name))
+                if os.path.isfile(cand):
+                    stack.append(cand)
+                    break
+    return sorted(seen)
+
+
 def compile_instantiation(cfunc, arg_types, source, symbol):
     """Path of the shared object that exports `symbol`; built if it is not there
     (or was built from another version of the source or of the headers)."""
@@ -177,8 +205,10 @@ def compile_instantiation(cfunc, arg_types, source, symbol):
     code = wrapper_source(cfunc, arg_types, source, symbol, include)
     digest = hashlib.md5()
     digest.update(code.encode())
-    for dep in (source, os.path.join(INC_PATH, 'mobula_op.h'), os.path.join(INC_PATH, 'mobula_jit.h'),
-                os.path.join(CSRC_PATH, 'runtime.h')):
+    deps = set(source_dependencies(source))
+    for header in (os.path.join(INC_PATH, 'mobula_op.h'), os.path.join(INC_PATH, 'mobula_jit.h')):
+        deps.update(source_dependencies(header))   # (the wrapper includes these two itself)
+    for dep in sorted(deps):
         with open(dep, 'rb') as fin:
             digest.update(fin.read())
     stem = '{}_{}'.format(symbol, digest.hexdigest()[:10])

@@ -335,6 +335,25 @@ def test_a_changed_source_is_rebuilt_and_a_broken_one_reports_the_compiler(tmp_p
     assert not [f for f in os.listdir(str(op_dir / 'build')) if '.tmp.' in f]   # nothing half-written stays
 
 
+def test_a_changed_header_of_the_source_is_rebuilt(tmp_path):
+    # headers the operator source includes itself are part of what a build is named by
+    op_dir = tmp_path / 'Dep'
+    op_dir.mkdir()
+    (op_dir / 'inner.h').write_text('#define DEP_VALUE 5\n')
+    (op_dir / 'outer.h').write_text('#include "inner.h"\n')
+    source = op_dir / 'Dep.cpp'
+    source.write_text('#include "outer.h"\nMOBULA_FUNC int dep_value() { return DEP_VALUE; }\n')
+    deps = jit.source_dependencies(str(source))
+    assert [os.path.basename(d) for d in deps] == ['Dep.cpp', 'inner.h', 'outer.h']
+    mobula.op.load('Dep', str(tmp_path))
+    decl = mobula.func.dep_value.func
+    first = jit.compile_instantiation(decl, [], str(source), 'dep_value_d41d8cd9')
+    assert ctypes.CDLL(first).dep_value_d41d8cd9() == 5
+    (op_dir / 'inner.h').write_text('#define DEP_VALUE 6\n')
+    second = jit.compile_instantiation(decl, [], str(source), 'dep_value_d41d8cd9')
+    assert second != first and ctypes.CDLL(second).dep_value_d41d8cd9() == 6
+
+
 _CONCURRENT_LOAD = r'''
 import ctypes, os, sys
 sys.path.insert(0, sys.argv[1])

@@ -541,6 +541,8 @@ def test_calls_recorded_in_a_graph_replay_bit_for_bit(layout):
         stream.synchronize()
         return y.clone(), dx.clone()
 
+    torch.cuda.synchronize()
+    native.release_workspace()   # (earlier tests may have left a larger one: this test wants it sized by its own calls)
     y_want, dx_want = direct()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=stream):
@@ -556,6 +558,26 @@ def test_calls_recorded_in_a_graph_replay_bit_for_bit(layout):
         assert torch.equal(dx, dx_want), 'backward, replay %d' % replay
         y_now, dx_now = direct()            # ordinary calls between the replays
         assert torch.equal(y_now, y_want) and torch.equal(dx_now, dx_want)
+    # the graph refers to the workspace by address: while it may be replayed the buffer is
+    # neither given back nor replaced by a larger one (host-side book-keeping, nothing faults)
+    held = native.workspace_bytes()
+    with pytest.raises(RuntimeError, match='recorded graph'):
+        native.release_workspace()
+    big = torch.zeros((8, 256, 200, 336), device='cuda')
+    if nhwc:
+        big = big.permute(0, 2, 3, 1).contiguous()
+    dy_big = torch.zeros_like(abi.to_dev(w['dy'].transpose(0, 2, 3, 1) if nhwc else w['dy'])).repeat(3, 1, 1, 1)
+    rois_big = rois.repeat(3, 1)
+    with pytest.raises(RuntimeError, match='recorded graph'):
+        bwd(dy_big, rois_big, big.shape, scale, S, assign=True)
+    assert native.workspace_bytes() == held
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(dx, dx_want)
+    del graph
+    native.unpin_workspace()
+    assert bwd(dy_big, rois_big, big.shape, scale, S, assign=True).shape == big.shape
+    assert native.workspace_bytes() > held
 
 
 @pytest.mark.parametrize('impl', IMPLS)
