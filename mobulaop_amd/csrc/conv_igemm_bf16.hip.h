@@ -1,0 +1,424 @@
+// The two gathered products of the convolution (forward, data gradient) with
+// bf16 operands in memory.
+//
+// conv_igemm.hip.h rounds fp32 operands to bf16 on their way into LDS; that mode
+// is bound by fetching the fp32 operands (sixteen 4-byte loads per lane and K
+// step) and converting them, not by the matrix cores.  Here a pre-pass writes
+// bf16 copies laid out so that one K step of a tile is contiguous memory:
+//   * the gathered tensor (x for the forward, dy for the data gradient) as
+//     [image][channel block][pixel][32 channels], channels padded with zeros to
+//     a multiple of 32: the 32 channels of a K step at one pixel are 64
+//     contiguous bytes, and neighbouring pixels follow;
+//   * the weights as [K step][row][32 channels] (rows and channels padded with
+//     zeros): the rows of a tile in one K step are one contiguous run.
+// (With rows of a K step a large power-of-two stride apart -- [row][K] weights,
+// [pixel][channel] activations -- all rows of a step fall into four of an L2's
+// sixteen channels, and the product runs at the pace of those four.)
+//
+// K runs in steps of 32 channels, the taps of a channel block one after the other
+// (step = block * taps + tap): the taps of a block read the same 64-byte pieces of
+// the same pixels, so after the first tap a step's gathered operand comes from
+// the L1 and L2 caches.  A workgroup of four
+// wavefronts owns a tile of 256 x 256 (each wavefront 128 x 128: 4 x 4
+// accumulators of v_mfma_f32_32x32x16_bf16, 256 accumulator registers, one
+// workgroup per CU), or 128 x 256 for products of at most 128 rows (each
+// wavefront 128 x 64).  A tile this large needs 64 bytes from memory and 128
+// bytes from LDS per matrix instruction, half of what 128 x 128 tiles need.
+//
+// Operands go from memory straight into LDS (buffer loads with the LDS flag,
+// 16 bytes per lane: one instruction moves sixteen 64-byte rows), three stages
+// deep: while step s is multiplied, step s + 1 has landed or is landing and
+// step s + 2 is requested.  No register staging, no LDS store instructions.
+// A column in the padding loads from beyond the buffer, which writes zeros.
+// LDS rows are 64 bytes with no padding; the four 16-byte chunks of row r sit
+// in slots chunk ^ ((r >> 2) & 3), which puts the 16-byte fragment reads of
+// sixteen neighbouring rows on all 64 banks, each once.
+//
+// Replaces, like conv_igemm.hip.h, the per-image im2col + matrix product of
+// opzoo/Convolution/Convolution.py:17-57.
+#pragma once
+#include "conv_igemm.hip.h"
+
+namespace conv {
+
+struct TileB16 {
+  static constexpr int BN = 256, BK = 32, STAGES = 3;
+  static constexpr int NT = 256;
+};
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+// dst[n][c / 32][p][c % 32] = bf16(src[n][c][p]) for c < C, zero for C <= c < Cpad.  One
+// workgroup: 64 pixels x 64 channels (two channel blocks) through LDS.
+__global__ void __launch_bounds__(256)
+to_blocked_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst, int C, int Cpad, int P) {
+  __shared__ float tile[64][65];
+  const int n = blockIdx.z, c0 = blockIdx.y * 64, p0 = blockIdx.x * 64;
+  const float* in = src + static_cast<size_t>(n) * C * P;
+  {
+    const int px = threadIdx.x & 63, cr = threadIdx.x >> 6;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int c = c0 + cr + 4 * k, p = p0 + px;
+      tile[cr + 4 * k][px] = (c < C && p < P) ? in[static_cast<size_t>(c) * P + p] : 0.0f;
+    }
+  }
+  __syncthreads();
+  // a thread: one pixel, 8 channels (16 bytes); four threads cover a pixel of one channel block
+  const int cq = threadIdx.x & 3, pl = (threadIdx.x >> 2) & 63;
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {   // the two channel blocks
+    const int p = p0 + pl, cl = 32 * k + 8 * cq, c = c0 + cl;
+    if (p < P && c < Cpad) {
+      u32x4 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = pack_bf16(tile[cl + 2 * j][pl], tile[cl + 2 * j + 1][pl]);
+      *reinterpret_cast<u32x4*>(dst + ((static_cast<size_t>(n) * (Cpad / 32) + c / 32) * P + p) * 32 + 8 * cq) = v;
+    }
+  }
+}
+
+// out[(c / 32) * taps + tap][m][c % 32] = bf16(w[m * stride_m + c * stride_c + tap]) for m < M and
+// c < C, else 0 (m < Mpad, c < Cpad).
+__global__ void __launch_bounds__(256)
+arrange_weights_bf16_kernel(const float* __restrict__ w, unsigned short* __restrict__ out, int M, int Mpad,
+                            int C, int Cpad, int taps, long long stride_m, long long stride_c) {
+  const long long total = static_cast<long long>(Mpad) * taps * Cpad / 2;   // pairs of channels
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int j = 2 * static_cast<int>(i % 16), m = static_cast<int>((i / 16) % Mpad);
+  const int s = static_cast<int>(i / (16ll * Mpad));
+  const int cb = s / taps, tap = s - cb * taps, c = cb * 32 + j;
+  const float lo = (m < M && c < C) ? w[m * stride_m + c * stride_c + tap] : 0.0f;
+  const float hi = (m < M && c + 1 < C) ? w[m * stride_m + (c + 1) * stride_c + tap] : 0.0f;
+  reinterpret_cast<unsigned*>(out)[i] = pack_bf16(lo, hi);
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of_bytes(const void* base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+// Row coordinate of a column that does not exist: fails every bounds test, whatever tap is added.
+constexpr int kFarOutside = -(1 << 30);
+
+// A K step as (filter row, filter column, channel block); wavefront-uniform, kept in scalar registers.
+struct StepCursor { int kh, kw, cb; };
+
+// What the operand functors of igemm_tile_b16 have in common: the weights and the walk over K.
+struct GatheredB16 {
+  const unsigned short* __restrict__ wp;    // [K / 32][mpad][32]
+  const unsigned short* __restrict__ src;   // [images][cpad / 32][pixels][32]
+  Geometry g; int M, Ncols, K, cpad, mpad;
+  __device__ __amdgpu_buffer_rsrc_t a_buffer() const {
+    return buffer_of_bytes(wp, static_cast<unsigned>(mpad) * static_cast<unsigned>(K) * 2u);
+  }
+  __device__ int a_offset(int m) const { return m * 64; }
+  __device__ int a_step_offset(int s) const { return s * mpad * 64; }
+  __device__ StepCursor cursor(int s) const {
+    const int taps = g.KH * g.KW, cb = s / taps, tap = s - cb * taps, kh = tap / g.KW;
+    return StepCursor{kh, tap - kh * g.KW, cb};
+  }
+  __device__ void advance(StepCursor& c) const {
+    if (++c.kw == g.KW) { c.kw = 0; if (++c.kh == g.KH) { c.kh = 0; ++c.cb; } }
+  }
+  // the images from the one column n0 lies in, as a raw buffer
+  __device__ __amdgpu_buffer_rsrc_t images_from(int first, size_t image_bytes) const {
+    const size_t skip = static_cast<size_t>(first) * image_bytes, left = static_cast<size_t>(g.N) * image_bytes - skip;
+    return buffer_of_bytes(reinterpret_cast<const char*>(src) + skip,
+                           static_cast<unsigned>(left < kRecordLimit ? left : kRecordLimit));
+  }
+};
+
+// Operand functors of igemm_tile_b16:
+//   Step step_at(cursor): what a K step adds to every column's offset (uniform);
+//   b_buffer(n0): the gathered tensor from the first image of the tile on;
+//   BCtx b_ctx(n, n0): what column n needs throughout;
+//   b_offset(ctx, step, chunk): byte offset of the column's 16-byte chunk in that buffer (kDead: zeros);
+//   Column column(n) / store(column, m, v): where results of column n go.
+
+// y[img, d, oh, ow] = bias[d] + sum over (c, kh, kw) of W[d, c, kh, kw] * x[img, c, ih, iw]
+struct ForwardOpsB16 : GatheredB16 {
+  const float* __restrict__ bias; float* __restrict__ y;
+  struct Step { int dh, dw, delta; };
+  struct BCtx { int anchor, ih0, iw0; };   // (a column past the last: ih0 far outside)
+  struct Column { float* p; bool ok; };
+  __device__ int plane_bytes() const { return g.H * g.W * 64; }
+  __device__ Step step_at(const StepCursor& c) const {
+    const int dh = c.kh * g.dil_h, dw = c.kw * g.dil_w;
+    return Step{dh, dw, c.cb * plane_bytes() + (dh * g.W + dw) * 64};
+  }
+  __device__ __amdgpu_buffer_rsrc_t b_buffer(int n0) const {
+    return images_from(__builtin_amdgcn_readfirstlane(n0 / (g.OH * g.OW)), static_cast<size_t>(plane_bytes()) * (cpad / 32));
+  }
+  __device__ BCtx b_ctx(int n, int n0) const {
+    BCtx c;
+    const int ohw = g.OH * g.OW, first = n0 / ohw;
+    const int img = n / ohw, r = n - img * ohw, oh = r / g.OW, ow = r - oh * g.OW;
+    c.ih0 = n < Ncols ? oh * g.stride_h - g.pad_h : kFarOutside;
+    c.iw0 = ow * g.stride_w - g.pad_w;
+    c.anchor = (img - first) * plane_bytes() * (cpad / 32) + (c.ih0 * g.W + c.iw0) * 64;
+    return c;
+  }
+  __device__ int b_offset(const BCtx& c, const Step& e, int chunk) const {
+    const int ih = c.ih0 + e.dh, iw = c.iw0 + e.dw;
+    const bool in = (static_cast<unsigned>(ih) < static_cast<unsigned>(g.H)) &
+                    (static_cast<unsigned>(iw) < static_cast<unsigned>(g.W));
+    return in ? c.anchor + e.delta + chunk * 16 : kDead;
+  }
+  __device__ Column column(int n) const {
+    const int ohw = g.OH * g.OW, img = n / ohw, r = n - img * ohw;
+    return Column{y + static_cast<size_t>(img) * g.D * ohw + r, n < Ncols};
+  }
+  __device__ void store(const Column& c, int m, float v) const {
+    if (m < M && c.ok) c.p[static_cast<size_t>(m) * (g.OH * g.OW)] = bias != nullptr ? v + bias[m] : v;
+  }
+};
+
+// dx[img, c, ih, iw] = sum over (d, kh, kw) of W[d, c, kh, kw] * dy[img, d, oh, ow]
+// with oh * stride = ih + pad - kh * dil (and likewise for columns).
+struct BackwardDataOpsB16 : GatheredB16 {
+  float* __restrict__ dx; int accumulate;
+  struct Step { int dh, dw, delta; };
+  struct BCtx { int anchor, ihp, iwp; };   // (a column past the last: ihp far outside)
+  struct Column { float* p; bool ok; };
+  __device__ bool unit_stride() const { return g.stride_h == 1 && g.stride_w == 1; }
+  __device__ int plane_bytes() const { return g.OH * g.OW * 64; }
+  __device__ Step step_at(const StepCursor& c) const {
+    const int dh = c.kh * g.dil_h, dw = c.kw * g.dil_w;
+    // stride 1: the tap's offset from the anchor pixel (ih + pad, iw + pad) of dy
+    return Step{dh, dw, c.cb * plane_bytes() - (unit_stride() ? (dh * g.OW + dw) * 64 : 0)};
+  }
+  __device__ __amdgpu_buffer_rsrc_t b_buffer(int n0) const {
+    return images_from(__builtin_amdgcn_readfirstlane(n0 / (g.H * g.W)), static_cast<size_t>(plane_bytes()) * (cpad / 32));
+  }
+  __device__ BCtx b_ctx(int n, int n0) const {
+    BCtx c;
+    const int hw = g.H * g.W, first = n0 / hw;
+    const int img = n / hw, r = n - img * hw, ih = r / g.W, iw = r - ih * g.W;
+    c.ihp = n < Ncols ? ih + g.pad_h : kFarOutside; c.iwp = iw + g.pad_w;
+    // stride 1: byte offset of dy[img, block 0, ihp, iwp]; otherwise of dy[img, block 0, 0, 0]
+    c.anchor = (img - first) * plane_bytes() * (cpad / 32) + (unit_stride() ? (c.ihp * g.OW + c.iwp) * 64 : 0);
+    return c;
+  }
+  __device__ int b_offset(const BCtx& c, const Step& e, int chunk) const {
+    const int th = c.ihp - e.dh, tw = c.iwp - e.dw;
+    if (unit_stride()) {
+      const bool in = (static_cast<unsigned>(th) < static_cast<unsigned>(g.OH)) &
+                      (static_cast<unsigned>(tw) < static_cast<unsigned>(g.OW));
+      return in ? c.anchor + e.delta + chunk * 16 : kDead;
+    }
+    const int oh = th / g.stride_h, ow = tw / g.stride_w;
+    const bool in = (th >= 0) & (tw >= 0) & (oh * g.stride_h == th) & (ow * g.stride_w == tw) &
+                    (oh < g.OH) & (ow < g.OW);
+    return in ? c.anchor + e.delta + (oh * g.OW + ow) * 64 + chunk * 16 : kDead;
+  }
+  __device__ Column column(int n) const {
+    const int hw = g.H * g.W, img = n / hw, r = n - img * hw;
+    return Column{dx + static_cast<size_t>(img) * g.C * hw + r, n < Ncols};
+  }
+  __device__ void store(const Column& c, int m, float v) const {
+    if (m >= M || !c.ok) return;
+    float* p = c.p + static_cast<size_t>(m) * (g.H * g.W);
+    *p = accumulate ? *p + v : v;
+  }
+};
+
+// s_waitcnt vmcnt(n), the other counters left alone (gfx9 encoding of the immediate)
+template <int N>
+__device__ __forceinline__ void wait_for_loads_but() {
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+__host__ __device__ inline int k_steps_b16(int K) { return (K + TileB16::BK - 1) / TileB16::BK; }
+
+// LDS of one workgroup of igemm_tile_b16<Ops, ROWS>
+template <int ROWS>
+struct StageB16 {
+  static constexpr int HALVES = (ROWS + TileB16::BN) * TileB16::BK;
+  static constexpr int BYTES = TileB16::STAGES * HALVES * 2;
+};
+
+// C[M, Ncols] = A[M, K] x B[K, Ncols], one ROWS x 256 tile (ROWS = 256: wavefronts 2 x 2 of
+// 128 x 128; ROWS = 128: wavefronts 1 x 4 of 128 x 64) over the K steps s_begin .. s_end - 1
+// (s_begin < s_end).  piece == nullptr: results go through ops.store; otherwise into the dense
+// ROWS x 256 piece.
+template <typename Ops, int ROWS>
+__device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, int s_begin, int s_end,
+                                               float* __restrict__ piece) {
+  using T = TileB16;
+  constexpr int NJ = ROWS == 256 ? 4 : 2;        // column fragments of a wavefront
+  constexpr int A_LOADS = ROWS / 64, B_LOADS = T::BN / 64, LOADS = A_LOADS + B_LOADS;
+  constexpr int STAGE = StageB16<ROWS>::HALVES;
+  __shared__ __attribute__((aligned(1024))) unsigned short lds[T::STAGES * STAGE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = ROWS == 256 ? (wave >> 1) * 128 : 0, wn = ROWS == 256 ? (wave & 1) * 128 : wave * 64;
+
+  // ---- loading: an instruction moves 16 rows x 64 bytes into LDS, lane l to byte 16 * l of them;
+  // the lane's chunk of its row is the one that belongs in that slot
+  const int l_row = lane >> 2, l_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+  const __amdgpu_buffer_rsrc_t a_buf = ops.a_buffer(), b_buf = ops.b_buffer(n0);
+  const int a_off = ops.a_offset(m0 + 16 * A_LOADS * wave + l_row) + l_chunk * 16;
+  typename Ops::BCtx bctx[B_LOADS];
+#pragma unroll
+  for (int k = 0; k < B_LOADS; ++k) bctx[k] = ops.b_ctx(n0 + 16 * (B_LOADS * wave + k) + l_row, n0);
+
+  // Requests for the next K step (one step after the other): request(k) is load k of the LOADS a
+  // wavefront contributes, step_requested() closes the step.  Past the last step the loads are
+  // aimed beyond the buffers and bring zeros into a stage nobody reads: the loop body stays free
+  // of branches and every step leaves the same number of loads in flight.
+  StepCursor cur = ops.cursor(s_begin);
+  int s_issue = s_begin, stage_issue = 0;
+  auto request = [&](int k) {
+    unsigned short* const base = lds + stage_issue * STAGE;
+    const int dead = s_issue < s_end ? 0 : kDead;
+    if (k < A_LOADS) {
+      const int a_s = s_issue < s_end ? ops.a_step_offset(s_issue) : 0;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_buf, base + 16 * (A_LOADS * wave + k) * 32, 16, a_off | dead,
+                                               a_s + k * ops.a_offset(16), 0, 0);
+    } else {
+      const int kb = k - A_LOADS;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_buf, base + (ROWS + 16 * (B_LOADS * wave + kb)) * 32, 16,
+                                               ops.b_offset(bctx[kb], ops.step_at(cur), l_chunk) | dead, 0, 0, 0);
+    }
+  };
+  auto step_requested = [&]() {
+    ops.advance(cur);
+    ++s_issue;
+    stage_issue = stage_issue + 1 == T::STAGES ? 0 : stage_issue + 1;
+  };
+
+  float16v acc[4][NJ];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  // ---- reading: fragment = rows base + col, K chunk 2 * kc + half (8 halves of a row) ----
+  const int half = lane >> 5, col = lane & 31, sw = (col >> 2) & 3;
+  int rd_a[2], rd_b[2];   // in halves
+#pragma unroll
+  for (int kc = 0; kc < 2; ++kc) {
+    const int slot = (2 * kc + half) ^ sw;
+    rd_a[kc] = (wm + col) * 32 + slot * 8;
+    rd_b[kc] = (ROWS + wn + col) * 32 + slot * 8;
+  }
+  bf16x8 fa[2][4], fb[2][NJ];
+  // fragment reads of a chunk in the order the products below first need them: a0 b0 b1 .. a1 a2 a3
+  constexpr int READS = 4 + NJ;
+  auto read_fragment = [&](int stage, int kc, int k) {
+    const unsigned short* const base = lds + stage * STAGE;
+    if (k == 0 || k > NJ) {
+      const int i = k == 0 ? 0 : k - NJ;
+      fa[kc][i] = *reinterpret_cast<const bf16x8*>(base + rd_a[kc] + i * 32 * 32);
+    } else {
+      fb[kc][k - 1] = *reinterpret_cast<const bf16x8*>(base + rd_b[kc] + (k - 1) * 32 * 32);
+    }
+  };
+  auto multiply = [&](int kc, int k) {   // product k of the 4 * NJ of a chunk
+    const int i = k / NJ, j = k % NJ;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kc][i], fb[kc][j], acc[i][j], 0, 0, 0);
+  };
+
+  // One K step: each of its 8 * NJ matrix instructions occupies the matrix pipeline for 32
+  // cycles, and whatever else the step needs is issued in their shadow, spread evenly over them
+  // (the scheduling barriers pin that order):
+  //   first half:  products of chunk 0 of stage s | fragment reads of chunk 1
+  //   wait for stage s + 1 (all loads but those of later stages), barrier
+  //   second half: products of chunk 1 | requests for stage s + STAGES - 1 (its LDS was stage
+  //                s - 1, read by everyone before the barrier) | fragment reads of chunk 0 of
+  //                stage s + 1
+  constexpr int SLOTS = 4 * NJ, ITEMS = LOADS + READS;   // products of a half step; what the second half issues besides
+#pragma unroll
+  for (int k = 0; k < T::STAGES - 1; ++k) {
+#pragma unroll
+    for (int q = 0; q < LOADS; ++q) request(q);
+    step_requested();
+  }
+  wait_for_loads_but<(T::STAGES - 2) * LOADS>();
+  __syncthreads();
+  int stage = 0;
+#pragma unroll
+  for (int k = 0; k < READS; ++k) read_fragment(0, 0, k);
+  for (int s = s_begin; s < s_end; ++s) {
+    const int next = stage + 1 == T::STAGES ? 0 : stage + 1;
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+      multiply(0, k);
+#pragma unroll
+      for (int q = k * READS / SLOTS; q < (k + 1) * READS / SLOTS; ++q) read_fragment(stage, 1, q);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    wait_for_loads_but<(T::STAGES - 3) * LOADS>();
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+      multiply(1, k);
+#pragma unroll
+      for (int q = k * ITEMS / SLOTS; q < (k + 1) * ITEMS / SLOTS; ++q) {
+        if (q < LOADS) request(q);
+        else read_fragment(next, 0, q - LOADS);
+        if (q == LOADS - 1) step_requested();
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    stage = next;
+  }
+  wait_for_loads_but<0>();   // (the requests past the last step)
+
+  // accumulator register v of a lane: row 8 * (v / 4) + 4 * (lane / 32) + v % 4, column lane % 32
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const int column = wn + j * 32 + col;
+    if (piece != nullptr) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          piece[(wm + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3)) * T::BN + column] = acc[i][j][v];
+    } else {
+      const typename Ops::Column out = ops.column(n0 + column);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          ops.store(out, m0 + wm + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3), acc[i][j][v]);
+    }
+  }
+}
+
+// Tiles in column-major order, whole tiles first, then the tiles cut along K (see igemm_kernel).
+template <typename Ops, int ROWS>
+__global__ void __launch_bounds__(TileB16::NT, ROWS == 256 ? 1 : 2)
+igemm_b16_kernel(Ops ops, int row_tiles, TileSplit split, float* __restrict__ piece_buffer) {
+  const int whole_blocks = tile_blocks(split.whole);
+  int t, s_begin = 0, s_end = k_steps_b16(ops.K);
+  float* piece = nullptr;
+  if (static_cast<int>(blockIdx.x) < whole_blocks) {
+    t = tile_of_block(split.whole);
+    if (t < 0) return;
+  } else {
+    const int q = blockIdx.x - whole_blocks;
+    t = split.whole + q / split.pieces;
+    s_begin = (q % split.pieces) * split.steps_per_piece;
+    s_end = min(s_end, s_begin + split.steps_per_piece);
+    piece = piece_buffer + static_cast<size_t>(q) * ROWS * TileB16::BN;
+  }
+  igemm_tile_b16<Ops, ROWS>(ops, (t % row_tiles) * ROWS, (t / row_tiles) * TileB16::BN, s_begin, s_end, piece);
+}
+
+// Results of the split tiles: sum of their pieces, in piece order.
+template <typename Ops, int ROWS>
+__global__ void __launch_bounds__(256)
+reduce_pieces_b16_kernel(Ops ops, int row_tiles, TileSplit split, const float* __restrict__ piece_buffer) {
+  constexpr int TILE = ROWS * TileB16::BN;
+  const int local = blockIdx.x / (TILE / 256), e = (blockIdx.x % (TILE / 256)) * 256 + threadIdx.x;
+  const int t = split.whole + local;
+  const float* p = piece_buffer + static_cast<size_t>(local) * split.pieces * TILE + e;
+  float sum = 0.0f;
+  for (int i = 0; i < split.pieces; ++i) sum += p[static_cast<size_t>(i) * TILE];
+  ops.store(ops.column((t / row_tiles) * TileB16::BN + e % TileB16::BN), (t % row_tiles) * ROWS + e / TileB16::BN, sum);
+}
+
+}  // namespace conv

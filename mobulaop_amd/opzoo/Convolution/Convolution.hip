@@ -11,6 +11,7 @@
 
 #include "runtime.h"
 #include "conv_igemm.hip.h"
+#include "conv_igemm_bf16.hip.h"
 
 namespace {
 
@@ -87,10 +88,56 @@ void launch_igemm(const Ops& ops, float* piece_buffer, hipStream_t stream) {
   }
 }
 
+// Workgroups of igemm_b16_kernel<Ops, ROWS> the device holds at a time.
+template <typename Ops, int ROWS>
+int resident_workgroups_b16() {
+  static thread_local int cached_device = -1, cached = 0;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return 0;
+  if (device != cached_device) {
+    int per_cu = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, conv::igemm_b16_kernel<Ops, ROWS>,
+                                                     conv::TileB16::NT, 0) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) {
+      (void)hipGetLastError();
+      return 0;
+    }
+    cached = per_cu * cus;
+    cached_device = device;
+  }
+  return cached;
+}
+
+// Pieces of the bf16 products are ROWS x 256 floats; the piece buffer holds kMaxPieceBlocks
+// pieces of 128 x 128.
+template <typename Ops, int ROWS>
+void launch_igemm_b16_rows(const Ops& ops, float* piece_buffer, hipStream_t stream) {
+  const int row_tiles = (ops.M + ROWS - 1) / ROWS;
+  const int count = row_tiles * ((ops.Ncols + conv::TileB16::BN - 1) / conv::TileB16::BN);
+  const int room = kMaxPieceBlocks * conv::Tile::BM * conv::Tile::BN / (ROWS * conv::TileB16::BN);
+  const int resident = std::min(resident_workgroups_b16<Ops, ROWS>(), room);
+  const conv::TileSplit split = split_tiles(count, conv::k_steps_b16(ops.K), resident);
+  const int rest = count - split.whole;
+  const dim3 grid(conv::tile_blocks(split.whole) + rest * split.pieces);
+  conv::igemm_b16_kernel<Ops, ROWS><<<grid, conv::TileB16::NT, 0, stream>>>(ops, row_tiles, split, piece_buffer);
+  if (rest > 0)
+    conv::reduce_pieces_b16_kernel<Ops, ROWS><<<rest * (ROWS * conv::TileB16::BN / 256), 256, 0, stream>>>(
+        ops, row_tiles, split, piece_buffer);
+}
+
+// Row tiles of 256, or of 128 when the product has at most 128 rows.
+template <typename Ops>
+void launch_igemm_b16(const Ops& ops, float* piece_buffer, hipStream_t stream) {
+  if (ops.M > 128) launch_igemm_b16_rows<Ops, 256>(ops, piece_buffer, stream);
+  else launch_igemm_b16_rows<Ops, 128>(ops, piece_buffer, stream);
+}
+
 // workgroups the weight gradient aims at: four per CU of a 256-CU device
 constexpr long long kWeightSlots = 1024;
 
 int blocks_for(long long n) { return static_cast<int>(std::min<long long>((n + 255) / 256, 256ll * 32)); }
+// (for kernels that take one element per thread and do not stride)
+int blocks_for_all(long long n) { return static_cast<int>((n + 255) / 256); }
 
 bool fits(const char* what, int arg, long long need) {
   const long long have = arg_extent(arg);
@@ -177,6 +224,41 @@ bool plan_gather(GatherPlan* plan, const char* what, const conv::Geometry& g, co
   return true;
 }
 
+// Workspace of a gathered product with bf16 operands in memory (conv_igemm_bf16.hip.h): the
+// weights as [K step][Mpad][32] bf16, the gathered tensor `src` ([images][channels][src_pixels]
+// fp32) as [images][channel block][src_pixels][32] bf16, the piece buffer.  Fills in the
+// fields of `ops` that describe them.
+bool plan_gather_b16(conv::GatheredB16* ops, float** pieces, const char* what, const conv::Geometry& g,
+                     const float* w, int M, int channels, const float* src, int images, int src_pixels,
+                     int columns_per_image, long long stride_m, long long stride_c, hipStream_t stream) {
+  const int taps = g.KH * g.KW, cpad = (channels + 31) / 32 * 32;
+  const long long image_bytes = static_cast<long long>(src_pixels) * cpad * 2;
+  // a tile's columns span this many images at most; their byte offsets must stay below 2^31
+  const long long span = (conv::TileB16::BN - 1) / std::max(columns_per_image, 1) + 2;
+  if (span * image_bytes >= (1ll << 31)) {
+    set_error("%s: images of %lld bytes are too large for the 32-bit offsets of the gather", what, image_bytes);
+    return false;
+  }
+  const int mpad = (M + 255) / 256 * 256;   // (covers row tiles of 128 and of 256)
+  const long long k = static_cast<long long>(taps) * cpad, wcount = k * mpad;
+  if (k >= (1ll << 31) || 2 * wcount >= (1ll << 31)) { set_error("%s: weights too large", what); return false; }
+  const size_t weight_bytes = (2 * wcount + 255) / 256 * 256;
+  const size_t source_bytes = (static_cast<size_t>(images) * image_bytes + 255) / 256 * 256;
+  const size_t piece_bytes = sizeof(float) * kMaxPieceBlocks * conv::Tile::BM * conv::Tile::BN;
+  char* ws = static_cast<char*>(mobula_hip::workspace(weight_bytes + source_bytes + piece_bytes));
+  if (failed()) return false;
+  unsigned short* const weights = reinterpret_cast<unsigned short*>(ws);
+  unsigned short* const source = reinterpret_cast<unsigned short*>(ws + weight_bytes);
+  *pieces = reinterpret_cast<float*>(ws + weight_bytes + source_bytes);
+  ops->wp = weights; ops->src = source; ops->g = g; ops->M = M;
+  ops->K = static_cast<int>(k); ops->cpad = cpad; ops->mpad = mpad;
+  conv::arrange_weights_bf16_kernel<<<blocks_for_all(wcount / 2), 256, 0, stream>>>(
+      w, weights, M, mpad, channels, cpad, taps, stride_m, stride_c);
+  const dim3 tgrid((src_pixels + 63) / 64, (cpad + 63) / 64, images);
+  conv::to_blocked_bf16_kernel<<<tgrid, 256, 0, stream>>>(src, source, channels, cpad, src_pixels);
+  return true;
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -237,6 +319,20 @@ MOBULA_KERNEL conv2d_forward_kernel(const int n, const T* x, const T* weight, co
   conv::ForwardOps ops;
   ops.x = x; ops.bias = has_bias ? bias : nullptr; ops.y = y; ops.g = g;
   ops.M = g.D; ops.Ncols = g.N * g.OH * g.OW;
+  if (compute_mode() == conv::kBf16 && g.N < 65536) {
+    // operands as bf16 in memory: channel-blocked copy of x, weights by K step
+    mobula_hip::KernelTimer timer("conv2d_forward", stream);
+    conv::ForwardOpsB16 ob;
+    ob.bias = ops.bias; ob.y = y; ob.Ncols = ops.Ncols;
+    float* pieces = nullptr;
+    const long long taps = g.KH * g.KW;
+    if (!plan_gather_b16(&ob, &pieces, "conv2d_forward", g, weight, g.D, g.C, x, g.N, g.H * g.W, g.OH * g.OW,
+                         g.C * taps, taps, stream))
+      return;
+    launch_igemm_b16(ob, pieces, stream);
+    MOBULA_HIP_TRY(hipGetLastError());
+    return;
+  }
   {
     mobula_hip::KernelTimer timer("conv2d_forward", stream);
     GatherPlan plan;
@@ -274,6 +370,20 @@ MOBULA_KERNEL conv2d_backward_data_kernel(const int n, const T* dy, const T* wei
   conv::BackwardDataOps ops;
   ops.dy = dy; ops.dx = dx; ops.g = g; ops.accumulate = accumulate;
   ops.M = g.C; ops.Ncols = g.N * g.H * g.W;
+  if (compute_mode() == conv::kBf16 && g.N < 65536) {
+    mobula_hip::KernelTimer timer("conv2d_backward_data", stream);
+    conv::BackwardDataOpsB16 ob;
+    ob.dx = dx; ob.accumulate = accumulate; ob.Ncols = ops.Ncols;
+    float* pieces = nullptr;
+    const long long taps = g.KH * g.KW;
+    // row m of the left operand is input channel m: element [m][tap][d] = weight[d][m][tap]
+    if (!plan_gather_b16(&ob, &pieces, "conv2d_backward_data", g, weight, g.C, g.D, dy, g.N, g.OH * g.OW,
+                         g.H * g.W, taps, g.C * taps, stream))
+      return;
+    launch_igemm_b16(ob, pieces, stream);
+    MOBULA_HIP_TRY(hipGetLastError());
+    return;
+  }
   {
     mobula_hip::KernelTimer timer("conv2d_backward_data", stream);
     GatherPlan plan;
