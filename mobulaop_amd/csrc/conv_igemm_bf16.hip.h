@@ -113,7 +113,7 @@ struct GatheredB16 {
     return buffer_of_bytes(wp, static_cast<unsigned>(mpad) * static_cast<unsigned>(K) * 2u);
   }
   __device__ int a_offset(int m) const { return m * 64; }
-  __device__ int a_step_offset(int s) const { return s * mpad * 64; }
+  typedef StepCursor Cursor;
   __device__ StepCursor cursor(int s) const {
     const int taps = g.KH * g.KW, cb = s / taps, tap = s - cb * taps, kh = tap / g.KW;
     return StepCursor{kh, tap - kh * g.KW, cb};
@@ -130,7 +130,9 @@ struct GatheredB16 {
 };
 
 // Operand functors of igemm_tile_b16:
-//   Step step_at(cursor): what a K step adds to every column's offset (uniform);
+//   Cursor cursor(s) / advance(cursor): the walk over the K steps;
+//   Step step_at(cursor, s): what a K step adds to every row's and column's offset (uniform);
+//   a_buffer() / a_offset(m): the left operand and the byte offset of row m in a K step;
 //   b_buffer(n0): the gathered tensor from the first image of the tile on;
 //   BCtx b_ctx(n, n0): what column n needs throughout;
 //   b_offset(ctx, step, chunk): byte offset of the column's 16-byte chunk in that buffer (kDead: zeros);
@@ -139,13 +141,13 @@ struct GatheredB16 {
 // y[img, d, oh, ow] = bias[d] + sum over (c, kh, kw) of W[d, c, kh, kw] * x[img, c, ih, iw]
 struct ForwardOpsB16 : GatheredB16 {
   const float* __restrict__ bias; float* __restrict__ y;
-  struct Step { int dh, dw, delta; };
+  struct Step { int dh, dw, delta, a_delta; };
   struct BCtx { int anchor, ih0, iw0; };   // (a column past the last: ih0 far outside)
   struct Column { float* p; bool ok; };
   __device__ int plane_bytes() const { return g.H * g.W * 64; }
-  __device__ Step step_at(const StepCursor& c) const {
+  __device__ Step step_at(const StepCursor& c, int s) const {
     const int dh = c.kh * g.dil_h, dw = c.kw * g.dil_w;
-    return Step{dh, dw, c.cb * plane_bytes() + (dh * g.W + dw) * 64};
+    return Step{dh, dw, c.cb * plane_bytes() + (dh * g.W + dw) * 64, s * mpad * 64};
   }
   __device__ __amdgpu_buffer_rsrc_t b_buffer(int n0) const {
     return images_from(__builtin_amdgcn_readfirstlane(n0 / (g.OH * g.OW)), static_cast<size_t>(plane_bytes()) * (cpad / 32));
@@ -178,15 +180,15 @@ struct ForwardOpsB16 : GatheredB16 {
 // with oh * stride = ih + pad - kh * dil (and likewise for columns).
 struct BackwardDataOpsB16 : GatheredB16 {
   float* __restrict__ dx; int accumulate;
-  struct Step { int dh, dw, delta; };
+  struct Step { int dh, dw, delta, a_delta; };
   struct BCtx { int anchor, ihp, iwp; };   // (a column past the last: ihp far outside)
   struct Column { float* p; bool ok; };
   __device__ bool unit_stride() const { return g.stride_h == 1 && g.stride_w == 1; }
   __device__ int plane_bytes() const { return g.OH * g.OW * 64; }
-  __device__ Step step_at(const StepCursor& c) const {
+  __device__ Step step_at(const StepCursor& c, int s) const {
     const int dh = c.kh * g.dil_h, dw = c.kw * g.dil_w;
     // stride 1: the tap's offset from the anchor pixel (ih + pad, iw + pad) of dy
-    return Step{dh, dw, c.cb * plane_bytes() - (unit_stride() ? (dh * g.OW + dw) * 64 : 0)};
+    return Step{dh, dw, c.cb * plane_bytes() - (unit_stride() ? (dh * g.OW + dw) * 64 : 0), s * mpad * 64};
   }
   __device__ __amdgpu_buffer_rsrc_t b_buffer(int n0) const {
     return images_from(__builtin_amdgcn_readfirstlane(n0 / (g.H * g.W)), static_cast<size_t>(plane_bytes()) * (cpad / 32));
@@ -219,6 +221,92 @@ struct BackwardDataOpsB16 : GatheredB16 {
   __device__ void store(const Column& c, int m, float v) const {
     if (m >= M || !c.ok) return;
     float* p = c.p + static_cast<size_t>(m) * (g.H * g.W);
+    *p = accumulate ? *p + v : v;
+  }
+};
+
+// ---- the weight gradient as shifted plain products ---------------------------------------
+//
+// With unit strides, dW[d, c, kh, kw] = sum over images and output pixels of
+// dy[d, oh, ow] * x[c, oh - pad + kh * dil, ow - pad + kw * dil].  On a common grid of
+// Hg x Wg = (H + 2 pad_h) x (W + 2 pad_w) positions per plane -- x placed at (pad_h, pad_w),
+// dy at (0, 0), zeros elsewhere -- this is, for every tap, a plain matrix product over the grid
+// positions g of all images: dW_tap[d, c] = sum_g dyg[d, g] * xg[c, g + kh * dil_h * Wg + kw * dil_w].
+// Where dyg is zero (outside the outputs, and in the tail that pads a plane to a multiple of
+// 32 positions) it does not matter what the shifted read of xg finds, as long as it is finite:
+// the next plane, or zeros beyond the buffer.  The positions are the K of the product, 32 to a
+// step, contiguous in memory for every row (filter d) and column (channel c, tap): the same
+// tile as for the gathered products applies, K cut into pieces that fill the device, the pieces
+// summed in order afterwards.  Loads of four bytes and more need an even position: taps with
+// an odd shift read a second copy of xg that is shifted by one position.
+//
+// Replaces the second im2col + product of opzoo/Convolution/Convolution.py:44-57.
+
+// dst[plane][g] = bf16(src[plane][gh - off_h][gw - off_w]) for g = gh * Wg + gw < Hg * Wg with the
+// source position inside H x W, zero elsewhere (g < Gp); shifted[plane][g] = dst[plane][g + 1]
+// (shifted may be null).  A thread: eight positions.
+__global__ void __launch_bounds__(256)
+to_padded_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst,
+                      unsigned short* __restrict__ shifted, int H, int W, int off_h, int off_w, int Hg, int Wg,
+                      int Gp) {
+  const int plane = blockIdx.x, g0 = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (g0 >= Gp) return;
+  const float* in = src + static_cast<size_t>(plane) * H * W;
+  float v[9];
+#pragma unroll
+  for (int j = 0; j < 9; ++j) {
+    const int g = g0 + j, gh = g / Wg, gw = g - gh * Wg, ih = gh - off_h, iw = gw - off_w;
+    const bool inside = (gh < Hg) & (static_cast<unsigned>(ih) < static_cast<unsigned>(H)) &
+                        (static_cast<unsigned>(iw) < static_cast<unsigned>(W));
+    v[j] = inside ? in[ih * W + iw] : 0.0f;
+  }
+  u32x4 a, b;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) { a[j] = pack_bf16(v[2 * j], v[2 * j + 1]); b[j] = pack_bf16(v[2 * j + 1], v[2 * j + 2]); }
+  const size_t at = static_cast<size_t>(plane) * Gp + g0;
+  *reinterpret_cast<u32x4*>(dst + at) = a;
+  if (shifted != nullptr) *reinterpret_cast<u32x4*>(shifted + at) = b;
+}
+
+// Rows: filters d; columns: (tap, channel), tap-major; K: (image, grid position).
+struct WeightGradOpsB16 {
+  const unsigned short* __restrict__ dyg;   // [N][D][Gp]
+  const unsigned short* __restrict__ xg;    // [2][N][C][Gp], the second copy shifted by one position
+  float* __restrict__ dw;
+  Geometry g; int M, Ncols, K, Gp, Wg, accumulate; unsigned copy_bytes;
+  struct Cursor { int n, j; };   // image, K step within the image
+  struct Step { int delta, a_delta; };
+  struct BCtx { int anchor; };   // (kDead for a column past the last)
+  struct Column { float* p; bool ok; };
+  __device__ __amdgpu_buffer_rsrc_t a_buffer() const {
+    return buffer_of_bytes(dyg, static_cast<unsigned>(g.N) * g.D * Gp * 2u);
+  }
+  __device__ int a_offset(int m) const { return m * Gp * 2; }
+  __device__ Cursor cursor(int s) const {
+    const int per_image = Gp / TileB16::BK, n = s / per_image;
+    return Cursor{n, s - n * per_image};
+  }
+  __device__ void advance(Cursor& c) const {
+    if (++c.j == Gp / TileB16::BK) { c.j = 0; ++c.n; }
+  }
+  __device__ Step step_at(const Cursor& c, int) const {
+    return Step{(c.n * g.C * Gp + c.j * TileB16::BK) * 2, (c.n * g.D * Gp + c.j * TileB16::BK) * 2};
+  }
+  __device__ __amdgpu_buffer_rsrc_t b_buffer(int) const { return buffer_of_bytes(xg, 2u * copy_bytes); }
+  __device__ BCtx b_ctx(int n, int) const {
+    const int tap = n / g.C, c = n - tap * g.C, kh = tap / g.KW, kw = tap - kh * g.KW;
+    const int shift = kh * g.dil_h * Wg + kw * g.dil_w, odd = shift & 1;
+    return BCtx{n < Ncols ? static_cast<int>(odd * copy_bytes) + (c * Gp + shift - odd) * 2 : kDead};
+  }
+  // (kDead plus the offsets of a step stays beyond every buffer)
+  __device__ int b_offset(const BCtx& c, const Step& e, int chunk) const { return c.anchor + e.delta + chunk * 16; }
+  __device__ Column column(int n) const {
+    const int tap = n / g.C, c = n - tap * g.C;
+    return Column{dw + static_cast<size_t>(c) * (g.KH * g.KW) + tap, n < Ncols};
+  }
+  __device__ void store(const Column& c, int m, float v) const {
+    if (m >= M || !c.ok) return;
+    float* p = c.p + static_cast<size_t>(m) * g.C * (g.KH * g.KW);
     *p = accumulate ? *p + v : v;
   }
 };
@@ -266,19 +354,19 @@ __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, i
   // wavefront contributes, step_requested() closes the step.  Past the last step the loads are
   // aimed beyond the buffers and bring zeros into a stage nobody reads: the loop body stays free
   // of branches and every step leaves the same number of loads in flight.
-  StepCursor cur = ops.cursor(s_begin);
+  typename Ops::Cursor cur = ops.cursor(s_begin);
   int s_issue = s_begin, stage_issue = 0;
   auto request = [&](int k) {
     unsigned short* const base = lds + stage_issue * STAGE;
     const int dead = s_issue < s_end ? 0 : kDead;
+    const typename Ops::Step e = ops.step_at(cur, s_issue);
     if (k < A_LOADS) {
-      const int a_s = s_issue < s_end ? ops.a_step_offset(s_issue) : 0;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_buf, base + 16 * (A_LOADS * wave + k) * 32, 16, a_off | dead,
-                                               a_s + k * ops.a_offset(16), 0, 0);
+                                               (s_issue < s_end ? e.a_delta : 0) + k * ops.a_offset(16), 0, 0);
     } else {
       const int kb = k - A_LOADS;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_buf, base + (ROWS + 16 * (B_LOADS * wave + kb)) * 32, 16,
-                                               ops.b_offset(bctx[kb], ops.step_at(cur), l_chunk) | dead, 0, 0, 0);
+                                               ops.b_offset(bctx[kb], e, l_chunk) | dead, 0, 0, 0);
     }
   };
   auto step_requested = [&]() {

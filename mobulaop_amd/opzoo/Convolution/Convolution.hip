@@ -422,6 +422,35 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
     return;
   }
   hipStream_t stream = call_state().stream;
+  if (compute_mode() == conv::kBf16 && g.stride_h == 1 && g.stride_w == 1 && wt > 0 && g.N > 0) {
+    // bf16 operands in memory on a common padded grid, one plain product per tap
+    const int Hg = g.H + 2 * g.pad_h, Wg = g.W + 2 * g.pad_w;
+    const long long G = static_cast<long long>(Hg) * Wg, Gp = (G + 31) / 32 * 32;
+    const long long dy_bytes = 2ll * g.N * g.D * Gp, x_bytes = 2ll * g.N * g.C * Gp;
+    if (dy_bytes < (1ll << 31) && 2 * x_bytes < (1ll << 31) && g.OH <= Hg && g.OW <= Wg) {
+      mobula_hip::KernelTimer timer("conv2d_backward_weight", stream);
+      const size_t dy_room = (dy_bytes + 255) / 256 * 256, x_room = (x_bytes + 255) / 256 * 256;
+      const size_t piece_bytes = sizeof(float) * kMaxPieceBlocks * conv::Tile::BM * conv::Tile::BN;
+      char* ws = static_cast<char*>(mobula_hip::workspace(dy_room + 2 * x_room + piece_bytes));
+      if (failed()) return;
+      conv::WeightGradOpsB16 ob;
+      unsigned short* const dyg = reinterpret_cast<unsigned short*>(ws);
+      unsigned short* const xg = reinterpret_cast<unsigned short*>(ws + dy_room);
+      ob.dyg = dyg; ob.xg = xg; ob.dw = dw; ob.g = g; ob.M = g.D; ob.Ncols = g.C * g.KH * g.KW;
+      ob.K = static_cast<int>(g.N * Gp); ob.Gp = static_cast<int>(Gp); ob.Wg = Wg; ob.accumulate = accumulate;
+      ob.copy_bytes = static_cast<unsigned>(x_room);
+      const dim3 pgrid_dy(g.N * g.D, static_cast<unsigned>((Gp / 8 + 255) / 256));
+      conv::to_padded_bf16_kernel<<<pgrid_dy, 256, 0, stream>>>(dy, dyg, nullptr, g.OH, g.OW, 0, 0, Hg, Wg,
+                                                              static_cast<int>(Gp));
+      const dim3 pgrid_x(g.N * g.C, static_cast<unsigned>((Gp / 8 + 255) / 256));
+      conv::to_padded_bf16_kernel<<<pgrid_x, 256, 0, stream>>>(
+          x, xg, reinterpret_cast<unsigned short*>(ws + dy_room + x_room), g.H, g.W, g.pad_h, g.pad_w, Hg, Wg,
+          static_cast<int>(Gp));
+      launch_igemm_b16(ob, reinterpret_cast<float*>(ws + dy_room + 2 * x_room), stream);
+      MOBULA_HIP_TRY(hipGetLastError());
+      return;
+    }
+  }
   conv::BackwardWeightOps ops;
   ops.dy = dy; ops.x = x; ops.g = g;
   ops.M = g.D; ops.Ncols = g.C * g.KH * g.KW; ops.K = 0; ops.k_begin = 0;
