@@ -186,10 +186,11 @@ def test_resnet_block_shape_properties(compute):
     assert abs(lhs - float((w.double() * dw.double()).sum())) <= bound
 
 
-@pytest.mark.parametrize('mode', ['fp32', 'bf16x3'])
+@pytest.mark.parametrize('mode', ['fp32', 'bf16x3', 'bf16'])
 def test_full_cfg5_against_torch(mode):
     # BASELINE configuration 5 at its full size: N=32, 256 -> 256 channels, 56 x 56, 3 x 3,
     # stride 1, pad 1; y, dx and dw against torch's conv2d and its autograd on the CPU, 1e-3
+    # (1e-2 with operands rounded to bf16)
     N, C, H, W, D = 32, 256, 56, 56, 256
     g = torch.Generator().manual_seed(1005)
     xh = torch.randn(N, C, H, W, generator=g)
@@ -206,37 +207,46 @@ def test_full_cfg5_against_torch(mode):
         y = torch.empty(N, D, H, W, device='cuda')
         _call('conv2d_forward_c6a7aa85', ctypes.c_int(y.numel()), _ptr(x), _ptr(w), _ptr(w), ctypes.c_int(0), *geo,
               _ptr(y))
-        _close(y, yr, 'cfg5 y ' + mode)
+        _close(y, yr, 'cfg5 y ' + mode, MODES[mode][1])
         dx = torch.empty_like(x)
         _call('conv2d_backward_data_ecf81c91', ctypes.c_int(dx.numel()), _ptr(dy), _ptr(w), ctypes.c_int(0), *geo,
               _ptr(dx))
-        _close(dx, xr.grad, 'cfg5 dx ' + mode)
+        _close(dx, xr.grad, 'cfg5 dx ' + mode, MODES[mode][1])
         dw = torch.empty_like(w)
         _call('conv2d_backward_weight_ecf81c91', ctypes.c_int(dw.numel()), _ptr(dy), _ptr(x), ctypes.c_int(0),
               *geo, _ptr(dw))
-        _close(dw, wr.grad, 'cfg5 dw ' + mode)
+        _close(dw, wr.grad, 'cfg5 dw ' + mode, MODES[mode][1])
     finally:
         native.set_option('conv_compute', 0)
 
 
-def test_bf16_mode_is_exact_on_bf16_valued_operands():
+@pytest.mark.parametrize('case', [
+    # N, C, H, W, D, kernel, pad, stride, dilation
+    (3, 64, 20, 20, 96, (3, 3), (1, 1), (1, 1), (1, 1)),      # 128-row tiles
+    (2, 70, 23, 17, 200, (3, 3), (1, 1), (1, 1), (1, 1)),     # 256-row tiles, channels not a multiple of 32
+    (2, 40, 19, 21, 130, (5, 3), (2, 0), (1, 1), (1, 2)),     # dilation, uneven padding
+    (2, 33, 30, 26, 300, (3, 3), (1, 1), (2, 2), (1, 1)),     # strides: two row tiles, gathered weight gradient
+    (9, 256, 28, 28, 256, (3, 3), (1, 1), (1, 1), (1, 1)),    # several images to a tile, K cut into pieces
+    (1, 16, 60, 60, 16, (1, 1), (0, 0), (1, 1), (1, 1)),      # one tap
+])
+def test_bf16_mode_is_exact_on_bf16_valued_operands(case):
     # Mode 1 rounds both operands of every product to bf16 and accumulates in fp32: against
     # the same products of the rounded operands in fp32 only the order of the sums differs,
     # well inside the 1e-3 bound (the 1e-2 of the other tests is the rounding of the inputs)
-    N, C, H, W, D = 3, 64, 20, 20, 96
+    N, C, H, W, D, k, pad, stride, dil = case
     g = torch.Generator().manual_seed(61)
     x = torch.randn(N, C, H, W, generator=g)
-    w = torch.randn(D, C, 3, 3, generator=g) * 0.1
-    dy = torch.randn(N, D, H, W, generator=g)
+    w = torch.randn(D, C, *k, generator=g) * 0.1
     rnd = lambda t: t.bfloat16().float()
     xr, wr = rnd(x).requires_grad_(True), rnd(w).requires_grad_(True)
-    F.conv2d(xr, wr, padding=1).backward(rnd(dy))
-    y_ref = F.conv2d(rnd(x), rnd(w), padding=1)
+    yr = F.conv2d(xr, wr, padding=pad, stride=stride, dilation=dil)
+    dy = torch.randn(yr.shape, generator=g)
+    yr.backward(rnd(dy))
     native.set_option('conv_compute', 1)
     try:
         xd, wd, dyd = x.cuda(), w.cuda(), dy.cuda()
-        geo = _ci(N, C, H, W, D, 3, 3, 1, 1, 1, 1, 1, 1)
-        y = torch.empty(N, D, H, W, device='cuda')
+        geo = _ci(N, C, H, W, D, k[0], k[1], pad[0], pad[1], stride[0], stride[1], dil[0], dil[1])
+        y = torch.empty(yr.shape, device='cuda')
         _call('conv2d_forward_c6a7aa85', ctypes.c_int(y.numel()), _ptr(xd), _ptr(wd), _ptr(wd), ctypes.c_int(0),
               *geo, _ptr(y))
         dx = torch.empty_like(xd)
@@ -245,11 +255,20 @@ def test_bf16_mode_is_exact_on_bf16_valued_operands():
         dw = torch.empty_like(wd)
         _call('conv2d_backward_weight_ecf81c91', ctypes.c_int(dw.numel()), _ptr(dyd), _ptr(xd), ctypes.c_int(0),
               *geo, _ptr(dw))
+        # accumulate: twice the gradient on top of what is there
+        dw2 = dw.clone()
+        _call('conv2d_backward_weight_ecf81c91', ctypes.c_int(dw.numel()), _ptr(dyd), _ptr(xd), ctypes.c_int(1),
+              *geo, _ptr(dw2))
+        dx2 = dx.clone()
+        _call('conv2d_backward_data_ecf81c91', ctypes.c_int(dx.numel()), _ptr(dyd), _ptr(wd), ctypes.c_int(1),
+              *geo, _ptr(dx2))
     finally:
         native.set_option('conv_compute', 0)
-    _close(y, y_ref, 'y', 1e-4)
+    _close(y, yr.detach(), 'y', 1e-4)
     _close(dx, xr.grad, 'dx', 1e-4)
     _close(dw, wr.grad, 'dw', 1e-4)
+    _close(dw2, 2 * wr.grad, 'dw accumulated', 1e-4)
+    _close(dx2, 2 * xr.grad, 'dx accumulated', 1e-4)
 
 
 def test_errors_surface_as_exceptions():
