@@ -43,19 +43,33 @@ namespace conv {
 
 struct TileB16 {
   static constexpr int BN = 256, BK = 32, STAGES = 3;
-  static constexpr int NT = 256;
 };
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 // dst[n][c / 32][p][c % 32] = bf16(src[n][c][p]) for c < C, zero for C <= c < Cpad.  One
-// workgroup: 64 pixels x 64 channels (two channel blocks) through LDS.
+// workgroup: 64 pixels x 64 channels (two channel blocks) through LDS.  VEC: P is a multiple
+// of four and src 16-byte aligned, a lane reads four pixels at a time.  The source is read
+// once: its loads leave the caches to the copy that is about to be read.
+template <bool VEC>
 __global__ void __launch_bounds__(256)
 to_blocked_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst, int C, int Cpad, int P) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
   __shared__ float tile[64][65];
   const int n = blockIdx.z, c0 = blockIdx.y * 64, p0 = blockIdx.x * 64;
   const float* in = src + static_cast<size_t>(n) * C * P;
-  {
+  if (VEC) {
+    const int q = threadIdx.x & 15, r = threadIdx.x >> 4;   // 16 quads of pixels, 16 channels per pass
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int c = c0 + r + 16 * k, p = p0 + 4 * q;
+      f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (c < C && p < P)
+        v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(in + static_cast<size_t>(c) * P + p));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) tile[r + 16 * k][4 * q + i] = v[i];
+    }
+  } else {
     const int px = threadIdx.x & 63, cr = threadIdx.x >> 6;
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
@@ -243,29 +257,44 @@ struct BackwardDataOpsB16 : GatheredB16 {
 // Replaces the second im2col + product of opzoo/Convolution/Convolution.py:44-57.
 
 // dst[plane][g] = bf16(src[plane][gh - off_h][gw - off_w]) for g = gh * Wg + gw < Hg * Wg with the
-// source position inside H x W, zero elsewhere (g < Gp); shifted[plane][g] = dst[plane][g + 1]
-// (shifted may be null).  A thread: eight positions.
+// source position inside H x W, zero elsewhere (g < Gp, a multiple of 8); shifted[plane][g] =
+// dst[plane][g + 1] (shifted may be null).  A workgroup: 2048 positions of a plane; neighbouring
+// lanes read neighbouring positions, the bf16 values go through LDS and leave 16 bytes per lane.
 __global__ void __launch_bounds__(256)
 to_padded_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst,
                       unsigned short* __restrict__ shifted, int H, int W, int off_h, int off_w, int Hg, int Wg,
                       int Gp) {
-  const int plane = blockIdx.x, g0 = (blockIdx.y * 256 + threadIdx.x) * 8;
-  if (g0 >= Gp) return;
+  __shared__ __attribute__((aligned(16))) unsigned short vals[2048 + 8];
+  const int plane = blockIdx.x, base = blockIdx.y * 2048;
   const float* in = src + static_cast<size_t>(plane) * H * W;
-  float v[9];
-#pragma unroll
-  for (int j = 0; j < 9; ++j) {
-    const int g = g0 + j, gh = g / Wg, gw = g - gh * Wg, ih = gh - off_h, iw = gw - off_w;
+  auto value_at = [&](int gh, int gw) {
+    const int ih = gh - off_h, iw = gw - off_w;
     const bool inside = (gh < Hg) & (static_cast<unsigned>(ih) < static_cast<unsigned>(H)) &
                         (static_cast<unsigned>(iw) < static_cast<unsigned>(W));
-    v[j] = inside ? in[ih * W + iw] : 0.0f;
-  }
-  u32x4 a, b;
+    return static_cast<unsigned short>(pack_bf16(inside ? in[inside ? ih * W + iw : 0] : 0.0f, 0.0f));
+  };
+  const int step_h = 256 / Wg, step_w = 256 - step_h * Wg;   // 256 positions further on
+  int g = base + threadIdx.x, gh = g / Wg, gw = g - gh * Wg;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) { a[j] = pack_bf16(v[2 * j], v[2 * j + 1]); b[j] = pack_bf16(v[2 * j + 1], v[2 * j + 2]); }
+  for (int j = 0; j < 8; ++j) {
+    vals[threadIdx.x + 256 * j] = value_at(gh, gw);
+    gh += step_h; gw += step_w;
+    if (gw >= Wg) { gw -= Wg; ++gh; }
+  }
+  if (threadIdx.x == 0) vals[2048] = value_at(gh, gw);   // (position base + 2048: for the shifted copy)
+  __syncthreads();
+  const int g0 = base + 8 * threadIdx.x;
+  if (g0 >= Gp) return;
+  const u32x4 a = *reinterpret_cast<const u32x4*>(vals + 8 * threadIdx.x);
   const size_t at = static_cast<size_t>(plane) * Gp + g0;
   *reinterpret_cast<u32x4*>(dst + at) = a;
-  if (shifted != nullptr) *reinterpret_cast<u32x4*>(shifted + at) = b;
+  if (shifted != nullptr) {
+    const unsigned next = vals[8 * threadIdx.x + 8];
+    u32x4 b;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b[j] = (a[j] >> 16) | ((j < 3 ? a[j + 1] : next) << 16);
+    *reinterpret_cast<u32x4*>(shifted + at) = b;
+  }
 }
 
 // Rows: filters d; columns: (tap, channel), tap-major; K: (image, grid position).
@@ -330,16 +359,18 @@ struct StageB16 {
 // 128 x 128; ROWS = 128: wavefronts 1 x 4 of 128 x 64) over the K steps s_begin .. s_end - 1
 // (s_begin < s_end).  piece == nullptr: results go through ops.store; otherwise into the dense
 // ROWS x 256 piece.
-template <typename Ops, int ROWS>
+template <typename Ops, int ROWS, int WAVES>
 __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, int s_begin, int s_end,
                                                float* __restrict__ piece) {
   using T = TileB16;
-  constexpr int NJ = ROWS == 256 ? 4 : 2;        // column fragments of a wavefront
-  constexpr int A_LOADS = ROWS / 64, B_LOADS = T::BN / 64, LOADS = A_LOADS + B_LOADS;
+  constexpr int NI = WAVES == 16 ? 2 : 4;                  // row fragments of a wavefront
+  constexpr int WM = ROWS / (32 * NI), WN = WAVES / WM;   // wavefronts down and across the tile
+  constexpr int NJ = T::BN / WN / 32;                      // column fragments of a wavefront
+  constexpr int A_LOADS = ROWS / 16 / WAVES, B_LOADS = T::BN / 16 / WAVES, LOADS = A_LOADS + B_LOADS;
   constexpr int STAGE = StageB16<ROWS>::HALVES;
   __shared__ __attribute__((aligned(1024))) unsigned short lds[T::STAGES * STAGE];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = ROWS == 256 ? (wave >> 1) * 128 : 0, wn = ROWS == 256 ? (wave & 1) * 128 : wave * 64;
+  const int wm = (wave / WN) * (32 * NI), wn = (wave % WN) * (32 * NJ);
 
   // ---- loading: an instruction moves 16 rows x 64 bytes into LDS, lane l to byte 16 * l of them;
   // the lane's chunk of its row is the one that belongs in that slot
@@ -375,9 +406,9 @@ __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, i
     stage_issue = stage_issue + 1 == T::STAGES ? 0 : stage_issue + 1;
   };
 
-  float16v acc[4][NJ];
+  float16v acc[NI][NJ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
 #pragma unroll
@@ -392,9 +423,9 @@ __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, i
     rd_a[kc] = (wm + col) * 32 + slot * 8;
     rd_b[kc] = (ROWS + wn + col) * 32 + slot * 8;
   }
-  bf16x8 fa[2][4], fb[2][NJ];
-  // fragment reads of a chunk in the order the products below first need them: a0 b0 b1 .. a1 a2 a3
-  constexpr int READS = 4 + NJ;
+  bf16x8 fa[2][NI], fb[2][NJ];
+  // fragment reads of a chunk in the order the products below first need them: a0 b0 b1 .. a1 a2 ..
+  constexpr int READS = NI + NJ;
   auto read_fragment = [&](int stage, int kc, int k) {
     const unsigned short* const base = lds + stage * STAGE;
     if (k == 0 || k > NJ) {
@@ -417,7 +448,7 @@ __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, i
   //   second half: products of chunk 1 | requests for stage s + STAGES - 1 (its LDS was stage
   //                s - 1, read by everyone before the barrier) | fragment reads of chunk 0 of
   //                stage s + 1
-  constexpr int SLOTS = 4 * NJ, ITEMS = LOADS + READS;   // products of a half step; what the second half issues besides
+  constexpr int SLOTS = NI * NJ, ITEMS = LOADS + READS;   // products of a half step; what the second half issues besides
 #pragma unroll
   for (int k = 0; k < T::STAGES - 1; ++k) {
 #pragma unroll
@@ -461,14 +492,14 @@ __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, i
     const int column = wn + j * 32 + col;
     if (piece != nullptr) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v)
           piece[(wm + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3)) * T::BN + column] = acc[i][j][v];
     } else {
       const typename Ops::Column out = ops.column(n0 + column);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v)
           ops.store(out, m0 + wm + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3), acc[i][j][v]);
@@ -477,8 +508,8 @@ __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, i
 }
 
 // Tiles in column-major order, whole tiles first, then the tiles cut along K (see igemm_kernel).
-template <typename Ops, int ROWS>
-__global__ void __launch_bounds__(TileB16::NT, ROWS == 256 ? 1 : 2)
+template <typename Ops, int ROWS, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES, ROWS == 256 ? 1 : 2)
 igemm_b16_kernel(Ops ops, int row_tiles, TileSplit split, float* __restrict__ piece_buffer) {
   const int whole_blocks = tile_blocks(split.whole);
   int t, s_begin = 0, s_end = k_steps_b16(ops.K);
@@ -493,7 +524,7 @@ igemm_b16_kernel(Ops ops, int row_tiles, TileSplit split, float* __restrict__ pi
     s_end = min(s_end, s_begin + split.steps_per_piece);
     piece = piece_buffer + static_cast<size_t>(q) * ROWS * TileB16::BN;
   }
-  igemm_tile_b16<Ops, ROWS>(ops, (t % row_tiles) * ROWS, (t / row_tiles) * TileB16::BN, s_begin, s_end, piece);
+  igemm_tile_b16<Ops, ROWS, WAVES>(ops, (t % row_tiles) * ROWS, (t / row_tiles) * TileB16::BN, s_begin, s_end, piece);
 }
 
 // Results of the split tiles: sum of their pieces, in piece order.

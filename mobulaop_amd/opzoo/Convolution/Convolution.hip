@@ -88,6 +88,10 @@ void launch_igemm(const Ops& ops, float* piece_buffer, hipStream_t stream) {
   }
 }
 
+// Wavefronts of a workgroup of the bf16 products: eight for 256-row tiles (two to a SIMD: one
+// issues matrix instructions while the other waits), four for 128-row tiles.
+constexpr int waves_b16(int rows) { return rows == 256 ? 8 : 4; }
+
 // Workgroups of igemm_b16_kernel<Ops, ROWS> the device holds at a time.
 template <typename Ops, int ROWS>
 int resident_workgroups_b16() {
@@ -96,8 +100,8 @@ int resident_workgroups_b16() {
   if (hipGetDevice(&device) != hipSuccess) return 0;
   if (device != cached_device) {
     int per_cu = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, conv::igemm_b16_kernel<Ops, ROWS>,
-                                                     conv::TileB16::NT, 0) != hipSuccess ||
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, conv::igemm_b16_kernel<Ops, ROWS, waves_b16(ROWS)>,
+                                                     64 * waves_b16(ROWS), 0) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) {
       (void)hipGetLastError();
       return 0;
@@ -119,7 +123,8 @@ void launch_igemm_b16_rows(const Ops& ops, float* piece_buffer, hipStream_t stre
   const conv::TileSplit split = split_tiles(count, conv::k_steps_b16(ops.K), resident);
   const int rest = count - split.whole;
   const dim3 grid(conv::tile_blocks(split.whole) + rest * split.pieces);
-  conv::igemm_b16_kernel<Ops, ROWS><<<grid, conv::TileB16::NT, 0, stream>>>(ops, row_tiles, split, piece_buffer);
+  conv::igemm_b16_kernel<Ops, ROWS, waves_b16(ROWS)><<<grid, 64 * waves_b16(ROWS), 0, stream>>>(ops, row_tiles, split,
+                                                                                           piece_buffer);
   if (rest > 0)
     conv::reduce_pieces_b16_kernel<Ops, ROWS><<<rest * (ROWS * conv::TileB16::BN / 256), 256, 0, stream>>>(
         ops, row_tiles, split, piece_buffer);
@@ -255,7 +260,10 @@ bool plan_gather_b16(conv::GatheredB16* ops, float** pieces, const char* what, c
   conv::arrange_weights_bf16_kernel<<<blocks_for_all(wcount / 2), 256, 0, stream>>>(
       w, weights, M, mpad, channels, cpad, taps, stride_m, stride_c);
   const dim3 tgrid((src_pixels + 63) / 64, (cpad + 63) / 64, images);
-  conv::to_blocked_bf16_kernel<<<tgrid, 256, 0, stream>>>(src, source, channels, cpad, src_pixels);
+  if (src_pixels % 4 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0)
+    conv::to_blocked_bf16_kernel<true><<<tgrid, 256, 0, stream>>>(src, source, channels, cpad, src_pixels);
+  else
+    conv::to_blocked_bf16_kernel<false><<<tgrid, 256, 0, stream>>>(src, source, channels, cpad, src_pixels);
   return true;
 }
 
@@ -439,10 +447,10 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
       ob.dyg = dyg; ob.xg = xg; ob.dw = dw; ob.g = g; ob.M = g.D; ob.Ncols = g.C * g.KH * g.KW;
       ob.K = static_cast<int>(g.N * Gp); ob.Gp = static_cast<int>(Gp); ob.Wg = Wg; ob.accumulate = accumulate;
       ob.copy_bytes = static_cast<unsigned>(x_room);
-      const dim3 pgrid_dy(g.N * g.D, static_cast<unsigned>((Gp / 8 + 255) / 256));
+      const dim3 pgrid_dy(g.N * g.D, static_cast<unsigned>((Gp + 2047) / 2048));
       conv::to_padded_bf16_kernel<<<pgrid_dy, 256, 0, stream>>>(dy, dyg, nullptr, g.OH, g.OW, 0, 0, Hg, Wg,
                                                               static_cast<int>(Gp));
-      const dim3 pgrid_x(g.N * g.C, static_cast<unsigned>((Gp / 8 + 255) / 256));
+      const dim3 pgrid_x(g.N * g.C, static_cast<unsigned>((Gp + 2047) / 2048));
       conv::to_padded_bf16_kernel<<<pgrid_x, 256, 0, stream>>>(
           x, xg, reinterpret_cast<unsigned short*>(ws + dy_room + x_room), g.H, g.W, g.pad_h, g.pad_w, Hg, Wg,
           static_cast<int>(Gp));
