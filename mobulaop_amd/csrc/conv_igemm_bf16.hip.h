@@ -348,29 +348,32 @@ __device__ __forceinline__ void wait_for_loads_but() {
 
 __host__ __device__ inline int k_steps_b16(int K) { return (K + TileB16::BK - 1) / TileB16::BK; }
 
-// LDS of one workgroup of igemm_tile_b16<Ops, ROWS>
-template <int ROWS>
-struct StageB16 {
-  static constexpr int HALVES = (ROWS + TileB16::BN) * TileB16::BK;
-  static constexpr int BYTES = TileB16::STAGES * HALVES * 2;
+// A tile of ROWS x COLS results and the WAVES wavefronts that share it, each NI x NJ fragments of
+// 32 x 32.  A stage in LDS always has room for 256 columns.
+template <int ROWS_, int COLS_, int WAVES_, int NI_>
+struct ShapeB16 {
+  static constexpr int ROWS = ROWS_, COLS = COLS_, WAVES = WAVES_, NI = NI_;
+  static constexpr int WM = ROWS / (32 * NI), WN = WAVES / WM;   // wavefronts down and across the tile
+  static constexpr int NJ = COLS / WN / 32;
+  static_assert(WM * NI * 32 == ROWS && WN * NJ * 32 == COLS && COLS <= TileB16::BN, "the wavefronts cover the tile");
+  static constexpr int STAGE_HALVES = (ROWS + TileB16::BN) * TileB16::BK;
 };
+typedef ShapeB16<256, 256, 8, 4> WideShapeB16;     // 2 x 4 wavefronts of 128 x 64: two to a SIMD
+typedef ShapeB16<128, 256, 4, 4> LowShapeB16;      // 1 x 4 wavefronts of 128 x 64, for products of at most 128 rows
 
-// C[M, Ncols] = A[M, K] x B[K, Ncols], one ROWS x 256 tile (ROWS = 256: wavefronts 2 x 2 of
-// 128 x 128; ROWS = 128: wavefronts 1 x 4 of 128 x 64) over the K steps s_begin .. s_end - 1
-// (s_begin < s_end).  piece == nullptr: results go through ops.store; otherwise into the dense
-// ROWS x 256 piece.
-template <typename Ops, int ROWS, int WAVES>
+// C[M, Ncols] = A[M, K] x B[K, Ncols], the tile of shape S at (m0, n0) over the K steps
+// s_begin .. s_end - 1 (s_begin < s_end).  piece == nullptr: results go through ops.store;
+// otherwise into the dense ROWS x 256 piece.
+template <typename Ops, typename S>
 __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, int s_begin, int s_end,
                                                float* __restrict__ piece) {
   using T = TileB16;
-  constexpr int NI = WAVES == 16 ? 2 : 4;                  // row fragments of a wavefront
-  constexpr int WM = ROWS / (32 * NI), WN = WAVES / WM;   // wavefronts down and across the tile
-  constexpr int NJ = T::BN / WN / 32;                      // column fragments of a wavefront
+  constexpr int ROWS = S::ROWS, WAVES = S::WAVES, NI = S::NI, NJ = S::NJ, WN = S::WN;
   constexpr int A_LOADS = ROWS / 16 / WAVES, B_LOADS = T::BN / 16 / WAVES, LOADS = A_LOADS + B_LOADS;
-  constexpr int STAGE = StageB16<ROWS>::HALVES;
+  constexpr int STAGE = S::STAGE_HALVES;
   __shared__ __attribute__((aligned(1024))) unsigned short lds[T::STAGES * STAGE];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = (wave / WN) * (32 * NI), wn = (wave % WN) * (32 * NJ);
+  const int wm = (wave / WN) * (32 * NI), wn = (wave % WN) * (32 * NJ);   // the wavefront's part of the tile
 
   // ---- loading: an instruction moves 16 rows x 64 bytes into LDS, lane l to byte 16 * l of them;
   // the lane's chunk of its row is the one that belongs in that slot
@@ -379,7 +382,10 @@ __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, i
   const int a_off = ops.a_offset(m0 + 16 * A_LOADS * wave + l_row) + l_chunk * 16;
   typename Ops::BCtx bctx[B_LOADS];
 #pragma unroll
-  for (int k = 0; k < B_LOADS; ++k) bctx[k] = ops.b_ctx(n0 + 16 * (B_LOADS * wave + k) + l_row, n0);
+  for (int k = 0; k < B_LOADS; ++k) {   // (columns of the stage past the tile's: none)
+    const int column = 16 * (B_LOADS * wave + k) + l_row;
+    bctx[k] = ops.b_ctx(column < S::COLS ? n0 + column : 0x7fffffff, n0);
+  }
 
   // Requests for the next K step (one step after the other): request(k) is load k of the LOADS a
   // wavefront contributes, step_requested() closes the step.  Past the last step the loads are
@@ -507,10 +513,11 @@ __device__ __forceinline__ void igemm_tile_b16(const Ops& ops, int m0, int n0, i
   }
 }
 
-// Tiles in column-major order, whole tiles first, then the tiles cut along K (see igemm_kernel).
-template <typename Ops, int ROWS, int WAVES>
-__global__ void __launch_bounds__(64 * WAVES, ROWS == 256 ? 1 : 2)
-igemm_b16_kernel(Ops ops, int row_tiles, TileSplit split, float* __restrict__ piece_buffer) {
+// The tiles of shape S of the columns from n_base on, in column-major order, whole tiles first,
+// then the tiles cut along K (see igemm_kernel).
+template <typename Ops, typename S>
+__global__ void __launch_bounds__(64 * S::WAVES, 1)
+igemm_b16_kernel(Ops ops, int row_tiles, int n_base, TileSplit split, float* __restrict__ piece_buffer) {
   const int whole_blocks = tile_blocks(split.whole);
   int t, s_begin = 0, s_end = k_steps_b16(ops.K);
   float* piece = nullptr;
@@ -522,22 +529,23 @@ igemm_b16_kernel(Ops ops, int row_tiles, TileSplit split, float* __restrict__ pi
     t = split.whole + q / split.pieces;
     s_begin = (q % split.pieces) * split.steps_per_piece;
     s_end = min(s_end, s_begin + split.steps_per_piece);
-    piece = piece_buffer + static_cast<size_t>(q) * ROWS * TileB16::BN;
+    piece = piece_buffer + static_cast<size_t>(q) * S::ROWS * TileB16::BN;
   }
-  igemm_tile_b16<Ops, ROWS, WAVES>(ops, (t % row_tiles) * ROWS, (t / row_tiles) * TileB16::BN, s_begin, s_end, piece);
+  igemm_tile_b16<Ops, S>(ops, (t % row_tiles) * S::ROWS, n_base + (t / row_tiles) * S::COLS, s_begin, s_end, piece);
 }
 
 // Results of the split tiles: sum of their pieces, in piece order.
-template <typename Ops, int ROWS>
+template <typename Ops, typename S>
 __global__ void __launch_bounds__(256)
-reduce_pieces_b16_kernel(Ops ops, int row_tiles, TileSplit split, const float* __restrict__ piece_buffer) {
-  constexpr int TILE = ROWS * TileB16::BN;
+reduce_pieces_b16_kernel(Ops ops, int row_tiles, int n_base, TileSplit split, const float* __restrict__ piece_buffer) {
+  constexpr int TILE = S::ROWS * TileB16::BN;
   const int local = blockIdx.x / (TILE / 256), e = (blockIdx.x % (TILE / 256)) * 256 + threadIdx.x;
-  const int t = split.whole + local;
+  const int t = split.whole + local, column = e % TileB16::BN;
+  if (column >= S::COLS) return;
   const float* p = piece_buffer + static_cast<size_t>(local) * split.pieces * TILE + e;
   float sum = 0.0f;
   for (int i = 0; i < split.pieces; ++i) sum += p[static_cast<size_t>(i) * TILE];
-  ops.store(ops.column((t / row_tiles) * TileB16::BN + e % TileB16::BN), (t % row_tiles) * ROWS + e / TileB16::BN, sum);
+  ops.store(ops.column(n_base + (t / row_tiles) * S::COLS + column), (t % row_tiles) * S::ROWS + e / TileB16::BN, sum);
 }
 
 }  // namespace conv

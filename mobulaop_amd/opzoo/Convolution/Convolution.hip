@@ -88,20 +88,16 @@ void launch_igemm(const Ops& ops, float* piece_buffer, hipStream_t stream) {
   }
 }
 
-// Wavefronts of a workgroup of the bf16 products: eight for 256-row tiles (two to a SIMD: one
-// issues matrix instructions while the other waits), four for 128-row tiles.
-constexpr int waves_b16(int rows) { return rows == 256 ? 8 : 4; }
-
-// Workgroups of igemm_b16_kernel<Ops, ROWS> the device holds at a time.
-template <typename Ops, int ROWS>
+// Workgroups of igemm_b16_kernel<Ops, S> the device holds at a time.
+template <typename Ops, typename S>
 int resident_workgroups_b16() {
   static thread_local int cached_device = -1, cached = 0;
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return 0;
   if (device != cached_device) {
     int per_cu = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, conv::igemm_b16_kernel<Ops, ROWS, waves_b16(ROWS)>,
-                                                     64 * waves_b16(ROWS), 0) != hipSuccess ||
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, conv::igemm_b16_kernel<Ops, S>, 64 * S::WAVES, 0) !=
+            hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) {
       (void)hipGetLastError();
       return 0;
@@ -112,29 +108,30 @@ int resident_workgroups_b16() {
   return cached;
 }
 
-// Pieces of the bf16 products are ROWS x 256 floats; the piece buffer holds kMaxPieceBlocks
-// pieces of 128 x 128.
-template <typename Ops, int ROWS>
-void launch_igemm_b16_rows(const Ops& ops, float* piece_buffer, hipStream_t stream) {
-  const int row_tiles = (ops.M + ROWS - 1) / ROWS;
-  const int count = row_tiles * ((ops.Ncols + conv::TileB16::BN - 1) / conv::TileB16::BN);
-  const int room = kMaxPieceBlocks * conv::Tile::BM * conv::Tile::BN / (ROWS * conv::TileB16::BN);
-  const int resident = std::min(resident_workgroups_b16<Ops, ROWS>(), room);
+// The columns from n_base on (`columns` of them) of a bf16 product in tiles of shape S.  Pieces of
+// these products are ROWS x 256 floats; the piece buffer holds kMaxPieceBlocks pieces of 128 x 128.
+template <typename Ops, typename S>
+void launch_igemm_b16_shape(const Ops& ops, int n_base, int columns, float* piece_buffer, hipStream_t stream) {
+  const int row_tiles = (ops.M + S::ROWS - 1) / S::ROWS, count = row_tiles * ((columns + S::COLS - 1) / S::COLS);
+  const int room = kMaxPieceBlocks * conv::Tile::BM * conv::Tile::BN / (S::ROWS * conv::TileB16::BN);
+  const int resident = std::min(resident_workgroups_b16<Ops, S>(), room);
   const conv::TileSplit split = split_tiles(count, conv::k_steps_b16(ops.K), resident);
   const int rest = count - split.whole;
   const dim3 grid(conv::tile_blocks(split.whole) + rest * split.pieces);
-  conv::igemm_b16_kernel<Ops, ROWS, waves_b16(ROWS)><<<grid, 64 * waves_b16(ROWS), 0, stream>>>(ops, row_tiles, split,
-                                                                                           piece_buffer);
+  conv::igemm_b16_kernel<Ops, S><<<grid, 64 * S::WAVES, 0, stream>>>(ops, row_tiles, n_base, split, piece_buffer);
   if (rest > 0)
-    conv::reduce_pieces_b16_kernel<Ops, ROWS><<<rest * (ROWS * conv::TileB16::BN / 256), 256, 0, stream>>>(
-        ops, row_tiles, split, piece_buffer);
+    conv::reduce_pieces_b16_kernel<Ops, S><<<rest * (S::ROWS * conv::TileB16::BN / 256), 256, 0, stream>>>(
+        ops, row_tiles, n_base, split, piece_buffer);
 }
 
-// Row tiles of 256, or of 128 when the product has at most 128 rows.
+// Tiles of 256 x 256, or 128 x 256 for products of at most 128 rows.  (Tried for a last round that
+// fills between half and three quarters of the device: one round of narrower tiles, 256 x 160,
+// over the same columns.  The two rounds then take as long as before -- the full round alone runs
+// slower than beside a half-empty one -- so there is one shape per product.)
 template <typename Ops>
 void launch_igemm_b16(const Ops& ops, float* piece_buffer, hipStream_t stream) {
-  if (ops.M > 128) launch_igemm_b16_rows<Ops, 256>(ops, piece_buffer, stream);
-  else launch_igemm_b16_rows<Ops, 128>(ops, piece_buffer, stream);
+  if (ops.M <= 128) launch_igemm_b16_shape<Ops, conv::LowShapeB16>(ops, 0, ops.Ncols, piece_buffer, stream);
+  else launch_igemm_b16_shape<Ops, conv::WideShapeB16>(ops, 0, ops.Ncols, piece_buffer, stream);
 }
 
 // workgroups the weight gradient aims at: four per CU of a 256-CU device
