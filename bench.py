@@ -175,10 +175,10 @@ def short_roialign_run(name, steps=5, warmup=2):
     return out
 
 
-def short_conv_run(steps=5, warmup=2):
-    """cfg5 with fp32 products: ms per step (forward + data gradient + weight gradient),
-    fraction of the fp32 matrix peak, parity of the first two images against torch's
-    conv2d on the CPU."""
+def short_conv_run(mode='fp32', steps=5, warmup=2):
+    """cfg5 with fp32 products, or with operands rounded to bf16: ms per step (forward + data
+    gradient + weight gradient), fraction of the matrix peak of that type, parity of the
+    first two images against torch's conv2d on the CPU."""
     import torch
     import torch.nn.functional as F
     from mobulaop_amd import native
@@ -192,7 +192,7 @@ def short_conv_run(steps=5, warmup=2):
     lib = native.library()
     stream = torch.cuda.current_stream().cuda_stream
     geo = [ctypes.c_int(v) for v in (N, C, H, W, D, K, K, 1, 1, 1, 1, 1, 1)]
-    native.set_option('conv_compute', 0)
+    native.set_option('conv_compute', {'fp32': 0, 'bf16': 1}[mode])
 
     def ptr(t):
         return ctypes.c_void_p(t.data_ptr())
@@ -222,8 +222,10 @@ def short_conv_run(steps=5, warmup=2):
 
     def rel(a, b):
         return float((a.cpu().double() - b.double()).abs().max() / b.double().abs().max())
-    return {'step': 'forward + data gradient + weight gradient, fp32 products', 'ms_per_step': ms,
-            'frac': flops / (ms * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 'bound': 'mfma fp32',
+    native.set_option('conv_compute', 0)
+    peak = MFMA_FP32_PEAK_TFLOPS if mode == 'fp32' else MFMA_BF16_PEAK_TFLOPS
+    return {'step': 'forward + data gradient + weight gradient, %s products' % mode, 'ms_per_step': ms,
+            'frac': flops / (ms * 1e-3) / 1e12 / peak, 'bound': 'mfma ' + mode,
             'tflops': flops / (ms * 1e-3) / 1e12,
             'parity_max_rel': {'forward': rel(y[:2], yr.detach()), 'data_gradient': rel(dx[:2], xr.grad)},
             'parity_sample': 'first 2 images against torch conv2d on the CPU'}
@@ -582,7 +584,8 @@ def main():
         for name in ('cfg1', 'cfg3', 'cfg4'):
             out['configs'][name] = short_roialign_run(name)
             torch.cuda.empty_cache()
-        out['configs']['cfg5'] = short_conv_run()
+        out['configs']['cfg5'] = short_conv_run('fp32')
+        out['configs']['cfg5_bf16'] = short_conv_run('bf16')
     print(json.dumps(out))
 
 
