@@ -43,15 +43,38 @@ inline int blocked_rows_per_pass(int C, long long H, long long W, int PH, int PW
   return min(PH, B::STAGE / (B::CB * PW));
 }
 
+struct OrderArgs { const float* rois; int* order; int R; float scale; int H, W; long long num_images; };
+
+template <int NT, int MAXC>
+__device__ __forceinline__ void roi_order_body(int* hist, int* wave_sum, int* carry, const float* __restrict__ rois,
+                                               int R, float scale, int H, int W, long long num_images,
+                                               int* __restrict__ order);
+
 // out[n][cb][p][CB] = in[n][cb*CB + k][p]; channels past C are written as zero.
+// With oa.order set the launch has one more column of workgroups, the first of which sorts the
+// ROIs (roi_order_body with the cells that fit the tile's LDS) while the others copy: the
+// ordering of a few thousand ROIs then costs nothing beside a copy that takes several times as long.
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
-transpose_to_blocked_kernel(const T* __restrict__ in, T* __restrict__ out, int C, int P) {
+transpose_to_blocked_kernel(const T* __restrict__ in, T* __restrict__ out, int C, int P, OrderArgs oa) {
   constexpr int CB = BlockOf<T>::CB;
   struct alignas(4 * sizeof(T)) V4 { T v[4]; };
   __shared__ T tile[CB][65];
+  int bx = blockIdx.x;
+  if (oa.order != nullptr) {
+    if (bx == 0) {
+      if (blockIdx.y == 0 && blockIdx.z == 0) {
+        constexpr int WORDS = static_cast<int>(sizeof(tile) / 4), MAXC = WORDS - 24;
+        int* const words = reinterpret_cast<int*>(&tile[0][0]);
+        roi_order_body<256, MAXC>(words, words + MAXC + 1, words + MAXC + 20, oa.rois, oa.R, oa.scale, oa.H, oa.W,
+                                  oa.num_images, oa.order);
+      }
+      return;
+    }
+    --bx;
+  }
   const int n = blockIdx.z, cb = blockIdx.y, cblk = gridDim.y;
-  const int p0 = blockIdx.x * 64, c0 = cb * CB;
+  const int p0 = bx * 64, c0 = cb * CB;
   const T* src = in + static_cast<size_t>(n) * C * P;
   T* dst = out + (static_cast<size_t>(n) * cblk + cb) * P * CB;
   if (VEC) {
@@ -103,20 +126,19 @@ transpose_to_blocked_kernel(const T* __restrict__ in, T* __restrict__ out, int C
 // rows of cells walked in alternating direction): consecutive wavefronts then
 // read neighbouring parts of the map.  One workgroup; counting sort with the
 // histogram in LDS.  ROIs that name no image sort last.
-__global__ void __launch_bounds__(1024)
-roi_order_kernel(const float* __restrict__ rois, int R, float scale, int H, int W,
-                 long long num_images, int* __restrict__ order) {
+// (the body: NT threads of one workgroup, at most MAXC cells; hist holds MAXC + 1 counters)
+template <int NT, int MAXC>
+__device__ __forceinline__ void roi_order_body(int* hist, int* wave_sum, int* carry, const float* __restrict__ rois,
+                                               int R, float scale, int H, int W, long long num_images,
+                                               int* __restrict__ order) {
   using K = FwdBlocked;
-  __shared__ int hist[K::MAXCELLS + 1];
-  __shared__ int wave_sum[16];
-  __shared__ int carry;
   int cell = K::CELL;
   long long cy = (H + cell - 1) / cell, cx = (W + cell - 1) / cell;
-  while (cy * cx * num_images > K::MAXCELLS && cell < (1 << 20)) {
+  while (cy * cx * num_images > MAXC && cell < (1 << 20)) {
     cell *= 2;
     cy = (H + cell - 1) / cell; cx = (W + cell - 1) / cell;
   }
-  const int cells = cy * cx * num_images > K::MAXCELLS ? 1 : static_cast<int>(cy * cx * num_images);
+  const int cells = cy * cx * num_images > MAXC ? 1 : static_cast<int>(cy * cx * num_images);
   auto key_of = [&](int r) {
     const float* q = rois + static_cast<long long>(r) * 5;
     const int b = static_cast<int>(q[0]);
@@ -128,13 +150,13 @@ roi_order_kernel(const float* __restrict__ rois, int R, float scale, int H, int 
     const int sx = (iy & 1) ? static_cast<int>(cx) - 1 - ix : ix;
     return static_cast<int>((b * cy + iy) * cx + sx);
   };
-  for (int i = threadIdx.x; i <= cells; i += 1024) hist[i] = 0;
-  if (threadIdx.x == 0) carry = 0;
+  for (int i = threadIdx.x; i <= cells; i += NT) hist[i] = 0;
+  if (threadIdx.x == 0) *carry = 0;
   __syncthreads();
-  for (int r = threadIdx.x; r < R; r += 1024) atomicAdd(&hist[key_of(r)], 1);
+  for (int r = threadIdx.x; r < R; r += NT) atomicAdd(&hist[key_of(r)], 1);
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int base = 0; base <= cells; base += 1024) {
+  for (int base = 0; base <= cells; base += NT) {
     const int i = base + threadIdx.x;
     const int v = i <= cells ? hist[i] : 0;
     int incl = v;
@@ -144,14 +166,23 @@ roi_order_kernel(const float* __restrict__ rois, int R, float scale, int H, int 
     }
     if (lane == 63) wave_sum[wave] = incl;
     __syncthreads();
-    int before = carry;
+    int before = *carry;
     for (int w = 0; w < wave; ++w) before += wave_sum[w];
     if (i <= cells) hist[i] = before + incl - v;
     __syncthreads();
-    if (threadIdx.x == 1023) carry = before + incl;
+    if (threadIdx.x == NT - 1) *carry = before + incl;
     __syncthreads();
   }
-  for (int r = threadIdx.x; r < R; r += 1024) order[atomicAdd(&hist[key_of(r)], 1)] = r;
+  for (int r = threadIdx.x; r < R; r += NT) order[atomicAdd(&hist[key_of(r)], 1)] = r;
+}
+
+__global__ void __launch_bounds__(1024)
+roi_order_kernel(const float* __restrict__ rois, int R, float scale, int H, int W,
+                 long long num_images, int* __restrict__ order) {
+  __shared__ int hist[FwdBlocked::MAXCELLS + 1];
+  __shared__ int wave_sum[16];
+  __shared__ int carry;
+  roi_order_body<1024, FwdBlocked::MAXCELLS>(hist, wave_sum, &carry, rois, R, scale, H, W, num_images, order);
 }
 
 // A row sample: byte offsets of its low and high row in a channel block's

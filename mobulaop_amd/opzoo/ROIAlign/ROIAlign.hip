@@ -29,6 +29,7 @@ enum Impl { kAuto = 0, kTiled = 1, kNaive = 2 };
 // Helper kernels move to a second stream only above these sizes (measured: below
 // them the hand-over costs more than the overlap gains).
 constexpr int kSideStreamRois = 4096;
+constexpr int kOrderInCopyRois = 16384;   // ROIs that the workgroup riding along with the transposition sorts
 constexpr long long kSideStreamBytes = 64ll << 20;
 // Maps up to this size are gathered in the caller's ROI order: each of the eight
 // L2 caches (4 MB) then holds its eighth of the map's channel blocks whole.
@@ -226,21 +227,24 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
     // ROIs are visited in spatial order when the map is larger than the L2 caches
     // hold; a small map is read in the caller's order and the ordering kernel is left out
     int* const order = xt_bytes > kSortedAboveBytes ? reinterpret_cast<int*>(ws + xt_bytes) : nullptr;
-    // the ROI ordering (one small workgroup) runs beside the transposition
-    // (handing work to a second stream and waiting for it costs 10-15 us: only
-    // worth it when the ordering of many ROIs would otherwise delay the gather)
-    mobula_hip::SideStream side(stream, !fixed && order != nullptr && p.R > kSideStreamRois);
-    if (order != nullptr)
+    // the ROI ordering (one small workgroup) runs beside the transposition: in the same launch
+    // for up to kOrderInCopyRois ROIs (nothing to hand over), on a second stream above that
+    // (handing work to a second stream and waiting for it costs 10-15 us: only worth it when
+    // the ordering of many ROIs would otherwise delay the gather)
+    const bool order_in_copy = order != nullptr && p.R <= kOrderInCopyRois;
+    mobula_hip::SideStream side(stream, !fixed && order != nullptr && !order_in_copy && p.R > kSideStreamRois);
+    if (order != nullptr && !order_in_copy)
       roialign::roi_order_kernel<<<1, 1024, 0, side.get()>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
-    const dim3 tgrid(static_cast<unsigned>((pixels + 63) / 64), static_cast<unsigned>(cblk),
-                     static_cast<unsigned>(p.N));
+    const roialign::OrderArgs oa{rois, order_in_copy ? order : nullptr, static_cast<int>(p.R), p.scale, p.H, p.W, p.N};
+    const dim3 tgrid(static_cast<unsigned>((pixels + 63) / 64) + (order_in_copy ? 1u : 0u),
+                     static_cast<unsigned>(cblk), static_cast<unsigned>(p.N));
     const bool vec = pixels % 4 == 0 && reinterpret_cast<size_t>(x) % (4 * sizeof(T)) == 0;
     if (vec)
       roialign::transpose_to_blocked_kernel<T, true><<<tgrid, 256, 0, stream>>>(
-          x, xt, p.C, static_cast<int>(pixels));
+          x, xt, p.C, static_cast<int>(pixels), oa);
     else
       roialign::transpose_to_blocked_kernel<T, false><<<tgrid, 256, 0, stream>>>(
-          x, xt, p.C, static_cast<int>(pixels));
+          x, xt, p.C, static_cast<int>(pixels), oa);
     side.join();
     if (small_grid) {
       mobula_hip::KernelTimer timer("forward_blocked_kernel", stream, !fixed);   // (its events are allocations)
