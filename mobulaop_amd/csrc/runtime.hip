@@ -39,8 +39,8 @@ struct Scratch {
   void* ptr = nullptr;
   size_t bytes = 0;
   hipStream_t last = nullptr;   // stream of the last call that used the buffer
-  hipEvent_t idle = nullptr;    // recorded behind that call when it did not wait itself
-  bool busy = false;            // `idle` is recorded and not known to have passed
+  hipEvent_t idle = nullptr;    // recorded on `last` when a call on another stream has to wait for it
+  bool busy = false;            // work on `last` may still use the buffer
   bool pinned = false;          // a call was recorded into a HIP graph while using the buffer:
                                 // replays use this very address, so it is neither freed nor moved
 };
@@ -68,7 +68,17 @@ void* workspace(size_t bytes) {
   if (s == nullptr) return nullptr;
   CallState& st = call_state();
   if (s->busy && s->last != st.stream) {
-    MOBULA_HIP_TRY(hipStreamWaitEvent(st.stream, s->idle, 0));
+    // The previous call went to another stream and did not wait: this stream waits for what that
+    // one holds now (an event is only recorded here, when the stream changes; an event behind
+    // every call costs each call boundary some ten microseconds).  A stream that no longer
+    // exists has finished its work; whatever else goes wrong, wait for the device.
+    if (s->idle == nullptr && hipEventCreateWithFlags(&s->idle, hipEventDisableTiming) != hipSuccess)
+      s->idle = nullptr;
+    if (s->idle == nullptr || hipEventRecord(s->idle, s->last) != hipSuccess ||
+        hipStreamWaitEvent(st.stream, s->idle, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      MOBULA_HIP_TRY(hipDeviceSynchronize());
+    }
     if (failed()) return nullptr;
   }
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -277,19 +287,7 @@ void finish_call() {
   if (st.used_workspace) {
     st.used_workspace = false;
     Scratch* const s = scratch_of_current_device();
-    if (s != nullptr) {
-      s->busy = false;
-      if (!st.synchronous) {   // the buffer stays in use until the stream gets here
-        if (s->idle == nullptr && hipEventCreateWithFlags(&s->idle, hipEventDisableTiming) != hipSuccess)
-          s->idle = nullptr;
-        if (s->idle != nullptr && hipEventRecord(s->idle, st.stream) == hipSuccess) {
-          s->busy = true;
-        } else {               // no event: wait here instead
-          (void)hipGetLastError();
-          MOBULA_HIP_TRY(hipStreamSynchronize(st.stream));
-        }
-      }
-    }
+    if (s != nullptr) s->busy = !st.synchronous;   // the buffer stays in use until the stream gets here
   }
   st.extents.clear();
 }

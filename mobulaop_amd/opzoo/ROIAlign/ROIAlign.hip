@@ -449,15 +449,17 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     MOBULA_HIP_TRY(hipGetLastError());
     return;
   }
-  // the pre-pass (small, latency-bound kernels) runs beside the dy transposition,
-  // when that is long enough to hide it
+  // the pre-pass (small, latency-bound kernels) runs beside the dy transposition, when that is
+  // long enough to hide it: the transposition on the second stream, the pre-pass -- the longer of
+  // the two beside a copy that saturates the memory -- on the caller's, so that the tile owners
+  // follow it without waiting for a signal from another queue
   // (without a second stream the transposition shares the launch of the list builder instead)
   const bool forked = static_cast<long long>(sizeof(T)) * p.n_out >= kSideStreamBytes &&
                       mobula_hip::option("side_stream", 1) != 0;
   mobula_hip::SideStream side(stream, forked);
   const int tw = tile_columns(p);
   if (use_tiled() && roialign::backward_blocked_supports(p.PH, p.PW, p.S) &&
-      plan_tiles<T>(p, rois, roialign::kTileRows, tw, /*with_dyb=*/true, side.get(), &plan,
+      plan_tiles<T>(p, rois, roialign::kTileRows, tw, /*with_dyb=*/true, stream, &plan,
                     side.get() == stream ? dy : nullptr)) {
     const int cblk = (p.C + BB::CB - 1) / BB::CB;
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
@@ -465,7 +467,7 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     if (grid < (1ll << 31) && dl.blocks < (1ll << 31) && (dl.per > 0 || dl.cap >= 4)) {
       const int pwp = plan.layout.col_stride;
       if (p.R > 0 && !plan.dy_transposed)
-        roialign::transpose_dy_blocked_kernel<T><<<static_cast<unsigned>(dl.blocks), 256, dl.lds, stream>>>(
+        roialign::transpose_dy_blocked_kernel<T><<<static_cast<unsigned>(dl.blocks), 256, dl.lds, side.get()>>>(
             dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dl.per, p.R, dl.cap);
       side.join();
       {
