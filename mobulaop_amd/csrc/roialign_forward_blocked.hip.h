@@ -210,17 +210,17 @@ __device__ __forceinline__ typename LaneData<T>::type buffer_load_lane(__amdgpu_
 
 // Number of workgroups for R ROIs and cblk channel blocks (see the job decode
 // at the top of forward_blocked_kernel).
-inline long long blocked_grid(long long R, int cblk) {
-  using K = FwdBlocked;
+// (nw: wavefronts per workgroup of the kernel that is launched)
+inline long long blocked_grid(long long R, int cblk, int nw = FwdBlocked::NW) {
   long long per_xcd;
   if (cblk >= 8) per_xcd = R * ((cblk + 7) / 8);
   else per_xcd = (R + (8 / cblk) - 1) / (8 / cblk);
-  return 8 * ((per_xcd + K::NW - 1) / K::NW);
+  return 8 * ((per_xcd + nw - 1) / nw);
 }
 
 // The same for channels-last maps (see the job decode).
-inline long long blocked_grid_nhwc(long long R, int cblk) {
-  return 8 * (((R + 7) / 8 * cblk + FwdBlocked::NW - 1) / FwdBlocked::NW);
+inline long long blocked_grid_nhwc(long long R, int cblk, int nw = FwdBlocked::NW) {
+  return 8 * (((R + 7) / 8 * cblk + nw - 1) / nw);
 }
 
 template <typename T, bool NHWC>

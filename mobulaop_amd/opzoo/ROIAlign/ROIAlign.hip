@@ -175,9 +175,10 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
   const long long pixels = static_cast<long long>(p.H) * p.W;
   const int cblk = (p.C + CB - 1) / CB;
   const int rpp = roialign::blocked_rows_per_pass<T>(p.C, p.H, p.W, p.PH, p.PW);
-  const long long grid = roialign::blocked_grid(p.R, cblk);
-  const bool fits = rpp > 0 && p.N > 0 && p.N < 65536 && cblk < 65536 && grid < (1ll << 31);
   const bool small_grid = p.S == 1 || p.S == 2;   // else: sampling grids above 2 x 2, merged lists
+  const int nw = small_grid ? FB::NW : roialign::FwdMerged::NW;   // wavefronts per workgroup of the gather
+  const long long grid = roialign::blocked_grid(p.R, cblk, nw);
+  const bool fits = rpp > 0 && p.N > 0 && p.N < 65536 && cblk < 65536 && grid < (1ll << 31);
   if (p.nhwc) {
     // the map is read where it lies: no copy, only the ROI ordering before the gather
     if (!fits || !nhwc_forward_supported<T>(p) || reinterpret_cast<size_t>(x) % 16 != 0 ||
@@ -192,7 +193,7 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
       if (failed()) return;
       roialign::roi_order_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.H, p.W, p.N, order);
     }
-    const long long grid = roialign::blocked_grid_nhwc(p.R, cblk);
+    const long long grid = roialign::blocked_grid_nhwc(p.R, cblk, nw);
     if (small_grid) {
       mobula_hip::KernelTimer timer("forward_blocked_kernel", stream);
       roialign::forward_blocked_kernel<T, true><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
@@ -200,7 +201,7 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
     } else {
       {
         mobula_hip::KernelTimer timer("forward_merged_kernel", stream);
-        roialign::forward_merged_kernel<T, true><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+        roialign::forward_merged_kernel<T, true><<<static_cast<unsigned>(grid), nw * 64, 0, stream>>>(
             x, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, p.PH, p.R);
       }
       // the boxes that kernel leaves out (sampling grids of more than 64 points per axis)
@@ -254,7 +255,7 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
       // every pixel of a bin is loaded once
       {
         mobula_hip::KernelTimer timer("forward_merged_kernel", stream, !fixed);
-        roialign::forward_merged_kernel<T, false><<<static_cast<unsigned>(grid), FB::NW * 64, 0, stream>>>(
+        roialign::forward_merged_kernel<T, false><<<static_cast<unsigned>(grid), nw * 64, 0, stream>>>(
             xt, rois, order, y, p.scale, p.C, p.H, p.W, p.PH, p.PW, p.S, p.N, cblk, rpp, p.R);
       }
       // the boxes that kernel leaves out (sampling grids of more than 64 points per axis), from the map itself
