@@ -444,13 +444,29 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
       ob.dyg = dyg; ob.xg = xg; ob.dw = dw; ob.g = g; ob.M = g.D; ob.Ncols = g.C * g.KH * g.KW;
       ob.K = static_cast<int>(g.N * Gp); ob.Gp = static_cast<int>(Gp); ob.Wg = Wg; ob.accumulate = accumulate;
       ob.copy_bytes = static_cast<unsigned>(x_room);
-      const dim3 pgrid_dy(g.N * g.D, static_cast<unsigned>((Gp + 2047) / 2048));
-      conv::to_padded_bf16_kernel<<<pgrid_dy, 256, 0, stream>>>(dy, dyg, nullptr, g.OH, g.OW, 0, 0, Hg, Wg,
-                                                              static_cast<int>(Gp));
-      const dim3 pgrid_x(g.N * g.C, static_cast<unsigned>((Gp + 2047) / 2048));
-      conv::to_padded_bf16_kernel<<<pgrid_x, 256, 0, stream>>>(
-          x, xg, reinterpret_cast<unsigned short*>(ws + dy_room + x_room), g.H, g.W, g.pad_h, g.pad_w, Hg, Wg,
-          static_cast<int>(Gp));
+      unsigned short* const xg1 = reinterpret_cast<unsigned short*>(ws + dy_room + x_room);
+      // whole grid rows per workgroup and 16-byte loads where rows of both tensors allow it (a span
+      // of rows must be a multiple of 8 positions: Wg even and four rows, or any rows if Wg % 8 == 0)
+      int rows = (conv::kPaddedSpan - 32) / Wg;   // (the last span also takes the tail of the plane: up to 31 positions)
+      if (Wg % 8 != 0) rows = Wg % 2 == 0 ? rows / 4 * 4 : 0;
+      const bool vec = rows > 0 && g.W % 4 == 0 && g.OW % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(dy) % 16 == 0;
+      if (vec) {
+        rows = std::min(rows, (Hg + 3) / 4 * 4);
+        const unsigned spans = static_cast<unsigned>((Hg + rows - 1) / rows);
+        conv::to_padded_bf16_rows_kernel<<<dim3(g.N * g.D, spans), 256, 0, stream>>>(
+            dy, dyg, nullptr, g.OH, g.OW, 0, 0, Hg, Wg, static_cast<int>(Gp), rows);
+        conv::to_padded_bf16_rows_kernel<<<dim3(g.N * g.C, spans), 256, 0, stream>>>(
+            x, xg, xg1, g.H, g.W, g.pad_h, g.pad_w, Hg, Wg, static_cast<int>(Gp), rows);
+      } else {
+        // a plane in as few, equally long spans as fit the kernel's LDS
+        const int spans = static_cast<int>((Gp + conv::kPaddedSpan - 1) / conv::kPaddedSpan);
+        const int span = static_cast<int>((Gp / 8 + spans - 1) / spans * 8);
+        conv::to_padded_bf16_kernel<<<dim3(g.N * g.D, spans), 256, 0, stream>>>(dy, dyg, nullptr, g.OH, g.OW, 0, 0, Hg,
+                                                                               Wg, static_cast<int>(Gp), span);
+        conv::to_padded_bf16_kernel<<<dim3(g.N * g.C, spans), 256, 0, stream>>>(
+            x, xg, xg1, g.H, g.W, g.pad_h, g.pad_w, Hg, Wg, static_cast<int>(Gp), span);
+      }
       launch_igemm_b16(ob, reinterpret_cast<float*>(ws + dy_room + 2 * x_room), stream);
       MOBULA_HIP_TRY(hipGetLastError());
       return;

@@ -228,6 +228,8 @@ def test_full_cfg5_against_torch(mode):
     (2, 33, 30, 26, 300, (3, 3), (1, 1), (2, 2), (1, 1)),     # strides: two row tiles, gathered weight gradient
     (9, 256, 28, 28, 256, (3, 3), (1, 1), (1, 1), (1, 1)),    # several images to a tile, K cut into pieces
     (1, 16, 60, 60, 16, (1, 1), (0, 0), (1, 1), (1, 1)),      # one tap
+    (2, 8, 96, 96, 12, (3, 3), (1, 1), (1, 1), (1, 1)),       # planes of several spans in the padded copies
+    (1, 8, 70, 104, 8, (1, 3), (0, 1), (1, 1), (1, 1)),       # likewise, no padded rows
 ])
 def test_bf16_mode_is_exact_on_bf16_valued_operands(case):
     # Mode 1 rounds both operands of every product to bf16 and accumulates in fp32: against
