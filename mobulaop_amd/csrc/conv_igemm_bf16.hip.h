@@ -18,12 +18,12 @@
 // K runs in steps of 32 channels, the taps of a channel block one after the other
 // (step = block * taps + tap): the taps of a block read the same 64-byte pieces of
 // the same pixels, so after the first tap a step's gathered operand comes from
-// the L1 and L2 caches.  A workgroup of four
-// wavefronts owns a tile of 256 x 256 (each wavefront 128 x 128: 4 x 4
-// accumulators of v_mfma_f32_32x32x16_bf16, 256 accumulator registers, one
-// workgroup per CU), or 128 x 256 for products of at most 128 rows (each
-// wavefront 128 x 64).  A tile this large needs 64 bytes from memory and 128
-// bytes from LDS per matrix instruction, half of what 128 x 128 tiles need.
+// the L1 and L2 caches.  A workgroup owns a tile of 256 x 256: eight wavefronts
+// of 128 x 64 (4 x 2 accumulators of v_mfma_f32_32x32x16_bf16, 128 accumulator
+// registers, two wavefronts to a SIMD so that one multiplies while the other
+// waits; one workgroup per CU), or 128 x 256 with four such wavefronts for
+// products of at most 128 rows.  A tile this large needs 64 bytes from memory
+// per matrix instruction, half of what 128 x 128 tiles need.
 //
 // Operands go from memory straight into LDS (buffer loads with the LDS flag,
 // 16 bytes per lane: one instruction moves sixteen 64-byte rows), three stages
