@@ -443,8 +443,11 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
       unsigned short* const xg = reinterpret_cast<unsigned short*>(ws + dy_room);
       ob.dyg = dyg; ob.xg = xg; ob.dw = dw; ob.g = g; ob.M = g.D; ob.Ncols = g.C * g.KH * g.KW;
       ob.K = static_cast<int>(g.N * Gp); ob.Gp = static_cast<int>(Gp); ob.Wg = Wg; ob.accumulate = accumulate;
-      ob.copy_bytes = static_cast<unsigned>(x_room);
-      unsigned short* const xg1 = reinterpret_cast<unsigned short*>(ws + dy_room + x_room);
+      // the shifted copy follows the first one directly (x_bytes is a multiple of 64): the reads of
+      // the last plane that run past its end then land in the other copy or beyond the buffer
+      // (zeros), never in workspace bytes that nothing wrote
+      ob.copy_bytes = static_cast<unsigned>(x_bytes);
+      unsigned short* const xg1 = reinterpret_cast<unsigned short*>(ws + dy_room + x_bytes);
       // whole grid rows per workgroup and 16-byte loads where rows of both tensors allow it (a span
       // of rows must be a multiple of 8 positions: Wg even and four rows, or any rows if Wg % 8 == 0)
       int rows = (conv::kPaddedSpan - 32) / Wg;   // (the last span also takes the tail of the plane: up to 31 positions)

@@ -220,6 +220,22 @@ def test_full_cfg5_against_torch(mode):
         native.set_option('conv_compute', 0)
 
 
+def _leave_nan_patterns_in_the_workspace():
+    # The bf16 products keep copies of their operands in the calling thread's workspace, which
+    # is not cleared between calls: a product of NaN inputs (conv_compute must be 1) leaves NaN
+    # bit patterns behind, so a later call that read bytes it had not written itself would show.
+    x = torch.full((2, 32, 40, 40), float('nan'), device='cuda')
+    w = torch.full((32, 32, 3, 3), float('nan'), device='cuda')
+    y = torch.empty(2, 32, 40, 40, device='cuda')
+    geo = _ci(2, 32, 40, 40, 32, 3, 3, 1, 1, 1, 1, 1, 1)
+    _call('conv2d_forward_c6a7aa85', ctypes.c_int(y.numel()), _ptr(x), _ptr(w), _ptr(w), ctypes.c_int(0), *geo,
+          _ptr(y))
+    dw = torch.empty_like(w)
+    _call('conv2d_backward_weight_ecf81c91', ctypes.c_int(dw.numel()), _ptr(y), _ptr(x), ctypes.c_int(0), *geo,
+          _ptr(dw))
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize('case', [
     # N, C, H, W, D, kernel, pad, stride, dilation
     (3, 64, 20, 20, 96, (3, 3), (1, 1), (1, 1), (1, 1)),      # 128-row tiles
@@ -230,6 +246,10 @@ def test_full_cfg5_against_torch(mode):
     (1, 16, 60, 60, 16, (1, 1), (0, 0), (1, 1), (1, 1)),      # one tap
     (2, 8, 96, 96, 12, (3, 3), (1, 1), (1, 1), (1, 1)),       # planes of several spans in the padded copies
     (1, 8, 70, 104, 8, (1, 3), (0, 1), (1, 1), (1, 1)),       # likewise, no padded rows
+    (1, 3, 12, 12, 5, (3, 3), (1, 1), (1, 1), (1, 1)),        # N * C odd: the padded copies end off a 256-byte boundary
+    (3, 5, 9, 11, 7, (3, 3), (1, 1), (1, 1), (1, 1)),         # likewise, odd grid width (the scalar copy)
+    (2, 20, 20, 20, 100, (3, 3), (1, 1), (1, 1), (1, 1)),     # 128-row tiles with channels not a multiple of 32
+    (1, 6, 21, 20, 9, (1, 2), (0, 0), (1, 1), (1, 1)),        # an odd shift without padding
 ])
 def test_bf16_mode_is_exact_on_bf16_valued_operands(case):
     # Mode 1 rounds both operands of every product to bf16 and accumulates in fp32: against
@@ -246,6 +266,7 @@ def test_bf16_mode_is_exact_on_bf16_valued_operands(case):
     yr.backward(rnd(dy))
     native.set_option('conv_compute', 1)
     try:
+        _leave_nan_patterns_in_the_workspace()
         xd, wd, dyd = x.cuda(), w.cuda(), dy.cuda()
         geo = _ci(N, C, H, W, D, k[0], k[1], pad[0], pad[1], stride[0], stride[1], dil[0], dil[1])
         y = torch.empty(yr.shape, device='cuda')
