@@ -161,10 +161,11 @@ void roi_align_backward_assign_86156afd(const int device_id, const int nthreads,
  * Device pointers only, 16-byte aligned.  A shape the fast kernels do not take is
  * an error (mobula_hip_last_error), not a slow path: ask
  * mobula_hip_roialign_nhwc_supported first and convert to NCHW otherwise.  Takes:
- * forward: channels a multiple of 4 (fp32) or 8 (fp16), pooled_width <= 50, one
- * image below 2 GiB; backward: fp32, channels a multiple of 4, sampling_ratio 1
- * or 2, pooled_width <= 16, pooled_height * sampling_ratio <= 32, top_diff below
- * 2 GiB. */
+ * forward: channels a multiple of 4 (fp32) or 8 (16-bit types), pooled_width <= 50,
+ * one image below 2 GiB; backward: fp32, fp16 or bfloat16, channels a multiple of
+ * 4, a fixed sampling_ratio of 1 .. 64 (an adaptive grid, sampling_ratio <= 0, is
+ * not taken: whether it fits depends on the boxes), pooled_width <= 32,
+ * pooled_height * min(sampling_ratio, 2) <= 64, R * PH * PW * C * 4 below 2 GiB. */
 void roi_align_forward_nhwc_ab78de3c(const int device_id, const int nthreads, const float* bottom_data,
                                      const float spatial_scale, const int channels, const int height,
                                      const int width, const int pooled_height, const int pooled_width,

@@ -67,26 +67,41 @@ void* workspace(size_t bytes) {
   Scratch* const s = scratch_of_current_device();
   if (s == nullptr) return nullptr;
   CallState& st = call_state();
+  auto is_capturing = [](hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (stream == nullptr) return false;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    return status == hipStreamCaptureStatusActive;
+  };
+  const bool capturing = is_capturing(st.stream);
   if (s->busy && s->last != st.stream) {
     // The previous call went to another stream and did not wait: this stream waits for what that
     // one holds now (an event is only recorded here, when the stream changes; an event behind
-    // every call costs each call boundary some ten microseconds).  A stream that no longer
-    // exists has finished its work; whatever else goes wrong, wait for the device.
-    if (s->idle == nullptr && hipEventCreateWithFlags(&s->idle, hipEventDisableTiming) != hipSuccess)
-      s->idle = nullptr;
-    if (s->idle == nullptr || hipEventRecord(s->idle, s->last) != hipSuccess ||
-        hipStreamWaitEvent(st.stream, s->idle, 0) != hipSuccess) {
-      (void)hipGetLastError();
-      MOBULA_HIP_TRY(hipDeviceSynchronize());
+    // every call costs each call boundary some ten microseconds).  The handle of that stream is
+    // used here: a caller that makes asynchronous calls keeps a stream alive until the next call
+    // of the same thread on the device has returned.  A call that was recorded into a graph (or
+    // a stream that is being recorded now) is left to the owner of the graph to order: an
+    // event there would become part of the recording.
+    if (!s->pinned && !is_capturing(s->last)) {
+      if (s->idle == nullptr && hipEventCreateWithFlags(&s->idle, hipEventDisableTiming) != hipSuccess)
+        s->idle = nullptr;
+      if (s->idle == nullptr || hipEventRecord(s->idle, s->last) != hipSuccess ||
+          hipStreamWaitEvent(st.stream, s->idle, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        if (capturing) {   // (a device-wide wait would break the recording)
+          set_error("the previous call of this thread ran on another stream and cannot be waited for while "
+                    "this stream is being captured: synchronise that stream before recording");
+          return nullptr;
+        }
+        MOBULA_HIP_TRY(hipDeviceSynchronize());
+      }
+      if (failed()) return nullptr;
     }
-    if (failed()) return nullptr;
+    s->busy = false;   // ordered behind it from here on (finish_call marks the new call)
   }
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  if (st.stream != nullptr && hipStreamIsCapturing(st.stream, &capture) != hipSuccess) {
-    (void)hipGetLastError();
-    capture = hipStreamCaptureStatusNone;
-  }
-  const bool capturing = capture == hipStreamCaptureStatusActive;
   if (s->bytes < bytes && (capturing || s->pinned)) {
     set_error("the workspace of this thread (%zu bytes) is too small for the call (%zu bytes) and cannot be "
               "replaced %s: make one ordinary call of the largest shape before recording, or call "

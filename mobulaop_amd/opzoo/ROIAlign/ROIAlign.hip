@@ -457,6 +457,13 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
   // (without a second stream the transposition shares the launch of the list builder instead)
   const bool forked = static_cast<long long>(sizeof(T)) * p.n_out >= kSideStreamBytes &&
                       mobula_hip::option("side_stream", 1) != 0;
+  if (forked) {
+    // the helper stream forks from the caller's: whatever the caller's stream has to wait for
+    // before the workspace may be written (a previous call on another stream) must be in it
+    // before the fork
+    (void)mobula_hip::workspace(256);
+    if (failed()) return;
+  }
   mobula_hip::SideStream side(stream, forked);
   const int tw = tile_columns(p);
   if (use_tiled() && roialign::backward_blocked_supports(p.PH, p.PW, p.S) &&

@@ -785,8 +785,10 @@ def test_full_size_properties(cfg):
     del y_n
     dx_n = abi.backward(dy, rois, x.shape, scale, S)
     assert_parity(dx.cpu().numpy(), dx_n.cpu().numpy(), BWD_TOL, cfg + ' bwd vs naive')
-    # (4) oracle backward on a few (image, channel) planes via the channel-sliced problem
-    ch = [0, w['data'].shape[1] // 2, w['data'].shape[1] - 1]
+    # (4) oracle backward on 32 channel planes of every image (one from each channel block, at
+    # varying positions inside it, and the last channel) via the channel-sliced problem
+    C = w['data'].shape[1]
+    ch = sorted(set([(8 * k + k % 8) % C for k in range(C // 8)] + [C - 1]))
     want_dx = oracle.backward(np.ascontiguousarray(w['dy'][:, ch]), w['rois'],
                               (x.shape[0], len(ch)) + tuple(x.shape[2:]), scale, S, impl='ordered')
     assert_parity(dx[:, ch].cpu().numpy(), want_dx, BWD_TOL, cfg + ' bwd planes')
