@@ -97,13 +97,12 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   long long slot;
   int cb;
   if (NHWC) {
-    // the caller's map: an XCD takes an eighth of the (spatially sorted) ROIs with
-    // all their channel blocks, neighbouring wavefronts read neighbouring lines
+    // the caller's map: an XCD takes an eighth of the (spatially sorted) ROIs, channel
+    // block by channel block
     const long long range = (R + 7) / 8;
-    const long long s = wi / cblk;
-    if (s >= range) return;
-    slot = xcd * range + s;
-    cb = static_cast<int>(wi - s * cblk);
+    cb = static_cast<int>(wi / range);
+    if (cb >= cblk) return;
+    slot = xcd * range + (wi - cb * range);
   } else if (cblk >= 8) {
     const int nx = (cblk - xcd + 7) >> 3;
     slot = wi / nx;
