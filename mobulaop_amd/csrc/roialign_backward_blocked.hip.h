@@ -40,6 +40,7 @@ struct BwdBlocked {
   static constexpr int CS = 32;
   static constexpr int G = 4;            // work entries per pipeline stage
   static constexpr int PWB = 8;          // pooled columns per turn (one per group of 8 lanes)
+  static constexpr int NSPLIT = 4;       // wavefronts that share a tile row of a map with few tile rows
 };
 
 inline bool backward_blocked_supports(int PH, int PW, int S) { return lists_supported(PH, PW, S); }
@@ -50,6 +51,12 @@ inline bool backward_blocked_supports(int PH, int PW, int S) { return lists_supp
 inline int backward_tile_columns(long long images, int H, int W, int cblk) {
   const long long wide = images * ((H + kTileRows - 1) / kTileRows) * ((W + BwdBlocked::TW - 1) / BwdBlocked::TW);
   return wide * kTileRows * cblk < 8192 ? BwdBlocked::TW_SMALL : BwdBlocked::TW;
+}
+
+// Wavefronts per tile row: the same maps also split every row's work list.
+inline int backward_row_split(long long images, int H, int W, int cblk) {
+  const long long wide = images * ((H + kTileRows - 1) / kTileRows) * ((W + BwdBlocked::TW - 1) / BwdBlocked::TW);
+  return wide * kTileRows * cblk < 8192 ? BwdBlocked::NSPLIT : 1;
 }
 
 // dy[r][c][ph][pw] -> dyb[cb][r][ph][PWp][32] (R: number of ROIs), zero where pw >= PW or the channel
@@ -180,19 +187,24 @@ __device__ __forceinline__ float lane_value(const unsigned __attribute__((ext_ve
 }
 
 // TO is the element type of dx (float, __half or bfloat16; sums are formed in fp32 and
-// rounded once).  TW: tile columns.
+// rounded once).  TW: tile columns.  NSPLIT: wavefronts that share a tile row: each takes
+// a contiguous part of the row's work list (whole items: an item belongs to the part its first
+// entry lies in) into a row of its own in LDS, and the parts are added in part order on the
+// way out -- for maps that give the SIMDs too few tile rows to keep them busy.
 // dy_any: the blocked fp32 copy dyb, or for channels-last tensors the caller's
 // dy[R][PH][PW][C] itself, of dx's element type.
-template <bool NHWC, typename TO, int TW>
-__global__ void __launch_bounds__(BwdBlocked::NT)
+template <bool NHWC, typename TO, int TW, int NSPLIT = 1>
+__global__ void __launch_bounds__(BwdBlocked::NT * NSPLIT)
 backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any,
                         const WorkRange* __restrict__ ranges, const WorkEntry* __restrict__ entries,
                         const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll, int C, int H,
                         int W, int PH, int PW, int cblk, unsigned dyb_bytes, unsigned list_bytes,
-                        int assign) {
+                        int assign) {   // assign: bit 0 = overwrite dx (else add to it), bit 1 = rows may be written four columns at a time
   using K = BwdBlocked;
   constexpr int RS = TW + 2;   // cells per row: one dummy on either side
-  __shared__ __attribute__((aligned(16))) float acc[K::TH * RS * K::CS];
+  static_assert(K::TH == 1, "the parts of a split row take the place of the rows of a band");
+  static_assert(TW % 4 == 0, "tiles start at multiples of four columns (the four-column write-out)");
+  __shared__ __attribute__((aligned(16))) float acc[NSPLIT * RS * K::CS];
 
   // Job decode.  Workgroups are dealt to the 8 XCDs round-robin, so blockIdx % 8
   // names the XCD: it takes the channel blocks b with b % 8 == xcd (their slice
@@ -223,18 +235,23 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
   const int r0 = ty * kTileRows + band * K::TH, q0 = tx * TW;
   const int c0 = cb * K::CB, nch = min(K::CB, C - c0);
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // = the tile row owned
-  const int rows = min(K::TH, H - r0), cols = min(TW, W - q0);
-  if (wave >= rows) return;   // no barrier below: rows are independent
+  const int part = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // which part of the row's work list
+  constexpr int wave = 0;                                               // the tile row owned within the band
+  const int cols = min(TW, W - q0);
+  if (r0 + wave >= H) return;   // (a band below the map: the same for every wavefront of the workgroup)
   const int grp = lane >> 3, quad = lane & 7;   // pooled column within a turn, channel quad
 
-  float* const row = acc + wave * (RS * K::CS);
+  float* const row = acc + part * (RS * K::CS);
   for (int i = lane; i < RS * K::CS / 4; i += 64)
     reinterpret_cast<float4*>(row)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 
   const WorkRange wr = ranges[tile * kTileRows + band * K::TH + wave];
   const int n_entries = wr.count;   // a multiple of 2 * G, and G more entries follow: the lists are padded
   const int16v* const wl = reinterpret_cast<const int16v*>(entries + wr.begin);
+  // this part's share: the items that start in [first_entry, end_entry), whole groups of 2 * G entries
+  const int rounds = n_entries / (2 * K::G);
+  const int first_entry = NSPLIT == 1 ? 0 : part * rounds / NSPLIT * (2 * K::G);
+  const int end_entry = NSPLIT == 1 ? n_entries : (part + 1) * rounds / NSPLIT * (2 * K::G);
   const int PWp = ll.col_stride;
   float* const cell0 = row + quad * 4;   // this lane's four channels of cell 0 (the left dummy)
 
@@ -299,11 +316,19 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
       *reinterpret_cast<float4*>(a) = lo;
       *reinterpret_cast<float4*>(a + K::CS) = hi;
     };
-    auto process = [&](const int16v& e, const u32x4 (&d)[K::G], const unsigned (&u)[K::G]) {
+    bool mine = NSPLIT == 1, done = false;   // (uniform) inside an item of this part; past the part's last item
+    auto process = [&](const int16v& e, const u32x4 (&d)[K::G], const unsigned (&u)[K::G], int at) {
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
         const float wy = __int_as_float(e[4 * j + 2]);
         const int fl = e[4 * j + 3];
+        if (NSPLIT > 1) {
+          if ((fl & 1) == 0) {   // an item starts here: this part's if it starts before the part's end
+            mine = at + j < end_entry;
+            done = !mine;
+          }
+          if (!mine) continue;
+        }
         if ((fl & 1) != 0) {   // (the same for the whole wavefront)
 #pragma unroll
           for (int i = 0; i < 4; ++i) g[i] = fmaf(lane_value<TI>(d[j], i), wy, g[i]);
@@ -337,36 +362,49 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
       }
     };
 
-    if (n_entries > 0) {
-      int16v e_cur = wl[0], e_nx = wl[1], e_n2;
+    if (first_entry < end_entry) {
+      const int w0 = first_entry >> 2;
+      int16v e_cur = wl[w0], e_nx = wl[w0 + 1], e_n2;
       u32x4 d_a[K::G], d_b[K::G];
       unsigned u_a[K::G], u_b[K::G];
       issue(e_cur, d_a, u_a);
-      for (int e0 = 0; e0 < n_entries; e0 += 2 * K::G) {
+      // (a part goes on past its end until the item it is in has ended: to the next item start)
+      for (int e0 = first_entry; e0 < n_entries && !done; e0 += 2 * K::G) {
         // group at e0 lives in set a, group at e0 + G in set b
         e_n2 = wl[(e0 >> 2) + 2];
         issue(e_nx, d_b, u_b);
-        process(e_cur, d_a, u_a);
+        process(e_cur, d_a, u_a, e0);
         e_cur = e_nx; e_nx = e_n2;
         e_n2 = wl[(e0 >> 2) + 3];
         issue(e_nx, d_a, u_a);   // past the end this is the padding: loaded, never used
-        process(e_cur, d_b, u_b);
+        process(e_cur, d_b, u_b, e0 + K::G);
         e_cur = e_nx; e_nx = e_n2;
       }
     }
   }
 
+  if (NSPLIT > 1) __syncthreads();   // every part of the row is complete
+  // element i of a cell, the parts added in part order
+  auto total4 = [&](int cell) {
+    float4 v = *reinterpret_cast<const float4*>(acc + cell * K::CS + quad * 4);
+#pragma unroll
+    for (int k = 1; k < NSPLIT; ++k) {
+      const float4 w = *reinterpret_cast<const float4*>(acc + k * (RS * K::CS) + cell * K::CS + quad * 4);
+      v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+    }
+    return v;
+  };
   if (NHWC) {
     // dx[n][row][col][C]: a pixel's channels of this block are contiguous;
     // eight pixels per step, a lane moves its four channels
     struct alignas(4 * sizeof(TO)) Four { TO v[4]; };
     TO* const px0 = dx_any + ((static_cast<size_t>(n) * H + r0 + wave) * W + q0) * C + c0 + quad * 4;
     if (quad * 4 < nch) {
-      for (int col = grp; col < cols; col += 8) {
-        const float4 v = *reinterpret_cast<const float4*>(row + (col + 1) * K::CS + quad * 4);
+      for (int col = grp + 8 * part; col < cols; col += 8 * NSPLIT) {
+        const float4 v = total4(col + 1);
         Four* const dst = reinterpret_cast<Four*>(px0 + static_cast<size_t>(col) * C);
         Four o;
-        if (assign) {
+        if ((assign & 1) != 0) {
           o.v[0] = from_float<TO>(v.x); o.v[1] = from_float<TO>(v.y);
           o.v[2] = from_float<TO>(v.z); o.v[3] = from_float<TO>(v.w);
         } else {
@@ -379,20 +417,59 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
     }
     return;
   }
-  // The owner writes its row: one channel plane at a time, lanes along x.
+  // The owner writes its row.
   TO* const out = dx_any + ((static_cast<size_t>(n) * C + c0) * H + r0 + wave) * W + q0;
   const size_t plane = static_cast<size_t>(H) * W;
+  if ((assign & 2) != 0) {
+    // Rows whose pieces start at multiples of four elements (the host says so): a lane reads its
+    // channel quad of four neighbouring cells -- the eight lanes of a group cover all the
+    // banks, as in the accumulation -- and writes four columns of each of its four planes at
+    // once.  (Read with lanes along x instead, the cells lie 32 words apart: one bank.)
+    struct alignas(4 * sizeof(TO)) Four { TO v[4]; };
+    if (quad * 4 < nch) {
+      for (int base = 4 * grp + 32 * part; base < cols; base += 32 * NSPLIT) {
+        float4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = total4(base + j + 1);
+        const float t[4][4] = {{v[0].x, v[1].x, v[2].x, v[3].x}, {v[0].y, v[1].y, v[2].y, v[3].y},
+                               {v[0].z, v[1].z, v[2].z, v[3].z}, {v[0].w, v[1].w, v[2].w, v[3].w}};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (quad * 4 + i >= nch) break;
+          Four* const dst = reinterpret_cast<Four*>(out + (quad * 4 + i) * plane + base);
+          Four o;
+          if ((assign & 1) != 0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o.v[j] = from_float<TO>(t[i][j]);
+          } else {
+            o = *dst;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o.v[j] = from_float<TO>(to_float(o.v[j]) + t[i][j]);
+          }
+          *dst = o;
+        }
+      }
+    }
+    return;
+  }
+  // Any other row: one channel plane at a time, lanes along x.
   // LPC lanes per channel plane (a power of two that covers the tile's columns):
   // 64 / LPC planes are written per step
   constexpr int LPC = TW <= 32 ? 32 : 64, PLANES = 64 / LPC;
   const int col = lane & (LPC - 1), first = lane / LPC;
   if (col < cols) {
-    const float* const src = row + (col + 1) * K::CS;
-    if (assign) {
-      for (int c = first; c < nch; c += PLANES) out[c * plane + col] = from_float<TO>(src[c]);
+    const float* const src = acc + (col + 1) * K::CS;
+    auto total = [&](int c) {
+      float v = src[c];
+#pragma unroll
+      for (int k = 1; k < NSPLIT; ++k) v += src[k * (RS * K::CS) + c];
+      return v;
+    };
+    if ((assign & 1) != 0) {
+      for (int c = first + PLANES * part; c < nch; c += PLANES * NSPLIT) out[c * plane + col] = from_float<TO>(total(c));
     } else {
-      for (int c = first; c < nch; c += PLANES)
-        out[c * plane + col] = from_float<TO>(to_float(out[c * plane + col]) + src[c]);
+      for (int c = first + PLANES * part; c < nch; c += PLANES * NSPLIT)
+        out[c * plane + col] = from_float<TO>(to_float(out[c * plane + col]) + total(c));
     }
   }
 }

@@ -333,7 +333,7 @@ void mobula_hip_clear_error(void) { call_state().error.clear(); }
 
 int mobula_hip_set_option(const char* name, long long value) {
   static const char* known[] = {"roialign_impl", "host_staging_device", "kernel_timing", "side_stream",
-                                "conv_compute", "roialign_tile_columns", nullptr};
+                                "conv_compute", "roialign_tile_columns", "roialign_row_split", "roialign_row_quads", nullptr};
   for (int i = 0; known[i] != nullptr; ++i) {
     if (std::strcmp(known[i], name) == 0) {
       std::lock_guard<std::mutex> lock(mobula_hip::g_mutex);

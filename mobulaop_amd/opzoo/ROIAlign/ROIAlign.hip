@@ -411,6 +411,15 @@ int tile_columns(const Problem& p) {
   return roialign::backward_tile_columns(p.N, p.H, p.W, (p.C + BB::CB - 1) / BB::CB);
 }
 
+// Wavefronts per tile row of the backward pass (1, or BwdBlocked::NSPLIT for maps with few tile
+// rows); the option "roialign_row_split" names one of the two (tests do).
+int row_split(const Problem& p) {
+  using BB = roialign::BwdBlocked;
+  const long long forced = mobula_hip::option("roialign_row_split", 0);
+  if (forced == 1 || forced == BB::NSPLIT) return static_cast<int>(forced);
+  return roialign::backward_row_split(p.N, p.H, p.W, (p.C + BB::CB - 1) / BB::CB);
+}
+
 // Fixed sampling grids only: whether an adaptive one fits the tiled backward
 // depends on the boxes, and this path has no other kernel to fall back on.
 bool nhwc_backward_supported(const Problem& p) {
@@ -441,9 +450,12 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     }
     const unsigned dy_bytes = static_cast<unsigned>(sizeof(T) * p.n_out);
     mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-    const auto kernel = tw == BB::TW ? roialign::backward_blocked_kernel<true, T, BB::TW>
-                                     : roialign::backward_blocked_kernel<true, T, BB::TW_SMALL>;
-    kernel<<<static_cast<unsigned>(roialign::backward_blocked_grid(plan.grid.total, cblk)), BB::NT, 0, stream>>>(
+    const int nsplit = row_split(p);
+    const auto kernel = nsplit > 1 ? (tw == BB::TW ? roialign::backward_blocked_kernel<true, T, BB::TW, BB::NSPLIT>
+                                                   : roialign::backward_blocked_kernel<true, T, BB::TW_SMALL, BB::NSPLIT>)
+                                   : (tw == BB::TW ? roialign::backward_blocked_kernel<true, T, BB::TW>
+                                                   : roialign::backward_blocked_kernel<true, T, BB::TW_SMALL>);
+    kernel<<<static_cast<unsigned>(roialign::backward_blocked_grid(plan.grid.total, cblk)), BB::NT * nsplit, 0, stream>>>(
         dy, dx, plan.ranges, plan.entries, plan.lists,
         plan.grid, plan.layout, p.C, p.H, p.W, p.PH, p.PW, cblk, dy_bytes,
         static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
@@ -480,12 +492,18 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
       side.join();
       {
         mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-        const auto kernel = tw == BB::TW ? roialign::backward_blocked_kernel<false, T, BB::TW>
-                                         : roialign::backward_blocked_kernel<false, T, BB::TW_SMALL>;
-        kernel<<<static_cast<unsigned>(grid), BB::NT, 0, stream>>>(
+        const int nsplit = row_split(p);
+        // every row piece of dx starts at a multiple of four elements (tile widths are): four columns per store
+        const bool quads = p.W % 4 == 0 && reinterpret_cast<size_t>(dx) % (4 * sizeof(T)) == 0 &&
+                           mobula_hip::option("roialign_row_quads", 1) != 0;
+        const auto kernel = nsplit > 1 ? (tw == BB::TW ? roialign::backward_blocked_kernel<false, T, BB::TW, BB::NSPLIT>
+                                                       : roialign::backward_blocked_kernel<false, T, BB::TW_SMALL, BB::NSPLIT>)
+                                       : (tw == BB::TW ? roialign::backward_blocked_kernel<false, T, BB::TW>
+                                                       : roialign::backward_blocked_kernel<false, T, BB::TW_SMALL>);
+        kernel<<<static_cast<unsigned>(grid), BB::NT * nsplit, 0, stream>>>(
             plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
             p.W, p.PH, p.PW, cblk, static_cast<unsigned>(plan.dyb_bytes),
-            static_cast<unsigned>(plan.list_bytes), assign ? 1 : 0);
+            static_cast<unsigned>(plan.list_bytes), (assign ? 1 : 0) | (quads ? 2 : 0));
       }
       MOBULA_HIP_TRY(hipGetLastError());
       return;

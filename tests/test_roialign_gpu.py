@@ -31,6 +31,8 @@ def _announce(request):
     yield
     abi.set_impl('auto')
     native.set_option('roialign_tile_columns', 0)
+    native.set_option('roialign_row_split', 0)
+    native.set_option('roialign_row_quads', 1)
 
 
 @pytest.mark.parametrize('impl', IMPLS)
@@ -228,13 +230,20 @@ def test_fp16_backward(C, S):
                   (want + base.astype(np.float32)).astype(np.float16).astype(np.float32), FP16_TOL, 'accumulate')
 
 
+@pytest.mark.parametrize('quads', [1, 0])
+@pytest.mark.parametrize('split', [1, 4])
 @pytest.mark.parametrize('columns', [56, 28])
 @pytest.mark.parametrize('cfg,down', [('cfg1', 8), ('cfg2', 16), ('cfg3', 32)])
-def test_both_tile_widths_of_the_backward(cfg, down, columns):
+def test_both_tile_widths_of_the_backward(cfg, down, columns, split, quads):
     """The backward chooses 28-column tiles for small maps and 56-column ones
-    otherwise; here each width is forced on every configuration."""
+    otherwise, on small maps lets four wavefronts share a tile row's work list,
+    and writes rows of maps whose width is a multiple of four 16 bytes at a
+    time; here each width, both sharings and both ways of writing are forced on
+    every configuration."""
     abi.set_impl('tiled')
     native.set_option('roialign_tile_columns', columns)
+    native.set_option('roialign_row_split', split)
+    native.set_option('roialign_row_quads', quads)
     w = workloads.make_workload(cfg, scale_down=down)
     scale, S = w['spatial_scale'], w['sampling_ratio']
     rois, dy = abi.to_dev(w['rois']), abi.to_dev(w['dy'])
@@ -249,6 +258,30 @@ def test_both_tile_widths_of_the_backward(cfg, down, columns):
     if native.roialign_channels_last_supported(True, 4, c, h, wd, w['pooled_size'], S, rois.shape[0]):
         got = abi.backward_nhwc(dy_cl, rois, (n, h, wd, c), scale, S, assign=True).permute(0, 3, 1, 2)
         assert_parity(got.cpu().numpy(), want, BWD_TOL, 'bwd channels-last')
+
+
+@pytest.mark.parametrize('C', [1, 6, 35])
+def test_four_column_write_out_with_odd_channel_counts(C):
+    """Maps whose width is a multiple of four are written four columns at a time
+    by the lanes of a channel quad: channel counts that end inside a quad, and
+    a dx that starts at an odd element (which takes the other way out)."""
+    abi.set_impl('tiled')
+    rng = np.random.default_rng(C)
+    N, H, W, PH, PW, scale, S, R = 2, 21, 60, 5, 7, 0.5, 2, 40
+    x1 = rng.uniform(-10, W / scale, R); y1 = rng.uniform(-10, H / scale, R)
+    rois = np.stack([rng.integers(0, N, R), x1, y1, x1 + rng.uniform(1, 90, R), y1 + rng.uniform(1, 40, R)],
+                    1).astype(np.float32)
+    dy = rng.standard_normal((R, C, PH, PW)).astype(np.float32)
+    want = oracle.backward(dy, rois, (N, C, H, W), scale, S, impl='ordered')
+    d_dy, d_rois = abi.to_dev(dy), abi.to_dev(rois)
+    assert_parity(abi.backward(d_dy, d_rois, (N, C, H, W), scale, S, assign=True).cpu().numpy(), want, BWD_TOL,
+                  'bwd assign')
+    room = torch.full((N * C * H * W + 1,), 3.0, device='cuda')
+    for shift in (0, 1):   # a dx at a multiple of 16 bytes, and one element further
+        seed = room[shift:shift + N * C * H * W].view(N, C, H, W)
+        seed.fill_(3.0)
+        assert_parity(abi.backward(d_dy, d_rois, (N, C, H, W), scale, S, dx=seed).cpu().numpy(), want + 3, BWD_TOL,
+                      'bwd accumulate, shift {}'.format(shift))
 
 
 def _last_bracketed_kernel():
