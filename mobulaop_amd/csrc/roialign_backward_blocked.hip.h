@@ -156,8 +156,10 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 lists_and_dy_kernel(ListsArgs lists, unsigned list_blocks, const T* __restrict__ dy, float* __restrict__ dyb,
                     int PWp, int cblk, int per, int C) {
-  if (blockIdx.x < list_blocks)
-    build_lists_body(blockIdx.x, lists);
+  if (blockIdx.x < list_blocks) {
+    if (lists.window_offsets != nullptr) build_window_lists_body(blockIdx.x, lists);
+    else build_lists_body(blockIdx.x, lists);
+  }
   else
     transpose_dy_blocked_body<T>(blockIdx.x - list_blocks, dy, dyb, C, lists.PH, lists.PW, PWp, cblk, per, lists.R, 0);
 }
@@ -191,9 +193,11 @@ __device__ __forceinline__ float lane_value(const unsigned __attribute__((ext_ve
 // a contiguous part of the row's work list (whole items: an item belongs to the part its first
 // entry lies in) into a row of its own in LDS, and the parts are added in part order on the
 // way out -- for maps that give the SIMDs too few tile rows to keep them busy.
+// WIN: the list items are windows of merged column weights (sampling grids of more than two
+// points per bin and axis) instead of pairs of sample columns.
 // dy_any: the blocked fp32 copy dyb, or for channels-last tensors the caller's
 // dy[R][PH][PW][C] itself, of dx's element type.
-template <bool NHWC, typename TO, int TW, int NSPLIT = 1>
+template <bool NHWC, typename TO, int TW, int NSPLIT = 1, bool WIN = false>
 __global__ void __launch_bounds__(BwdBlocked::NT * NSPLIT)
 backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any,
                         const WorkRange* __restrict__ ranges, const WorkEntry* __restrict__ entries,
@@ -252,7 +256,7 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
   const int rounds = n_entries / (2 * K::G);
   const int first_entry = NSPLIT == 1 ? 0 : part * rounds / NSPLIT * (2 * K::G);
   const int end_entry = NSPLIT == 1 ? n_entries : (part + 1) * rounds / NSPLIT * (2 * K::G);
-  const int PWp = ll.col_stride;
+  const int PWp = ll.pw_padded;
   float* const cell0 = row + quad * 4;   // this lane's four channels of cell 0 (the left dummy)
 
   // dyb and the sample lists as raw buffers: a scalar byte offset per entry
@@ -270,6 +274,9 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
   const __amdgpu_buffer_rsrc_t list_buf = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<AxisUnit*>(lists), 0, static_cast<int>(list_bytes), 0x00020000);
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  // what a lane holds of an item's column list: one dword of a ColPair, or two of a ColWindow
+  typedef typename std::conditional<WIN, u32x2, unsigned>::type UT;
 
   // Each wavefront streams through the work list of its tile row: entries
   // (ROI, pooled row, weight) in ROI order, four at a time, double buffered:
@@ -279,16 +286,17 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
   for (int pwb = 0; pwb < PW; pwb += K::PWB) {
     const unsigned dy_fixed = (NHWC ? cb * K::CB * E : 0u) + pwb * dy_pw;
     const unsigned list_fixed = static_cast<unsigned>(
-        (static_cast<long long>(ll.ty) * ll.row_stride + static_cast<long long>(tx) * ll.col_stride + pwb) *
-        sizeof(AxisUnit));
+        (static_cast<long long>(ll.ty) * ll.row_stride + static_cast<long long>(tx) * ll.col_stride +
+         pwb * (WIN ? 2 : 1)) * sizeof(AxisUnit));
     // a lane whose pooled column or channels do not exist loads from outside the buffer (zero, no access)
     const int dy_lane = pwb + grp < PW && quad * 4 < nch ? static_cast<int>(grp * dy_pw + quad * 4 * E)
                                                          : static_cast<int>(0x80000000u);
     // The 16-byte column sample of the lane's pooled column comes as one dword per
     // lane (lane & 3 picks it; a 4-byte load costs the texture path half of a
     // 16-byte one) and is spread over the quad with DPP moves where it is used.
-    const int list_lane = grp * 16 + (lane & 3) * 4;
-    auto issue = [&](const int16v& e, u32x4 (&d)[K::G], unsigned (&u)[K::G]) {
+    // (The 32-byte window of merged weights: two dwords per lane.)
+    const int list_lane = WIN ? grp * 32 + (lane & 3) * 8 : grp * 16 + (lane & 3) * 4;
+    auto issue = [&](const int16v& e, u32x4 (&d)[K::G], UT (&u)[K::G]) {
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
         // the item's lists, the dy of the ROI it belongs to
@@ -296,11 +304,13 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
         if (E == 4) {
           d[j] = __builtin_amdgcn_raw_buffer_load_b128(dy_buf, dy_lane, owner * dy_roi + ph * dy_ph + dy_fixed, 0);
         } else {   // four 16-bit values: eight bytes
-          typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
           const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(dy_buf, dy_lane, owner * dy_roi + ph * dy_ph + dy_fixed, 0);
           d[j] = u32x4{w.x, w.y, 0u, 0u};
         }
-        u[j] = __builtin_amdgcn_raw_buffer_load_b32(list_buf, list_lane, roi * list_roi + list_fixed, 0);
+        if constexpr (WIN)
+          u[j] = __builtin_amdgcn_raw_buffer_load_b64(list_buf, list_lane, roi * list_roi + list_fixed, 0);
+        else
+          u[j] = __builtin_amdgcn_raw_buffer_load_b32(list_buf, list_lane, roi * list_roi + list_fixed, 0);
       }
     };
     float g[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -317,7 +327,21 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
       *reinterpret_cast<float4*>(a + K::CS) = hi;
     };
     bool mine = NSPLIT == 1, done = false;   // (uniform) inside an item of this part; past the part's last item
-    auto process = [&](const int16v& e, const u32x4 (&d)[K::G], const unsigned (&u)[K::G], int at) {
+    // adds g * w[i] to the cells a, a + 1, ... of the row (N of them; all reads before the first write)
+    auto add_cells = [&](float* a, const float* w, auto count) {
+      constexpr int N = decltype(count)::value;
+      float4 v[N];
+#pragma unroll
+      for (int i = 0; i < N; ++i) v[i] = *reinterpret_cast<const float4*>(a + i * K::CS);
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        v[i].x = fmaf(g[0], w[i], v[i].x); v[i].y = fmaf(g[1], w[i], v[i].y);
+        v[i].z = fmaf(g[2], w[i], v[i].z); v[i].w = fmaf(g[3], w[i], v[i].w);
+      }
+#pragma unroll
+      for (int i = 0; i < N; ++i) *reinterpret_cast<float4*>(a + i * K::CS) = v[i];
+    };
+    auto process = [&](const int16v& e, const u32x4 (&d)[K::G], const UT (&u)[K::G], int at) {
 #pragma unroll
       for (int j = 0; j < K::G; ++j) {
         const float wy = __int_as_float(e[4 * j + 2]);
@@ -336,7 +360,89 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
 #pragma unroll
           for (int i = 0; i < 4; ++i) g[i] = lane_value<TI>(d[j], i) * wy;
         }
-        if ((fl & 2) != 0) {
+        if constexpr (WIN) {
+          if ((fl & 2) != 0) {
+            // last tap of this item on this row: g times the weights of the window's cells.
+            // The lanes lane & 3 = k of a quad hold dwords 2k and 2k + 1 of the window:
+            // quad_perm [k, k, k, k] hands them to everyone
+            const int ulo = static_cast<int>(u[j][0]), uhi = static_cast<int>(u[j][1]);
+            const int header = __builtin_amdgcn_mov_dpp(ulo, 0x00, 0xf, 0xf, true);
+            const float w[kWindowCells] = {
+                __int_as_float(__builtin_amdgcn_mov_dpp(uhi, 0x00, 0xf, 0xf, true)),
+                __int_as_float(__builtin_amdgcn_mov_dpp(ulo, 0x55, 0xf, 0xf, true)),
+                __int_as_float(__builtin_amdgcn_mov_dpp(uhi, 0x55, 0xf, 0xf, true)),
+                __int_as_float(__builtin_amdgcn_mov_dpp(ulo, 0xaa, 0xf, 0xf, true)),
+                __int_as_float(__builtin_amdgcn_mov_dpp(uhi, 0xaa, 0xf, 0xf, true)),
+                __int_as_float(__builtin_amdgcn_mov_dpp(ulo, 0xff, 0xf, 0xf, true)),
+                __int_as_float(__builtin_amdgcn_mov_dpp(uhi, 0xff, 0xf, 0xf, true))};
+            float* const a = cell0 + (header & 0xffff) * K::CS;
+            const int turns = 1 << ((__builtin_amdgcn_readfirstlane(header) >> 16) & 3);
+            // (the eight lanes of a pooled column decide alike: a window that ends early costs the LDS nothing)
+            auto add_window = [&] {
+              if (w[0] != 0.0f || w[1] != 0.0f || w[2] != 0.0f || w[3] != 0.0f)
+                add_cells(a, w, std::integral_constant<int, 4>());
+              if (w[4] != 0.0f || w[5] != 0.0f || w[6] != 0.0f)
+                add_cells(a + 4 * K::CS, w + 4, std::integral_constant<int, 3>());
+            };
+            if (turns == 1) {
+              add_window();
+            } else {
+              // Neighbouring windows overlap.  An LDS instruction costs the same with few lanes as
+              // with all, so the two windows of a pair of lane groups (a row of 16 lanes) are taken
+              // one after the other by both groups together: one group adds the even cells, the
+              // other the odd ones (the gradient and the window of the other group: its lanes,
+              // eight further).
+              const int which = grp & 1, pair = grp >> 1, rounds = turns >> 1;
+              const int ulo_x = __builtin_amdgcn_mov_dpp(ulo, 0x128, 0xf, 0xf, true);   // row_ror:8
+              const int uhi_x = __builtin_amdgcn_mov_dpp(uhi, 0x128, 0xf, 0xf, true);
+              float gx[4];
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                gx[i] = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(g[i]), 0x128, 0xf, 0xf, true));
+#pragma unroll
+              for (int t = 0; t < 2; ++t) {   // the pair's first window, then its second
+                const bool own = which == t;
+                const int vlo = own ? ulo : ulo_x, vhi = own ? uhi : uhi_x;
+                const float gg[4] = {own ? g[0] : gx[0], own ? g[1] : gx[1], own ? g[2] : gx[2], own ? g[3] : gx[3]};
+                const int hd = __builtin_amdgcn_mov_dpp(vlo, 0x00, 0xf, 0xf, true);
+                const float x0 = __int_as_float(__builtin_amdgcn_mov_dpp(vhi, 0x00, 0xf, 0xf, true));
+                const float x1 = __int_as_float(__builtin_amdgcn_mov_dpp(vlo, 0x55, 0xf, 0xf, true));
+                const float x2 = __int_as_float(__builtin_amdgcn_mov_dpp(vhi, 0x55, 0xf, 0xf, true));
+                const float x3 = __int_as_float(__builtin_amdgcn_mov_dpp(vlo, 0xaa, 0xf, 0xf, true));
+                const float x4 = __int_as_float(__builtin_amdgcn_mov_dpp(vhi, 0xaa, 0xf, 0xf, true));
+                const float x5 = __int_as_float(__builtin_amdgcn_mov_dpp(vlo, 0xff, 0xf, 0xf, true));
+                const float x6 = __int_as_float(__builtin_amdgcn_mov_dpp(vhi, 0xff, 0xf, 0xf, true));
+                const bool head = x0 != 0.0f || x1 != 0.0f || x2 != 0.0f || x3 != 0.0f;
+                const bool tail = x4 != 0.0f || x5 != 0.0f || x6 != 0.0f;
+                // this lane's cells: which, which + 2 of w[0..3]; 4 + which (and 6) of w[4..6]
+                float* const b = cell0 + ((hd & 0xffff) + which) * K::CS;
+                const float wa = which ? x1 : x0, wb = which ? x3 : x2, wc = which ? x5 : x4;
+                auto fold = [&](float4& v, float w) {
+                  v.x = fmaf(gg[0], w, v.x); v.y = fmaf(gg[1], w, v.y);
+                  v.z = fmaf(gg[2], w, v.z); v.w = fmaf(gg[3], w, v.w);
+                };
+                for (int r = 0; r < rounds; ++r)
+                  if ((pair & (rounds - 1)) == r) {
+                    if (head) {
+                      float4 va = *reinterpret_cast<const float4*>(b);
+                      float4 vb = *reinterpret_cast<const float4*>(b + 2 * K::CS);
+                      fold(va, wa); fold(vb, wb);
+                      *reinterpret_cast<float4*>(b) = va;
+                      *reinterpret_cast<float4*>(b + 2 * K::CS) = vb;
+                    }
+                    if (tail) {
+                      float4 vc = *reinterpret_cast<const float4*>(b + 4 * K::CS);
+                      float4 vd = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                      if (which == 0) vd = *reinterpret_cast<const float4*>(b + 6 * K::CS);
+                      fold(vc, wc); fold(vd, x6);
+                      *reinterpret_cast<float4*>(b + 4 * K::CS) = vc;
+                      if (which == 0) *reinterpret_cast<float4*>(b + 6 * K::CS) = vd;
+                    }
+                  }
+              }
+            }
+          }
+        } else if ((fl & 2) != 0) {
           // last tap of this ROI on this row: spread g over the column samples
           // dword k of the quad's four: quad_perm [k, k, k, k]
           const int uj = static_cast<int>(u[j]);
@@ -355,8 +461,43 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
           if (turns == 1) {
             add_both();
           } else {
-            for (int t = 0; t < turns; ++t)
-              if ((grp & (turns - 1)) == t) add_both();
+            // Neighbouring pooled columns may share cells.  An LDS instruction costs the same with
+            // few lanes as with all, so instead of letting every second column wait, the two
+            // columns of a pair of lane groups (a row of 16 lanes) are taken one after the other
+            // by both groups together: one group adds the low corners, the other the high ones
+            // (the gradient and the column pair of the other group: its lanes, eight further).
+            const int which = grp & 1, pair = grp >> 1, rounds = turns >> 1;
+            const int uj_x = __builtin_amdgcn_mov_dpp(uj, 0x128, 0xf, 0xf, true);   // row_ror:8
+            float gx[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              gx[i] = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(g[i]), 0x128, 0xf, 0xf, true));
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {   // the pair's first column, then its second
+              const bool own = which == t;
+              const int uu = own ? uj : uj_x;
+              const float gg[4] = {own ? g[0] : gx[0], own ? g[1] : gx[1], own ? g[2] : gx[2], own ? g[3] : gx[3]};
+              const unsigned pc = static_cast<unsigned>(__builtin_amdgcn_mov_dpp(uu, 0x00, 0xf, 0xf, true));
+              const int pf = __builtin_amdgcn_mov_dpp(uu, 0x55, 0xf, 0xf, true);
+              const float m0 = __int_as_float(__builtin_amdgcn_mov_dpp(uu, 0xaa, 0xf, 0xf, true));
+              const float m1 = __int_as_float(__builtin_amdgcn_mov_dpp(uu, 0xff, 0xf, 0xf, true));
+              // this lane's corner of the two samples: its cell, its weight, whether it counts
+              float* const a0 = cell0 + ((pc & 0xffff) + which) * K::CS;
+              float* const a1 = cell0 + ((pc >> 16) + which) * K::CS;
+              const float w0 = which ? m0 : 1.0f - m0, w1 = which ? m1 : 1.0f - m1;
+              const bool live0 = ((pf >> which) & 1) != 0, live1 = ((pf >> (2 + which)) & 1) != 0;
+              auto add_corner = [&](float* a, float w) {
+                float4 v = *reinterpret_cast<const float4*>(a);
+                v.x = fmaf(gg[0], w, v.x); v.y = fmaf(gg[1], w, v.y);
+                v.z = fmaf(gg[2], w, v.z); v.w = fmaf(gg[3], w, v.w);
+                *reinterpret_cast<float4*>(a) = v;
+              };
+              for (int r = 0; r < rounds; ++r)
+                if ((pair & (rounds - 1)) == r) {
+                  if (live0) add_corner(a0, w0);
+                  if (live1) add_corner(a1, w1);
+                }
+            }
           }
         }
       }
@@ -366,7 +507,7 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
       const int w0 = first_entry >> 2;
       int16v e_cur = wl[w0], e_nx = wl[w0 + 1], e_n2;
       u32x4 d_a[K::G], d_b[K::G];
-      unsigned u_a[K::G], u_b[K::G];
+      UT u_a[K::G], u_b[K::G];
       issue(e_cur, d_a, u_a);
       // (a part goes on past its end until the item it is in has ended: to the next item start)
       for (int e0 = first_entry; e0 < n_entries && !done; e0 += 2 * K::G) {

@@ -21,12 +21,17 @@
 //                           by tile row, then by sample order
 //   col list  of (roi, tx): one 16-byte ColPair per pooled column (padded to a
 //                           multiple of 8 columns): its one or two sample columns
-// The lists hold one or two sample points per bin and axis.  A larger sampling
-// grid (a ratio above 2, or the adaptive ceil(bin size)) is cut into pieces of
-// 2 x 2 points: every piece is a list item of its own, with the box, the row
-// taps and the column pairs of its own points, and the tile owners add the
-// pieces up like so many ROIs that share one dy (the gradient is a sum over
-// sample points).  `piece_offsets_kernel` numbers the pieces.
+// These lists hold one or two sample points per bin and axis.  A larger sampling
+// grid (a ratio above 2, or the adaptive ceil(bin size)) is merged instead: the
+// gradient of a pixel is dy times (sum of the row weights its row gets from the
+// bin's sample rows) times (sum of the column weights its column gets from
+// the bin's sample columns), so a bin is described by one weight per row and one
+// per column it touches.  Rows become row taps as before (one per pooled row and
+// tile row, the weights of that pooled row's samples added up).  The columns of a
+// bin are cut into windows of kWindowCells cells, window j of every pooled column
+// together forming list item j of the ROI: its column list holds one 32-byte
+// ColWindow per pooled column, and the tile owners add the items up like so many
+// ROIs that share one dy.  `window_offsets_kernel` numbers the items.
 // Sample coordinates come from roialign_geometry.h (reference operation order).
 #pragma once
 #include "roialign_tiles.hip.h"
@@ -66,61 +71,151 @@ inline int row_table_units(int slots) { return 2 + slots; }
 
 struct ListLayout {
   int ty, tx;            // tiles per image
-  int row_stride;        // 16-byte units per (roi, ty) row-tap table
-  int col_stride;        // 16-byte units per (roi, tx) column list: PW rounded up to 8
-  long long roi_stride;  // units per ROI: ty*row_stride + tx*col_stride
+  int row_stride;        // 16-byte units per (item, ty) row-tap table
+  int col_stride;        // 16-byte units per (item, tx) column list
+  long long roi_stride;  // units per item: ty*row_stride + tx*col_stride
+  int pw_padded;         // PW rounded up to 8: pooled columns of a column list (and of a row of dyb)
+  int windows;           // 1: merged weights (WindowRowTable, ColWindow), 0: sample lists (RowTapTable, ColPair)
 };
+
+constexpr int kWindowCells = 7;   // cells of a column window (with its header: eight dwords)
+
+inline bool lists_in_windows(int S) { return S != 1 && S != 2; }
 
 inline ListLayout make_list_layout(const TileGrid& tg, int PH, int PW, int S) {
   ListLayout l;
   l.ty = tg.ty; l.tx = tg.tx;
-  l.row_stride = row_table_units(PH * (S == 1 ? 1 : 2));
-  l.col_stride = (PW + 7) / 8 * 8;
+  l.pw_padded = (PW + 7) / 8 * 8;
+  l.windows = lists_in_windows(S) ? 1 : 0;
+  if (l.windows) {
+    l.row_stride = 4 + kTileRows * PH / 2 + 1;   // 64-byte index, then at most one tap per tile row and pooled row
+    l.col_stride = 2 * l.pw_padded;
+  } else {
+    l.row_stride = row_table_units(PH * (S == 1 ? 1 : 2));
+    l.col_stride = l.pw_padded;
+  }
   l.roi_stride = static_cast<long long>(l.ty) * l.row_stride + static_cast<long long>(l.tx) * l.col_stride;
   return l;
 }
 
-inline bool lists_in_pieces(int S) { return S != 1 && S != 2; }
 inline bool lists_supported(int PH, int PW, int S) {
   return PH * (S == 1 ? 1 : 2) <= kRowSlots && PW <= kMaxListPW;
 }
 
-// offsets[r] = number of the first piece of ROI r, offsets[R] = their total;
-// info[0] = the total, info[1] = 1 if some ROI's grid has more than
-// kSearchedGrid points along an axis (such ROIs are not cut up: the caller
-// takes another path).  One workgroup of 1024 threads.
+// ---- merged weights (sampling grids of more than two points per bin and axis) ----
+
+// Grids up to this many points per axis are merged (sample numbers are found from
+// coordinates in fp32: beyond this the search margin of one sample would not do).
+constexpr int kMergedGrid = 1 << 15;
+
+// The cells the samples of pooled index p can touch along one axis, [*low, *low + *span):
+// a superset, found from the first and the last sample coordinate alone (coordinates never
+// decrease with the sample number), clamped the way the interpolation clamps them
+// (opzoo/ROIAlign/bilinear.h:15-40).
+__device__ __forceinline__ void bin_cells(float start, int p, float bin, int grid, int size, int* low,
+                                          int* span) {
+  const float c0 = sample_coord(start, p, bin, 0, grid), c1 = sample_coord(start, p, bin, grid - 1, grid);
+  *low = 0; *span = 0;
+  if (c1 < -1.0f || c0 > static_cast<float>(size)) return;   // every sample lies outside [-1, size]
+  // (a coordinate that is not a number passes the reference's test; fmaxf/fminf then give the bound)
+  const AxisSample a = axis_sample(fmaxf(c0, -1.0f), size), b = axis_sample(fminf(c1, static_cast<float>(size)), size);
+  *low = a.low;
+  *span = max(b.high - a.low + 1, 1);
+}
+
+// Sum of the weights that the valid samples of pooled index p give to `cell`
+// (samples in sample order; a sample whose two cells coincide at the border counts once).
+__device__ __forceinline__ float merged_weight(float start, int p, float bin, int grid, int size, int cell) {
+  // samples that can reach the cell have coordinates in (cell - 1, cell + 1); the border
+  // cells also take what is clamped onto them.  Sample numbers from coordinates, one to
+  // spare on either side; every candidate is then evaluated exactly.
+  const float lo = cell == 0 ? -1.0f : static_cast<float>(cell - 1);
+  const float hi = cell == size - 1 ? static_cast<float>(size) : static_cast<float>(cell + 1);
+  const float origin = start + static_cast<float>(p) * bin, step = bin / static_cast<float>(grid);
+  const float fa = (lo - origin) / step - 0.5f, fb = (hi - origin) / step - 0.5f;
+  int first = 0, last = grid;
+  if (fabsf(fa) < 1.0e9f && fabsf(fb) < 1.0e9f) {   // (false for coordinates that are not numbers)
+    first = max(0, static_cast<int>(floorf(fa)) - 1);
+    last = min(grid, static_cast<int>(ceilf(fb)) + 2);
+  }
+  float w = 0.0f;
+  for (int i = first; i < last; ++i) {
+    const AxisSample a = axis_sample(sample_coord(start, p, bin, i, grid), size);
+    if (!a.valid) continue;
+    if (a.low == cell) w += a.h;
+    if (a.high == cell && a.high != a.low) w += a.l;
+  }
+  return w;
+}
+
+// What the window items of one ROI need: their number (windows per pooled column), the
+// tile columns they span and an upper bound of the row taps of one of them.
+struct WindowCount { int windows; int tiles_x; int taps; };
+__device__ __forceinline__ WindowCount count_windows(const RoiGeom& g, int PH, int PW, int H, int W, int tw) {
+  WindowCount c{0, 0, 0};
+  int widest = 0, clo = W, chi = -1;
+  for (int pw = 0; pw < PW; ++pw) {
+    int low, span;
+    bin_cells(g.start_w, pw, g.bin_w, g.grid_w, W, &low, &span);
+    if (span > 0) { widest = max(widest, span); clo = min(clo, low); chi = max(chi, low + span - 1); }
+  }
+  for (int ph = 0; ph < PH; ++ph) {
+    int low, span;
+    bin_cells(g.start_h, ph, g.bin_h, g.grid_h, H, &low, &span);
+    c.taps += span;
+  }
+  if (widest == 0 || c.taps == 0) return WindowCount{0, 0, 0};
+  c.windows = (widest + kWindowCells - 1) / kWindowCells;
+  c.tiles_x = chi / tw - clo / tw + 1;
+  return c;
+}
+
+// offsets[r] = number of the first window item of ROI r, offsets[R] = their total;
+// info[0] = the total, info[1] = 1 if some ROI's grid has more than kMergedGrid
+// points along an axis (the caller then takes another path), info[2] = an upper
+// bound of the work entries of all items (saturating at 2^30).
+// One workgroup of 1024 threads.
 __global__ void __launch_bounds__(1024)
-piece_offsets_kernel(const float* __restrict__ rois, int R, float scale, int PH, int PW, int S,
-                     int* __restrict__ offsets, int* __restrict__ info) {
+window_offsets_kernel(const float* __restrict__ rois, int R, float scale, int PH, int PW, int S, int H, int W,
+                      int tw, int* __restrict__ offsets, int* __restrict__ info) {
   __shared__ int part[1024];
+  __shared__ long long work[1024];
   __shared__ int too_big;
   const int t = threadIdx.x, share = (R + 1023) / 1024;
   const int first = min(R, t * share), last = min(R, first + share);
   if (t == 0) too_big = 0;
   __syncthreads();
-  auto pieces_of = [&](int r) {
+  auto count_of = [&](int r) {
     const RoiGeom g = roi_geometry(rois + static_cast<long long>(r) * 5, scale, PH, PW, S);
-    if (g.grid_h > kSearchedGrid || g.grid_w > kSearchedGrid || g.grid_h < 1 || g.grid_w < 1) {
+    if (g.grid_h > kMergedGrid || g.grid_w > kMergedGrid || g.grid_h < 1 || g.grid_w < 1) {
       too_big = 1;
-      return 0;
+      return WindowCount{0, 0, 0};
     }
-    return ((g.grid_h + 1) / 2) * ((g.grid_w + 1) / 2);
+    return count_windows(g, PH, PW, H, W, tw);
   };
   int sum = 0;
-  for (int r = first; r < last; ++r) sum += pieces_of(r);
+  long long entries = 0;
+  for (int r = first; r < last; ++r) {
+    const WindowCount c = count_of(r);
+    sum += c.windows;
+    entries += static_cast<long long>(c.windows) * c.tiles_x * c.taps;
+  }
   part[t] = sum;
+  work[t] = entries;
   __syncthreads();
   if (t == 0) {   // exclusive prefix over the threads
     int run = 0;
-    for (int i = 0; i < 1024; ++i) { const int c = part[i]; part[i] = run; run += c; }
+    long long all = 0;
+    for (int i = 0; i < 1024; ++i) { const int c = part[i]; part[i] = run; run += c; all += work[i]; }
     offsets[R] = run;
     info[0] = run;
+    info[2] = static_cast<int>(min(all, 1ll << 30));
   }
   __syncthreads();
   int at = part[t];
   for (int r = first; r < last; ++r) {
     offsets[r] = at;
-    at += pieces_of(r);
+    at += count_of(r).windows;
   }
   __syncthreads();
   if (t == 0) info[1] = too_big;
@@ -156,12 +251,12 @@ struct ListsArgs {
   TileBox* boxes;
   int* cursors;
   AxisUnit* lists;
-  const int* piece_offsets;
+  const int* window_offsets;   // merged weights: the first item of every ROI (null: one item per ROI)
 };
 
 __device__ __forceinline__ void build_lists_body(unsigned block, const ListsArgs& a) {
   const float* __restrict__ rois = a.rois;
-  const int items = a.items, R = a.R, PH = a.PH, PW = a.PW, S_given = a.S_given, H = a.H, W = a.W;
+  const int items = a.items, PH = a.PH, PW = a.PW, S = a.S_given, H = a.H, W = a.W;
   const float scale = a.scale;
   const long long num_images = a.num_images;
   const TileGrid tg = a.tg;
@@ -169,33 +264,15 @@ __device__ __forceinline__ void build_lists_body(unsigned block, const ListsArgs
   TileBox* __restrict__ boxes = a.boxes;
   int* __restrict__ cursors = a.cursors;
   AxisUnit* __restrict__ lists = a.lists;
-  const int* __restrict__ piece_offsets = a.piece_offsets;
   // the two bump pointers of build_tile_work_kernel, which runs after this one
   if (block == 0 && threadIdx.x < 2) cursors[threadIdx.x] = 0;
-  // item: a ROI, or (piece_offsets given) one 2 x 2 piece of a ROI's sampling grid
   const int item = static_cast<int>((block * 256u + threadIdx.x) >> 6);
   if (item >= items) return;
   const int lane = threadIdx.x & 63;
-  int roi = item;
-  if (piece_offsets != nullptr) {   // the ROI whose pieces include this one
-    int lo = 0, hi = R;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) / 2;
-      if (piece_offsets[mid] <= item) lo = mid; else hi = mid;
-    }
-    roi = lo;
-  }
-  const RoiGeom g = roi_geometry(rois + static_cast<long long>(roi) * 5, scale, PH, PW, S_given);
-  // S points per bin and axis in this item, the first of them point (y_first, x_first) of the grid
-  const int S = piece_offsets != nullptr ? 2 : S_given;
-  int y_first = 0, x_first = 0;
-  if (piece_offsets != nullptr) {
-    const int local = item - piece_offsets[roi], across = (g.grid_w + 1) / 2;
-    y_first = 2 * (local / across);
-    x_first = 2 * (local % across);
-  }
+  const int roi = item;
+  const RoiGeom g = roi_geometry(rois + static_cast<long long>(roi) * 5, scale, PH, PW, S);
   // one row sample and one column sample per lane
-  const int iy = y_first + lane % S, ix_of_lane = x_first + lane % S;
+  const int iy = lane % S, ix_of_lane = lane % S;
   AxisSample ay = axis_sample(sample_coord(g.start_h, lane / S, g.bin_h, iy, g.grid_h), H);
   ay.valid = ay.valid && lane < PH * S && iy < g.grid_h;
   AxisSample ax = axis_sample(sample_coord(g.start_w, lane / S, g.bin_w, ix_of_lane, g.grid_w), W);
@@ -282,7 +359,144 @@ __device__ __forceinline__ void build_lists_body(unsigned block, const ListsArgs
   }
 }
 
-__global__ void __launch_bounds__(256) build_lists_kernel(ListsArgs a) { build_lists_body(blockIdx.x, a); }
+// Merged weights.  Row taps of one (item, tile row): per tile row start | count << 16, then the
+// taps by tile row and pooled row: at most one per pair, ListLayout::row_stride leaves room for all.
+struct alignas(16) WindowRowTable {
+  unsigned index[kTileRows];
+  RowTap taps[kTileRows * 32];
+};
+// The cells of one window of one pooled column inside one tile column band.
+//   header  cell | turns_log << 16: `cell` is the cell of w[0] in a tile row whose cell 0 is a
+//           dummy to the left of the tile (so the tile's first column is cell 1); the window is
+//           shifted so that all seven cells lie in the tile, cells it does not reach weigh zero.
+//           turns_log: log2 of the smallest power-of-two distance (in pooled columns, at most 8)
+//           at which the windows of this item never share a cell their owner touches (w[0..3]
+//           are added together, and so are w[4..6]: a group is skipped if all of it is zero).
+//   w       weight of cells cell .. cell + 6
+struct alignas(32) ColWindow { int header; float w[kWindowCells]; };
+static_assert(sizeof(ColWindow) == 32, "eight dwords: the tile owners load one per lane");
+
+// One wavefront per window item (ROI, j): the row taps of every tile row the ROI
+// touches -- the same for all windows of a ROI -- and window j of every pooled column.
+__device__ __forceinline__ void build_window_lists_body(unsigned block, const ListsArgs& a) {
+  const int items = a.items, R = a.R, PH = a.PH, PW = a.PW, H = a.H, W = a.W;
+  const TileGrid tg = a.tg;
+  const ListLayout ll = a.ll;
+  if (block == 0 && threadIdx.x < 2) a.cursors[threadIdx.x] = 0;
+  const int item = static_cast<int>((block * 256u + threadIdx.x) >> 6);
+  if (item >= items) return;
+  const int lane = threadIdx.x & 63;
+  int roi;
+  {   // the ROI whose items include this one
+    int lo = 0, hi = R;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) / 2;
+      if (a.window_offsets[mid] <= item) lo = mid; else hi = mid;
+    }
+    roi = lo;
+  }
+  const int j = item - a.window_offsets[roi];
+  const RoiGeom g = roi_geometry(a.rois + static_cast<long long>(roi) * 5, a.scale, PH, PW, a.S_given);
+  // lane p < 32: pooled row p and pooled column p
+  int rlow = 0, rspan = 0, clow = 0, cspan = 0;
+  if (lane < PH) bin_cells(g.start_h, lane, g.bin_h, g.grid_h, H, &rlow, &rspan);
+  if (lane < PW) bin_cells(g.start_w, lane, g.bin_w, g.grid_w, W, &clow, &cspan);
+  const int wlow_mine = clow + kWindowCells * j;                    // first cell of the window
+  const int wn_mine = max(0, min(kWindowCells, cspan - kWindowCells * j));   // its cells
+  int row_lo, row_hi, col_lo, col_hi;
+  {
+    int rlo = rspan > 0 ? rlow : H, rhi = rspan > 0 ? rlow + rspan - 1 : -1;
+    int clo = wn_mine > 0 ? wlow_mine : W, chi = wn_mine > 0 ? wlow_mine + wn_mine - 1 : -1;
+    for (int off = 32; off > 0; off >>= 1) {
+      rlo = min(rlo, __shfl_xor(rlo, off)); rhi = max(rhi, __shfl_xor(rhi, off));
+      clo = min(clo, __shfl_xor(clo, off)); chi = max(chi, __shfl_xor(chi, off));
+    }
+    const bool image_ok = g.batch >= 0 && g.batch < a.num_images;
+    const bool any = image_ok && rlo <= rhi && clo <= chi;
+    row_lo = any ? rlo : 0; row_hi = any ? rhi : -1;
+    col_lo = any ? clo : 0; col_hi = any ? chi : -1;
+    const int ty0 = row_lo / tg.th, ty1 = any ? row_hi / tg.th : -1;
+    const int tx0 = col_lo / tg.tw, tx1 = any ? col_hi / tg.tw : -1;
+    if (lane == 0) a.boxes[item] = TileBox{any ? g.batch : -1, ty0 | (ty1 << 16), tx0 | (tx1 << 16), roi};
+    if (!any) return;
+  }
+  AxisUnit* const base = a.lists + static_cast<long long>(item) * ll.roi_stride;
+  const float inv_count = 1.0f / g.count;
+  {
+    // row taps: lane = tile row * 4 + k; the lane takes the pooled rows k, k + 4, ...
+    const int r = lane >> 2, k4 = lane & 3;
+    for (int ty = row_lo / tg.th; ty <= row_hi / tg.th; ++ty) {
+      const int row = ty * tg.th + r;
+      WindowRowTable* const table = reinterpret_cast<WindowRowTable*>(base + ty * ll.row_stride);
+      float w[8];
+      int at[8];
+      int mine = 0;   // taps of this lane's tile row so far
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        w[q] = 0.0f; at[q] = 0;
+        if (4 * q < PH) {   // (the same for every lane)
+          const int ph = 4 * q + k4;
+          if (ph < PH && row < H)
+            w[q] = merged_weight(g.start_h, ph, g.bin_h, g.grid_h, H, row) * inv_count;
+          const unsigned nib = static_cast<unsigned>(__ballot(w[q] != 0.0f) >> (4 * r)) & 15u;
+          at[q] = mine + __popc(nib & ((1u << k4) - 1u));
+          mine += __popc(nib);
+        }
+      }
+      int start = 0;
+      for (int q = 0; q < kTileRows; ++q) {
+        const int t = __shfl(mine, 4 * q);
+        if (q < r) start += t;
+      }
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+        if (w[q] != 0.0f) table->taps[start + at[q]] = RowTap{4 * q + k4, w[q]};
+      if (k4 == 0) table->index[r] = static_cast<unsigned>(start) | (static_cast<unsigned>(mine) << 16);
+    }
+  }
+  {
+    // windows: lane = pooled column (of eight) * 8 + dword of its ColWindow
+    const int sub = lane >> 3, slot = (lane & 7) - 1;   // slot -1: the header
+    int* const cols = reinterpret_cast<int*>(base + static_cast<long long>(ll.ty) * ll.row_stride);
+    for (int tx = col_lo / tg.tw; tx <= col_hi / tg.tw; ++tx) {
+      for (int pw0 = 0; pw0 < ll.pw_padded; pw0 += 8) {
+        const int pw = pw0 + sub;
+        // (every lane takes part in the exchange: the lane asked may be one whose column does not exist)
+        const int wlow = __shfl(wlow_mine, pw & 63), wn_any = __shfl(wn_mine, pw & 63);
+        const int wn = pw < PW ? wn_any : 0;
+        // local cell of the window's first cell, and of w[0] once the window lies inside the tile
+        const int s0 = wlow - tx * tg.tw;
+        const int b = max(0, min(s0, tg.tw - kWindowCells));
+        const int cell = tx * tg.tw + b + slot;           // the cell this lane weighs
+        const int c = cell - wlow;                        // its place in the window
+        float w = 0.0f;
+        if (slot >= 0 && c >= 0 && c < wn && b + slot < tg.tw && cell < W)
+          w = merged_weight(g.start_w, pw, g.bin_w, g.grid_w, W, cell);
+        // The cells the tile owner reads and writes for this window (local): w[0..3] if one of
+        // them is not zero, w[4..6] likewise -- cells of weight zero among them included.
+        const unsigned live = static_cast<unsigned>(__ballot(w != 0.0f) >> (8 * sub)) & 0xffu;
+        const bool head = (live & 0x1eu) != 0, tail = (live & 0xe0u) != 0;
+        const int lo = head ? b : tail ? b + 4 : tg.tw;
+        const int hi = tail ? b + kWindowCells - 1 : head ? b + 3 : -1;
+        // smallest power-of-two distance at which no two windows of these eight columns share a cell
+        int lg = 0;
+#pragma unroll
+        for (int d = 1; d <= 4; d <<= 1) {
+          const int lo_d = __shfl_down(lo, 8 * d), hi_d = __shfl_down(hi, 8 * d);
+          const bool clash = sub + d < 8 && lo <= hi && lo_d <= hi_d && lo_d <= hi && lo <= hi_d;
+          if (__ballot(clash) != 0) lg = __builtin_ctz(d) + 1;
+        }
+        const int out = slot < 0 ? ((b + 1) | (lg << 16)) : __float_as_int(w);
+        cols[(static_cast<long long>(tx) * ll.col_stride + 2 * pw) * 4 + (lane & 7)] = out;
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) build_lists_kernel(ListsArgs a) {
+  if (a.window_offsets != nullptr) build_window_lists_body(blockIdx.x, a);
+  else build_lists_body(blockIdx.x, a);
+}
 
 
 // One wavefront's share of a tile: the (ROI, pooled row, weight) taps that land
@@ -293,7 +507,7 @@ struct alignas(16) WorkEntry {
   int ph;
   float wy;
   int flags;   // bit 0: continues the previous entry's item; bit 1: last entry of its item;
-               // bits 2..: the ROI whose dy the entry reads (the item itself, or the ROI it is a piece of)
+               // bits 2..: the ROI whose dy the entry reads (the item itself, or the ROI it is a window of)
 };
 struct WorkRange { int begin; int count; };
 
@@ -307,6 +521,8 @@ struct WorkRange { int begin; int count; };
 // sixteen lists comes from one bump-pointer allocation per tile (cursors[1]).
 // The order in which tiles take their space varies from run to run; what is
 // written into it does not.
+// WIN: the items are windows of merged weights (WindowRowTable) rather than sample lists.
+template <bool WIN>
 __global__ void __launch_bounds__(kTileRows * 64)
 build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict__ tile_rois,
                        const AxisUnit* __restrict__ lists, TileGrid tg, ListLayout ll,
@@ -356,14 +572,26 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
   __syncthreads();   // the list is complete and visible to the whole workgroup
 
   // ---- the work lists of the sixteen rows ----
-  auto table_of = [&](int roi) {
-    return reinterpret_cast<const RowTapTable*>(lists + static_cast<long long>(roi) * ll.roi_stride +
-                                                static_cast<long long>(ty) * ll.row_stride);
+  // taps of list item `roi` on this wavefront's tile row: where they start, how many
+  auto taps_of = [&](int roi, const RowTap** taps) {
+    const AxisUnit* const table = lists + static_cast<long long>(roi) * ll.roi_stride +
+                                  static_cast<long long>(ty) * ll.row_stride;
+    if (WIN) {
+      const WindowRowTable* const tb = reinterpret_cast<const WindowRowTable*>(table);
+      const unsigned idx = tb->index[row];
+      *taps = tb->taps + (idx & 0xffffu);
+      return static_cast<int>(idx >> 16);
+    }
+    const RowTapTable* const tb = reinterpret_cast<const RowTapTable*>(table);
+    const unsigned idx = tb->index[row];
+    *taps = tb->taps + (idx & 0xffu);
+    return static_cast<int>(idx >> 8);
   };
   int total = 0;
   for (int base = begin; base < end; base += 64) {
     int c = 0;
-    if (base + lane < end) c = table_of(tile_rois[base + lane])->index[row] >> 8;
+    const RowTap* unused;
+    if (base + lane < end) c = taps_of(tile_rois[base + lane], &unused);
     for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
     total += c;
   }
@@ -388,10 +616,7 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
     if (base + lane < end) {
       roi = tile_rois[base + lane];
       owner = boxes[roi].roi << 2;
-      const RowTapTable* tb = table_of(roi);
-      const unsigned idx = tb->index[row];
-      c = idx >> 8;
-      taps = tb->taps + (idx & 0xffu);
+      c = taps_of(roi, &taps);
     }
     int incl = c;
     for (int off = 1; off < 64; off <<= 1) {

@@ -17,7 +17,7 @@ struct TileGrid {
   long long total;   // per_image * num_images
 };
 
-// The tiles a list item (a ROI, or a piece of its sampling grid) touches: image
+// The tiles a list item (a ROI, or one window of its merged weights) touches: image
 // (-1: none), first | last << 16 tile row, first | last << 16 tile column; and
 // the ROI it belongs to.
 struct alignas(16) TileBox { int batch; int ty; int tx; int roi; };

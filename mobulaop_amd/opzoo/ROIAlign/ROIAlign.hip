@@ -312,23 +312,29 @@ DyLaunch dy_launch(const Problem& p) {
 template <typename T>
 bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_dyb,
                 hipStream_t stream, TilePlan* plan, const T* fuse_dy = nullptr) {
-  // List items: the ROIs, or for sampling grids of more than 2 x 2 points their
-  // 2 x 2 pieces.  An adaptive grid depends on the boxes, so the number of
-  // pieces has to come back from the device (one blocking copy).
-  const bool pieces = roialign::lists_in_pieces(p.S);
-  long long items = p.R;
-  if (p.S > roialign::kSearchedGrid) return false;   // (such grids are not cut up)
-  if (pieces && p.S > 2) items = static_cast<long long>(p.R) * ((p.S + 1) / 2) * ((p.S + 1) / 2);
-  if (pieces && p.S <= 0) {
-    int* const scratch = static_cast<int*>(mobula_hip::workspace(sizeof(int) * (p.R + 3)));
+  // List items: the ROIs, or for sampling grids of more than 2 x 2 points the
+  // windows of merged weights their bins are cut into.  How many depends on the
+  // boxes, so their number has to come back from the device (one blocking copy:
+  // not while the stream is being captured into a graph).
+  const bool windows = roialign::lists_in_windows(p.S);
+  long long items = p.R, window_entries = 0;
+  if (p.S > roialign::kSearchedGrid) return false;   // (fixed grids of that size are not merged)
+  if (windows) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      return false;
+    }
+    int* const scratch = static_cast<int*>(mobula_hip::workspace(sizeof(int) * (p.R + 4)));
     if (failed()) return false;
-    roialign::piece_offsets_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.PH, p.PW, p.S, scratch,
-                                                           scratch + p.R + 1);
-    int info[2] = {0, 1};
+    roialign::window_offsets_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, tw,
+                                                            scratch, scratch + p.R + 1);
+    int info[3] = {0, 1, 0};
     MOBULA_HIP_TRY(hipMemcpyAsync(info, scratch + p.R + 1, sizeof(info), hipMemcpyDeviceToHost, stream));
     MOBULA_HIP_TRY(hipStreamSynchronize(stream));
-    if (failed() || info[1] != 0) return false;   // a grid of more than 64 points per axis: not cut up
+    if (failed() || info[1] != 0) return false;   // an adaptive grid too large to merge
     items = info[0];
+    window_entries = info[2];
   }
   if (items > (1ll << 22)) return false;
   roialign::TileGrid& g = plan->grid;
@@ -348,10 +354,11 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256) + 256;  // blocks are read whole
   const int cblk = (p.C + 31) / 32;
   // dyb: one slab per channel block (all ROIs), 256-byte aligned
-  const size_t b_slab = with_dyb ? align_up(sizeof(float) * 32 * plan->layout.col_stride * p.R * p.PH, 256) : 0;
+  const size_t b_slab = with_dyb ? align_up(sizeof(float) * 32 * plan->layout.pw_padded * p.R * p.PH, 256) : 0;
   const size_t b_dyt = b_slab * cblk;
   // work lists: every tap of every ROI once per tile column it spans
-  const long long n_entries = items * 2 * p.PH * (p.S == 1 ? 1 : 2) * g.tx +
+  // (windows: the bound that came back with their number)
+  const long long n_entries = (windows ? window_entries : items * 2 * p.PH * (p.S == 1 ? 1 : 2) * g.tx) +
                               11 * roialign::kTileRows * g.total;
   if (n_entries > (1ll << 27)) return false;
   // the consumer addresses both with 32-bit byte offsets
@@ -359,7 +366,7 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   plan->dyb_bytes = b_slab; plan->list_bytes = b_units;
   const size_t b_ranges = align_up(sizeof(roialign::WorkRange) * g.total * roialign::kTileRows, 256);
   const size_t b_entries = align_up(sizeof(roialign::WorkEntry) * n_entries, 256) + 512;
-  const size_t b_offsets = pieces ? align_up(sizeof(int) * (p.R + 3), 256) : 0;
+  const size_t b_offsets = windows ? align_up(sizeof(int) * (p.R + 4), 256) : 0;
   char* base = static_cast<char*>(mobula_hip::workspace(b_recs + b_cnt + b_list + b_units + b_dyt +
                                                         b_ranges + b_entries + b_offsets + 256));
   if (failed()) return false;
@@ -375,10 +382,10 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   plan->entries = reinterpret_cast<roialign::WorkEntry*>(cur);
   cur += b_entries;
   int* offsets = nullptr;
-  if (pieces) {   // (again, for an adaptive grid: the buffer of the first pass may have moved)
+  if (windows) {   // (again: the buffer of the first pass may have moved)
     offsets = reinterpret_cast<int*>(cur);
-    roialign::piece_offsets_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.PH, p.PW, p.S, offsets,
-                                                           offsets + p.R + 1);
+    roialign::window_offsets_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, tw,
+                                                            offsets, offsets + p.R + 1);
   }
   // two kernels: per-item tables (which also resets the bump pointers), then per-tile lists
   const int n_items = static_cast<int>(items);
@@ -388,14 +395,15 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   const DyLaunch dl = dy_launch<T>(p);
   if (fuse_dy != nullptr && with_dyb && dl.per > 0 && dl.blocks > 0 && dl.blocks + list_blocks < (1ll << 31)) {
     roialign::lists_and_dy_kernel<T><<<static_cast<unsigned>(dl.blocks + list_blocks), 256, dl.lds, stream>>>(
-        la, static_cast<unsigned>(list_blocks), fuse_dy, plan->dyb, plan->layout.col_stride, cblk, dl.per, p.C);
+        la, static_cast<unsigned>(list_blocks), fuse_dy, plan->dyb, plan->layout.pw_padded, cblk, dl.per, p.C);
     plan->dy_transposed = true;
   } else {
     roialign::build_lists_kernel<<<static_cast<unsigned>(list_blocks), 256, 0, stream>>>(la);
   }
-  roialign::build_tile_work_kernel<<<static_cast<unsigned>(g.total), roialign::kTileRows * 64, 0, stream>>>(
-      plan->boxes, n_items, plan->tile_rois, plan->lists, g, plan->layout, plan->cursors, plan->ranges,
-      plan->entries);
+  (windows ? roialign::build_tile_work_kernel<true> : roialign::build_tile_work_kernel<false>)
+      <<<static_cast<unsigned>(g.total), roialign::kTileRows * 64, 0, stream>>>(
+          plan->boxes, n_items, plan->tile_rois, plan->lists, g, plan->layout, plan->cursors, plan->ranges,
+          plan->entries);
   MOBULA_HIP_TRY(hipGetLastError());
   return !failed();
 }
@@ -420,10 +428,29 @@ int row_split(const Problem& p) {
   return roialign::backward_row_split(p.N, p.H, p.W, (p.C + BB::CB - 1) / BB::CB);
 }
 
-// Fixed sampling grids only: whether an adaptive one fits the tiled backward
-// depends on the boxes, and this path has no other kernel to fall back on.
+// The tile owner for a problem: tile columns tw, nsplit wavefronts per tile row (lists of
+// merged windows are not split), sample lists or windows.
+template <bool NHWC, typename T>
+auto owner_kernel(int tw, int* nsplit, bool windows) {
+  using BB = roialign::BwdBlocked;
+  const bool wide = tw == BB::TW;
+  if (windows) {
+    *nsplit = 1;
+    return wide ? roialign::backward_blocked_kernel<NHWC, T, BB::TW, 1, true>
+                : roialign::backward_blocked_kernel<NHWC, T, BB::TW_SMALL, 1, true>;
+  }
+  if (*nsplit > 1)
+    return wide ? roialign::backward_blocked_kernel<NHWC, T, BB::TW, BB::NSPLIT, false>
+                : roialign::backward_blocked_kernel<NHWC, T, BB::TW_SMALL, BB::NSPLIT, false>;
+  return wide ? roialign::backward_blocked_kernel<NHWC, T, BB::TW, 1, false>
+              : roialign::backward_blocked_kernel<NHWC, T, BB::TW_SMALL, 1, false>;
+}
+
+// Any sampling grid the lists take: fixed ones up to kSearchedGrid points, adaptive ones
+// (whether an adaptive one is small enough to merge depends on the boxes; if not the call
+// fails: this path has no other kernel to fall back on).
 bool nhwc_backward_supported(const Problem& p) {
-  return roialign::backward_blocked_supports(p.PH, p.PW, p.S) && p.S >= 1 && p.S <= roialign::kSearchedGrid &&
+  return roialign::backward_blocked_supports(p.PH, p.PW, p.S) && p.S <= roialign::kSearchedGrid &&
          p.C % 4 == 0 &&
          static_cast<long long>(p.R) * p.PH * p.PW * p.C * 4 < (1ll << 31);
 }
@@ -450,11 +477,8 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     }
     const unsigned dy_bytes = static_cast<unsigned>(sizeof(T) * p.n_out);
     mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-    const int nsplit = row_split(p);
-    const auto kernel = nsplit > 1 ? (tw == BB::TW ? roialign::backward_blocked_kernel<true, T, BB::TW, BB::NSPLIT>
-                                                   : roialign::backward_blocked_kernel<true, T, BB::TW_SMALL, BB::NSPLIT>)
-                                   : (tw == BB::TW ? roialign::backward_blocked_kernel<true, T, BB::TW>
-                                                   : roialign::backward_blocked_kernel<true, T, BB::TW_SMALL>);
+    int nsplit = row_split(p);
+    const auto kernel = owner_kernel<true, T>(tw, &nsplit, plan.layout.windows != 0);
     kernel<<<static_cast<unsigned>(roialign::backward_blocked_grid(plan.grid.total, cblk)), BB::NT * nsplit, 0, stream>>>(
         dy, dx, plan.ranges, plan.entries, plan.lists,
         plan.grid, plan.layout, p.C, p.H, p.W, p.PH, p.PW, cblk, dy_bytes,
@@ -485,21 +509,18 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
     const DyLaunch dl = dy_launch<T>(p);
     if (grid < (1ll << 31) && dl.blocks < (1ll << 31) && (dl.per > 0 || dl.cap >= 4)) {
-      const int pwp = plan.layout.col_stride;
+      const int pwp = plan.layout.pw_padded;
       if (p.R > 0 && !plan.dy_transposed)
         roialign::transpose_dy_blocked_kernel<T><<<static_cast<unsigned>(dl.blocks), 256, dl.lds, side.get()>>>(
             dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dl.per, p.R, dl.cap);
       side.join();
       {
         mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
-        const int nsplit = row_split(p);
+        int nsplit = row_split(p);
         // every row piece of dx starts at a multiple of four elements (tile widths are): four columns per store
         const bool quads = p.W % 4 == 0 && reinterpret_cast<size_t>(dx) % (4 * sizeof(T)) == 0 &&
                            mobula_hip::option("roialign_row_quads", 1) != 0;
-        const auto kernel = nsplit > 1 ? (tw == BB::TW ? roialign::backward_blocked_kernel<false, T, BB::TW, BB::NSPLIT>
-                                                       : roialign::backward_blocked_kernel<false, T, BB::TW_SMALL, BB::NSPLIT>)
-                                       : (tw == BB::TW ? roialign::backward_blocked_kernel<false, T, BB::TW>
-                                                       : roialign::backward_blocked_kernel<false, T, BB::TW_SMALL>);
+        const auto kernel = owner_kernel<false, T>(tw, &nsplit, plan.layout.windows != 0);
         kernel<<<static_cast<unsigned>(grid), BB::NT * nsplit, 0, stream>>>(
             plan.dyb, dx, plan.ranges, plan.entries, plan.lists, plan.grid, plan.layout, p.C, p.H,
             p.W, p.PH, p.PW, cblk, static_cast<unsigned>(plan.dyb_bytes),

@@ -79,11 +79,22 @@ class ROIAlign:
                                                         rois.shape[0])):
             import torch
             dy_cl = dy.contiguous(memory_format=torch.channels_last)
-            mobula.func.roi_align_backward_nhwc_assign(_numel(dy), _nhwc(dy_cl), *geometry, int(data.shape[0]),
-                                                       _nhwc(dx), rois)
-            if self.req[1] not in (req.null, req.add):
-                self.dX[1][:] = 0
-            return
+            try:
+                mobula.func.roi_align_backward_nhwc_assign(_numel(dy), _nhwc(dy_cl), *geometry, int(data.shape[0]),
+                                                           _nhwc(dx), rois)
+                taken = True
+            except RuntimeError:
+                # Sampling grids other than 1 or 2 points are merged into lists whose size
+                # depends on the boxes: an adaptive grid of more than 2^15 points per bin, or
+                # a stream that is being captured (the size comes back through a blocking
+                # copy), is refused there.  The NCHW entry point below takes every grid.
+                if self.sampling_ratio in (1, 2):
+                    raise
+                taken = False
+            if taken:
+                if self.req[1] not in (req.null, req.add):
+                    self.dX[1][:] = 0
+                return
         fused = getattr(mobula.func, 'roi_align_backward_assign', None)
         if self.req[0] != req.add and fused is not None:
             fused(_numel(dy), dy, *geometry, int(data.shape[0]), self.dX[0], rois)

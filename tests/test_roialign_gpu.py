@@ -351,9 +351,10 @@ def test_tiled_backward_beyond_two_gib_of_blocked_gradient():
 @pytest.mark.parametrize('columns', [56, 28])
 @pytest.mark.parametrize('S', [0, 3, 4, 5, 7, 65])
 def test_tiled_backward_with_larger_sampling_grids(S, columns):
-    """Sampling grids other than 1 or 2 points per bin are cut into 2 x 2 pieces
-    for the tiled backward (odd grids leave half-filled pieces; S = 0 gives every
-    ROI its own grid; 65 is beyond what is cut up and takes the plain kernel).
+    """Sampling grids other than 1 or 2 points per bin are merged for the tiled
+    backward: one weight per row and per column a bin touches, the columns in
+    windows of seven cells (S = 0 gives every ROI its own grid; a fixed grid of
+    65 points is beyond what is merged and takes the plain kernel).
     Boxes: tiny, ordinary, wider than the map, partly off the map."""
     abi.set_impl('tiled')
     native.set_option('roialign_tile_columns', columns)
@@ -464,10 +465,13 @@ def test_channels_last_rejects_what_it_does_not_take():
     dy = torch.zeros(1, 7, 33, 8, device='cuda')         # 33 pooled columns: more than the backward's lists hold
     with pytest.raises(RuntimeError, match='channels-last'):
         abi.backward_nhwc(dy, rois, (1, 8, 8, 8), 1.0, 2)
-    dy = torch.zeros(1, 2, 2, 8, device='cuda')          # adaptive grid: whether it fits depends on the boxes
-    assert not native.roialign_channels_last_supported(True, 4, 8, 8, 8, (2, 2), 0, 1)
+    dy = torch.zeros(1, 2, 2, 8, device='cuda')          # a fixed grid of more than 64 points per bin and axis
+    assert not native.roialign_channels_last_supported(True, 4, 8, 8, 8, (2, 2), 65, 1)
     with pytest.raises(RuntimeError, match='channels-last'):
-        abi.backward_nhwc(dy, rois, (1, 8, 8, 8), 1.0, 0)
+        abi.backward_nhwc(dy, rois, (1, 8, 8, 8), 1.0, 65)
+    # an adaptive grid is taken (its bins' weights are merged)
+    assert native.roialign_channels_last_supported(True, 4, 8, 8, 8, (2, 2), 0, 1)
+    assert abi.backward_nhwc(dy, rois, (1, 8, 8, 8), 1.0, 0, assign=True).abs().sum().item() == 0.0
     # the library is usable afterwards
     assert abi.forward_nhwc(torch.zeros(1, 8, 8, 8, device='cuda'), rois, (2, 2), 1.0, 2).shape == (1, 2, 2, 8)
 
