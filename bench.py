@@ -38,6 +38,18 @@ def kernel_source_digest():
     return h.hexdigest()[:16]
 
 
+def conv_source_digest():
+    """Digest of the Conv2D kernel sources, named by profiles/conv2d_cfg5_mfma.txt the same way."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    files = sorted(glob.glob(os.path.join(ROOT, 'mobulaop_amd', 'csrc', 'conv_*.h')) +
+                   [os.path.join(ROOT, 'mobulaop_amd', 'opzoo', 'Convolution', 'Convolution.hip')])
+    for f in files:
+        h.update(open(f, 'rb').read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(path, kernel):
     """HBM bytes per launch of `kernel` from a summary under profiles/ (two rocprofv3 --pmc
     runs of this script, FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
@@ -121,7 +133,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 
 
-def short_roialign_run(name, steps=5, warmup=2, nhwc=False):
+def short_roialign_run(name, steps=20, warmup=3, nhwc=False):
     """One of the other BASELINE configurations (nhwc: on channels-last tensors through the
     channels-last entry points), a few steps through the C ABI: ms per
     step, fraction of the HBM peak on the algorithmic bytes, and the largest difference
@@ -144,7 +156,7 @@ def short_roialign_run(name, steps=5, warmup=2, nhwc=False):
     stream = torch.cuda.current_stream().cuda_stream
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
     fwd_ms = bwd_ms = 0.0
-    for k in range(warmup + steps):
+    for k in range(warmup + steps):   # the passes, one step at a time
         ev[0].record()
         run_forward(x, rois, pooled, scale, S, stream=stream)
         ev[1].record()
@@ -155,9 +167,17 @@ def short_roialign_run(name, steps=5, warmup=2, nhwc=False):
         if k >= warmup:
             fwd_ms += ev[0].elapsed_time(ev[1]) / steps
             bwd_ms += ev[1].elapsed_time(ev[2]) / steps
+    # the step as the bench line's own workload is timed: `steps` of them back to back
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run_forward(x, rois, pooled, scale, S, stream=stream)
+        if has_bwd:
+            run_backward(dy, rois, x.shape, scale, S, dx=dx, assign=True, stream=stream)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
     b_fwd, b_bwd = workloads.algorithmic_bytes(w)
     nbytes = b_fwd + (b_bwd if has_bwd else 0)
-    ms = fwd_ms + bwd_ms
     n = min(32, rois.shape[0])
     part = rois[:n].contiguous()
 

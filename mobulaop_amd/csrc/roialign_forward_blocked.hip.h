@@ -441,22 +441,38 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
     }
     if (NHWC) continue;
     // the wavefront's outputs of this pass leave LDS in the order of y
-    const int total = nch * seg;
+    // (the lane number through an empty asm: the addresses below are then formed here, not
+    // ahead of the gather, where they would take registers the gather needs)
+    int lane_now = lane;
+    asm volatile("" : "+v"(lane_now));
     if (rp == PH) {
+      const int total = nch * seg;
       T* const dst = y + (static_cast<size_t>(roi) * C + c0) * bins;
       constexpr int per = 16 / sizeof(T);
       if (reinterpret_cast<size_t>(dst) % 16 == 0) {
         const int nvec = total / per;
-        for (int i = lane; i < nvec; i += 64)
+        for (int i = lane_now; i < nvec; i += 64)
           __builtin_nontemporal_store(reinterpret_cast<const u32x4*>(stage)[i], reinterpret_cast<u32x4*>(dst) + i);
-        for (int i = nvec * per + lane; i < total; i += 64) dst[i] = stage[i];
+        for (int i = nvec * per + lane_now; i < total; i += 64) dst[i] = stage[i];
       } else {
-        for (int i = lane; i < total; i += 64) dst[i] = stage[i];
+        for (int i = lane_now; i < total; i += 64) dst[i] = stage[i];
       }
     } else {
-      for (int i = lane; i < total; i += 64) {
-        const int c = i / seg, j = i - c * seg;
-        y[(static_cast<size_t>(roi) * C + c0 + c) * bins + ph0 * PW + j] = stage[i];
+      // some pooled rows of every channel: seg contiguous elements per channel, the lanes cover
+      // as many channels at a time as fit (one division per pass, none per element)
+      const int chans = max(1, 64 / seg), cl = lane_now / seg, j0 = lane_now - cl * seg;
+      if (seg <= 64) {
+        if (cl < chans) {
+          // (the same base for every lane: scalar registers; 32-bit offsets per lane)
+          T* const base = y + (static_cast<size_t>(roi) * C + c0) * bins + ph0 * PW;
+          int to = cl * bins + j0, from = cl * seg + j0;
+#pragma nounroll
+          for (int c = cl; c < nch; c += chans, to += chans * bins, from += chans * seg) base[to] = stage[from];
+        }
+      } else {
+        for (int c = 0; c < nch; ++c)
+          for (int j = lane_now; j < seg; j += 64)
+            y[(static_cast<size_t>(roi) * C + c0 + c) * bins + ph0 * PW + j] = stage[c * seg + j];
       }
     }
   }

@@ -262,8 +262,8 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
     }
     if (NHWC) continue;
     // the wavefront's outputs of this pass leave LDS in the order of y
-    const int total = nch * seg;
     if (rp == PH) {
+      const int total = nch * seg;
       T* const dst = y + (static_cast<size_t>(roi) * C + c0) * bins;
       constexpr int per = 16 / sizeof(T);
       if (reinterpret_cast<size_t>(dst) % 16 == 0) {
@@ -275,9 +275,21 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
         for (int i = lane; i < total; i += 64) dst[i] = stage[i];
       }
     } else {
-      for (int i = lane; i < total; i += 64) {
-        const int c = i / seg, j = i - c * seg;
-        y[(static_cast<size_t>(roi) * C + c0 + c) * bins + ph0 * PW + j] = stage[i];
+      // some pooled rows of every channel: seg contiguous elements per channel, the lanes cover
+      // as many channels at a time as fit (one division per pass, none per element)
+      const int chans = max(1, 64 / seg), cl = lane / seg, j0 = lane - cl * seg;
+      if (seg <= 64) {
+        if (cl < chans) {
+          // (the same base for every lane: scalar registers; 32-bit offsets per lane)
+          T* const base = y + (static_cast<size_t>(roi) * C + c0) * bins + ph0 * PW;
+          int to = cl * bins + j0, from = cl * seg + j0;
+#pragma nounroll
+          for (int c = cl; c < nch; c += chans, to += chans * bins, from += chans * seg) base[to] = stage[from];
+        }
+      } else {
+        for (int c = 0; c < nch; ++c)
+          for (int j = lane; j < seg; j += 64)
+            y[(static_cast<size_t>(roi) * C + c0 + c) * bins + ph0 * PW + j] = stage[c * seg + j];
       }
     }
   }

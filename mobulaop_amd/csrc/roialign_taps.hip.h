@@ -170,55 +170,66 @@ __device__ __forceinline__ WindowCount count_windows(const RoiGeom& g, int PH, i
   return c;
 }
 
-// offsets[r] = number of the first window item of ROI r, offsets[R] = their total;
-// info[0] = the total, info[1] = 1 if some ROI's grid has more than kMergedGrid
-// points along an axis (the caller then takes another path), info[2] = an upper
-// bound of the work entries of all items (saturating at 2^30).
-// One workgroup of 1024 threads.
+// Window items, step 1: counts[r] = windows of ROI r (-1: its grid has more than kMergedGrid
+// points along an axis), work[r] = an upper bound of the work entries of its items.
+__global__ void __launch_bounds__(256)
+window_counts_kernel(const float* __restrict__ rois, int R, float scale, int PH, int PW, int S, int H, int W,
+                     int tw, int* __restrict__ counts, long long* __restrict__ work) {
+  for (long long r = blockIdx.x * 256ll + threadIdx.x; r < R; r += 256ll * gridDim.x) {
+    const RoiGeom g = roi_geometry(rois + r * 5, scale, PH, PW, S);
+    if (g.grid_h > kMergedGrid || g.grid_w > kMergedGrid || g.grid_h < 1 || g.grid_w < 1) {
+      counts[r] = -1;
+      work[r] = 0;
+      continue;
+    }
+    const WindowCount c = count_windows(g, PH, PW, H, W, tw);
+    counts[r] = c.windows;
+    work[r] = static_cast<long long>(c.windows) * c.tiles_x * c.taps;
+  }
+}
+
+// Step 2: offsets[r] = number of the first window item of ROI r, offsets[R] = their total
+// (offsets may be the array of counts: every thread reads its share before any writes);
+// info[0] = the total, info[1] = 1 if some ROI's grid is too large to merge (the caller
+// then takes another path), info[2] = an upper bound of the work entries of all items
+// (saturating at 2^30).  One workgroup of 1024 threads.
 __global__ void __launch_bounds__(1024)
-window_offsets_kernel(const float* __restrict__ rois, int R, float scale, int PH, int PW, int S, int H, int W,
-                      int tw, int* __restrict__ offsets, int* __restrict__ info) {
+window_offsets_kernel(const int* __restrict__ counts, const long long* __restrict__ work, int R,
+                      int* __restrict__ offsets, int* __restrict__ info) {
   __shared__ int part[1024];
-  __shared__ long long work[1024];
+  __shared__ long long entries[1024];
   __shared__ int too_big;
   const int t = threadIdx.x, share = (R + 1023) / 1024;
   const int first = min(R, t * share), last = min(R, first + share);
   if (t == 0) too_big = 0;
   __syncthreads();
-  auto count_of = [&](int r) {
-    const RoiGeom g = roi_geometry(rois + static_cast<long long>(r) * 5, scale, PH, PW, S);
-    if (g.grid_h > kMergedGrid || g.grid_w > kMergedGrid || g.grid_h < 1 || g.grid_w < 1) {
-      too_big = 1;
-      return WindowCount{0, 0, 0};
-    }
-    return count_windows(g, PH, PW, H, W, tw);
-  };
   int sum = 0;
-  long long entries = 0;
+  long long all = 0;
   for (int r = first; r < last; ++r) {
-    const WindowCount c = count_of(r);
-    sum += c.windows;
-    entries += static_cast<long long>(c.windows) * c.tiles_x * c.taps;
+    const int c = counts[r];
+    if (c < 0) too_big = 1;
+    sum += max(c, 0);
+    all += work[r];
   }
   part[t] = sum;
-  work[t] = entries;
+  entries[t] = all;
   __syncthreads();
   if (t == 0) {   // exclusive prefix over the threads
     int run = 0;
-    long long all = 0;
-    for (int i = 0; i < 1024; ++i) { const int c = part[i]; part[i] = run; run += c; all += work[i]; }
+    long long total = 0;
+    for (int i = 0; i < 1024; ++i) { const int c = part[i]; part[i] = run; run += c; total += entries[i]; }
     offsets[R] = run;
     info[0] = run;
-    info[2] = static_cast<int>(min(all, 1ll << 30));
+    info[1] = too_big;
+    info[2] = static_cast<int>(min(total, 1ll << 30));
   }
   __syncthreads();
   int at = part[t];
   for (int r = first; r < last; ++r) {
+    const int c = max(counts[r], 0);
     offsets[r] = at;
-    at += count_of(r).windows;
+    at += c;
   }
-  __syncthreads();
-  if (t == 0) info[1] = too_big;
 }
 
 __device__ __forceinline__ AxisUnit clip_unit(int bin, const AxisSample& a, int t0, int tsize,

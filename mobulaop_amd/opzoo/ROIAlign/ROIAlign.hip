@@ -318,6 +318,19 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   // not while the stream is being captured into a graph).
   const bool windows = roialign::lists_in_windows(p.S);
   long long items = p.R, window_entries = 0;
+  // the head of the workspace: offsets[R + 1], info[3], counts[R], work[R] (see window_offsets_kernel)
+  const size_t b_offsets = windows ? align_up(sizeof(int) * (p.R + 4) + sizeof(int) * p.R + 8, 256) +
+                                         align_up(sizeof(long long) * p.R, 256) : 0;
+  char* head = nullptr;
+  auto number_windows = [&](char* at) {
+    int* const offsets = reinterpret_cast<int*>(at);
+    int* const counts = offsets + p.R + 4;
+    long long* const work = reinterpret_cast<long long*>(at + align_up(sizeof(int) * (2 * p.R + 4) + 8, 256));
+    if (p.R > 0)
+      roialign::window_counts_kernel<<<grid_for(p.R, 256), 256, 0, stream>>>(rois, p.R, p.scale, p.PH, p.PW, p.S, p.H,
+                                                                            p.W, tw, counts, work);
+    roialign::window_offsets_kernel<<<1, 1024, 0, stream>>>(counts, work, p.R, offsets, offsets + p.R + 1);
+  };
   if (p.S > roialign::kSearchedGrid) return false;   // (fixed grids of that size are not merged)
   if (windows) {
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -325,12 +338,12 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
       (void)hipGetLastError();
       return false;
     }
-    int* const scratch = static_cast<int*>(mobula_hip::workspace(sizeof(int) * (p.R + 4)));
+    head = static_cast<char*>(mobula_hip::workspace(b_offsets));
     if (failed()) return false;
-    roialign::window_offsets_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, tw,
-                                                            scratch, scratch + p.R + 1);
+    number_windows(head);
     int info[3] = {0, 1, 0};
-    MOBULA_HIP_TRY(hipMemcpyAsync(info, scratch + p.R + 1, sizeof(info), hipMemcpyDeviceToHost, stream));
+    MOBULA_HIP_TRY(hipMemcpyAsync(info, reinterpret_cast<int*>(head) + p.R + 1, sizeof(info), hipMemcpyDeviceToHost,
+                                  stream));
     MOBULA_HIP_TRY(hipStreamSynchronize(stream));
     if (failed() || info[1] != 0) return false;   // an adaptive grid too large to merge
     items = info[0];
@@ -366,10 +379,15 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   plan->dyb_bytes = b_slab; plan->list_bytes = b_units;
   const size_t b_ranges = align_up(sizeof(roialign::WorkRange) * g.total * roialign::kTileRows, 256);
   const size_t b_entries = align_up(sizeof(roialign::WorkEntry) * n_entries, 256) + 512;
-  const size_t b_offsets = windows ? align_up(sizeof(int) * (p.R + 4), 256) : 0;
-  char* base = static_cast<char*>(mobula_hip::workspace(b_recs + b_cnt + b_list + b_units + b_dyt +
-                                                        b_ranges + b_entries + b_offsets + 256));
+  char* base = static_cast<char*>(mobula_hip::workspace(b_offsets + b_recs + b_cnt + b_list + b_units + b_dyt +
+                                                        b_ranges + b_entries + 256));
   if (failed()) return false;
+  int* offsets = nullptr;
+  if (windows) {
+    if (base != head) number_windows(base);   // the workspace has grown: it is another buffer now
+    offsets = reinterpret_cast<int*>(base);
+    base += b_offsets;
+  }
   plan->boxes = reinterpret_cast<roialign::TileBox*>(base);
   plan->cursors = reinterpret_cast<int*>(base + b_recs);
   plan->tile_rois = reinterpret_cast<int*>(base + b_recs + b_cnt);
@@ -381,12 +399,6 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   cur += b_ranges;
   plan->entries = reinterpret_cast<roialign::WorkEntry*>(cur);
   cur += b_entries;
-  int* offsets = nullptr;
-  if (windows) {   // (again: the buffer of the first pass may have moved)
-    offsets = reinterpret_cast<int*>(cur);
-    roialign::window_offsets_kernel<<<1, 1024, 0, stream>>>(rois, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, tw,
-                                                            offsets, offsets + p.R + 1);
-  }
   // two kernels: per-item tables (which also resets the bump pointers), then per-tile lists
   const int n_items = static_cast<int>(items);
   const roialign::ListsArgs la{rois, n_items, p.R, p.scale, p.PH, p.PW, p.S, p.H, p.W, p.N, g, plan->layout,

@@ -9,6 +9,7 @@ sys.path.insert(0, ROOT)
 import bench   # noqa: E402
 
 TRAFFIC = os.path.join(ROOT, 'profiles', 'roialign_cfg2_hbm_traffic.txt')
+CONV = os.path.join(ROOT, 'profiles', 'conv2d_cfg5_mfma.txt')
 
 
 def test_traffic_summary_names_the_kernel_sources_of_this_tree():
@@ -16,6 +17,12 @@ def test_traffic_summary_names_the_kernel_sources_of_this_tree():
     assert 'kernel sources: ' + bench.kernel_source_digest() in text, (
         'profiles/roialign_cfg2_hbm_traffic.txt was measured on other kernel sources: collect the '
         'FETCH_SIZE / WRITE_SIZE runs again (the file says how)')
+
+
+def test_conv_summary_names_the_kernel_sources_of_this_tree():
+    assert 'kernel sources: ' + bench.conv_source_digest() in open(CONV).read(), (
+        'profiles/conv2d_cfg5_mfma.txt was measured on other Conv2D kernel sources: collect its runs again '
+        '(the file says how)')
 
 
 def test_traffic_is_read_from_the_summary():
