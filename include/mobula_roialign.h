@@ -163,9 +163,11 @@ void roi_align_backward_assign_86156afd(const int device_id, const int nthreads,
  * mobula_hip_roialign_nhwc_supported first and convert to NCHW otherwise.  Takes:
  * forward: channels a multiple of 4 (fp32) or 8 (16-bit types), pooled_width <= 50,
  * one image below 2 GiB; backward: fp32, fp16 or bfloat16, channels a multiple of
- * 4, a fixed sampling_ratio of 1 .. 64 (an adaptive grid, sampling_ratio <= 0, is
- * not taken: whether it fits depends on the boxes), pooled_width <= 32,
- * pooled_height * min(sampling_ratio, 2) <= 64, R * PH * PW * C * 4 below 2 GiB. */
+ * 4, sampling_ratio <= 64 (an adaptive grid, sampling_ratio <= 0, is taken; a call
+ * whose boxes give it more than 2^15 points per bin along an axis, or whose stream
+ * is being captured into a graph while sampling_ratio is not 1 or 2, fails with an
+ * error: the NCHW entry points take those), pooled_width <= 32, pooled_height <= 32,
+ * R * PH * PW * C * 4 below 2 GiB. */
 void roi_align_forward_nhwc_ab78de3c(const int device_id, const int nthreads, const float* bottom_data,
                                      const float spatial_scale, const int channels, const int height,
                                      const int width, const int pooled_height, const int pooled_width,
@@ -258,6 +260,10 @@ void conv2d_backward_data_ecf81c91(const int device_id, const int n, const float
                                    const int pad_h, const int pad_w, const int stride_h,
                                    const int stride_w, const int dilation_h, const int dilation_w,
                                    float* dx);
+/* (With the option "conv_compute" set to 1 and unit strides the weight gradient is formed from
+ * whole zero-padded planes: a non-finite value of x then also meets zeros of dy that belong to a
+ * neighbouring channel's or image's positions, and 0 x inf = NaN ends up in the gradient of that
+ * neighbouring channel's weights.  Modes 0 and 2 confine a non-finite x to its own channel.) */
 void conv2d_backward_weight_ecf81c91(const int device_id, const int n, const float* dy, const float* x,
                                      const int accumulate, const int batch, const int channels,
                                      const int height, const int width, const int filters,
@@ -289,10 +295,17 @@ void mobula_hip_clear_error(void);
  * lets helper kernels of a call run on a second stream of the device, 0 keeps
  * everything on the caller's stream; "conv_compute": 0 (default) multiplies the
  * convolution's fp32 operands as they are, 1 rounds them to bf16 and accumulates
- * in fp32 (results about 2e-3 off), 2 splits every operand into two bf16 and
- * forms three bf16 products per multiply-add (results about 5e-6 off);
+ * in fp32 (results about 2e-3 off; a non-finite value in x can make the weight
+ * gradient of a neighbouring channel NaN, see conv2d_backward_weight), 2 splits
+ * every operand into two bf16 and forms three bf16 products per multiply-add
+ * (results about 5e-6 off);
  * "roialign_tile_columns": 0 (default) lets the backward pass choose its tile
- * width from the size of the map, 56 or 28 fixes it).  set returns 0, or -1 for an unknown name; get
+ * width from the size of the map, 56 or 28 fixes it; "roialign_row_split": 0
+ * (default) lets it choose how many wavefronts share a tile row's work list,
+ * 1 or 4 fixes it; "roialign_row_quads": 1 (default) lets it write rows of maps
+ * whose width is a multiple of four 16 bytes at a time, 0 element by element --
+ * all three for tests, the results do not depend on them beyond the order of
+ * fp32 sums).  set returns 0, or -1 for an unknown name; get
  * returns -1 for a name never set. */
 int mobula_hip_set_option(const char* name, long long value);
 long long mobula_hip_get_option(const char* name);

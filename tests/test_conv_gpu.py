@@ -250,6 +250,8 @@ def _leave_nan_patterns_in_the_workspace():
     (3, 5, 9, 11, 7, (3, 3), (1, 1), (1, 1), (1, 1)),         # likewise, odd grid width (the scalar copy)
     (2, 20, 20, 20, 100, (3, 3), (1, 1), (1, 1), (1, 1)),     # 128-row tiles with channels not a multiple of 32
     (1, 6, 21, 20, 9, (1, 2), (0, 0), (1, 1), (1, 1)),        # an odd shift without padding
+    (1, 4, 70, 71, 6, (3, 3), (1, 1), (1, 1), (1, 1)),        # odd width: the scalar copy over planes of two spans
+    (1, 2, 3, 4100, 4, (3, 3), (1, 1), (1, 1), (1, 1)),       # grid rows longer than a span
 ])
 def test_bf16_mode_is_exact_on_bf16_valued_operands(case):
     # Mode 1 rounds both operands of every product to bf16 and accumulates in fp32: against
