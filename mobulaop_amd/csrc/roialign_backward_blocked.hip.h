@@ -16,8 +16,8 @@
 // Pooled columns whose cells may coincide are taken in separate turns (the
 // pre-pass stores the spacing at which they cannot).
 //
-// dy is read from a channel-blocked copy dyb[C/32][R][PH][PWp][32] (PWp = PW
-// rounded up to 8): one 16-byte load per lane fetches a pooled row (1 KB); the
+// dy is read from a channel-blocked copy dyb[C/32][R][PH][PW][32]: one 16-byte
+// load per lane fetches (eight pooled columns of) a pooled row, up to 1 KB; the
 // slab of a channel block is addressed with 32-bit offsets (up to 2 GiB each).
 #pragma once
 #include <type_traits>
@@ -59,8 +59,8 @@ inline int backward_row_split(long long images, int H, int W, int cblk) {
   return wide * kTileRows * cblk < 8192 ? BwdBlocked::NSPLIT : 1;
 }
 
-// dy[r][c][ph][pw] -> dyb[cb][r][ph][PWp][32] (R: number of ROIs), zero where pw >= PW or the channel
-// does not exist.  One workgroup per (ROI, group of `per` channel blocks):
+// dy[r][c][ph][pw] -> dyb[cb][r][ph][PWp][32] (R: number of ROIs; PWp >= PW: the pooled columns
+// of a row of the copy, PW as launched), zero where pw >= PW or the channel does not exist.  One workgroup per (ROI, group of `per` channel blocks):
 // the input words of the group are contiguous and so are its output words.
 // LDS holds the input as it is; the transposition happens in the reads.
 // T is the element type of dy (float or __half); dyb is fp32 either way.
@@ -256,7 +256,6 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
   const int rounds = n_entries / (2 * K::G);
   const int first_entry = NSPLIT == 1 ? 0 : part * rounds / NSPLIT * (2 * K::G);
   const int end_entry = NSPLIT == 1 ? n_entries : (part + 1) * rounds / NSPLIT * (2 * K::G);
-  const int PWp = ll.pw_padded;
   float* const cell0 = row + quad * 4;   // this lane's four channels of cell 0 (the left dummy)
 
   // dyb and the sample lists as raw buffers: a scalar byte offset per entry
@@ -264,7 +263,7 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
   typedef typename std::conditional<NHWC, TO, float>::type TI;   // element type of what dy_any points to
   constexpr unsigned E = sizeof(TI);
   const unsigned dy_pw = (NHWC ? C : K::CB) * E;
-  const unsigned dy_ph = static_cast<unsigned>(NHWC ? PW : PWp) * dy_pw;
+  const unsigned dy_ph = static_cast<unsigned>(PW) * dy_pw;
   const unsigned dy_roi = dy_ph * PH;
   const unsigned list_roi = static_cast<unsigned>(ll.roi_stride) * sizeof(AxisUnit);
   // (dyb_bytes: the bytes of one channel block's slab of dyb, or of the caller's whole dy)

@@ -17,6 +17,8 @@
 // on scheduling; they differ from the per-sample order of the reference by
 // rounding only.
 #pragma once
+#include <type_traits>
+
 #include "roialign_forward_blocked.hip.h"
 
 namespace roialign {
@@ -128,7 +130,7 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
   // A box far larger than the map (or infinite) has up to 2^31 sample points per
   // bin, nearly all outside the map: forward_large_grid_kernel does those boxes.
   if (gh > kSearchedGrid || gw > kSearchedGrid) return;
-  const float count = uni_f(g.count);
+  const float inv_count = 1.0f / uni_f(g.count);
   MergedEntry (*const rowm)[M::LCAP] = rowm_s[wave];
   MergedEntry (*const colm)[M::LCAP] = colm_s[wave];
   int* const rown = rown_s[wave];
@@ -197,53 +199,78 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
               need_cols(pwb, ixw);
               const int nc = bin_on ? coln[grp] : 0;
               const MergedEntry* const clist = colm[grp];
-#pragma nounroll
-              for (int r0 = 0; r0 < nr; r0 += 4) {
-                int roff[4];
-                float rw[4];
-                bool rlive[4];
+              // blocks of four map rows (scalar) x four or two map columns (per lane): the columns
+              // of a block are decoded once for all its rows; a last block of at most two columns
+              // is not padded to four
+              auto block = [&](const int (&roff)[4], const float (&rw)[4], const bool (&rlive)[4], const int (&coff)[4],
+                               const float (&cw)[4], auto width) {
+                constexpr int NC = decltype(width)::value;
+                typename LaneData<T>::type v[4][NC];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                  const MergedEntry e = rlist[min(r0 + k, nr - 1)];
-                  roff[k] = uni_i(e.off); rw[k] = uni_f(e.w);
-                  rlive[k] = r0 + k < nr;
-                }
-#pragma nounroll
-                for (int cc = 0; cc < col_max; cc += 4) {
-                  int coff[4];
-                  float cw[4];
+                for (int r = 0; r < 4; ++r)
+                  if (rlive[r]) {
 #pragma unroll
-                  for (int k = 0; k < 4; ++k) {
-                    const MergedEntry e = clist[min(cc + k, M::LCAP - 1)];
-                    const bool ok = cc + k < nc;
-                    coff[k] = ok ? e.off + lane_off : kDead;
-                    cw[k] = ok ? e.w : 0.0f;
+                    for (int c = 0; c < NC; ++c) v[r][c] = buffer_load_lane<T>(plane, coff[c], roff[r]);
                   }
-                  typename LaneData<T>::type v[4][4];
 #pragma unroll
-                  for (int r = 0; r < 4; ++r)
-                    if (rlive[r]) {
+                for (int r = 0; r < 4; ++r)
+                  if (rlive[r]) {
+                    if constexpr (CPL > NC) {
+                      // more channels than columns per lane: the weight of a pixel first, then one
+                      // multiply-add per pixel and channel
+                      float w[NC];
 #pragma unroll
-                      for (int c = 0; c < 4; ++c) v[r][c] = buffer_load_lane<T>(plane, coff[c], roff[r]);
-                    }
+                      for (int c = 0; c < NC; ++c) w[c] = rw[r] * cw[c];
 #pragma unroll
-                  for (int r = 0; r < 4; ++r)
-                    if (rlive[r]) {
+                      for (int i = 0; i < CPL; ++i) {
+#pragma unroll
+                        for (int c = 0; c < NC; ++c) acc[i] = fmaf(w[c], static_cast<float>(v[r][c][i]), acc[i]);
+                      }
+                    } else {
 #pragma unroll
                       for (int i = 0; i < CPL; ++i) {
                         float t = cw[0] * static_cast<float>(v[r][0][i]);
 #pragma unroll
-                        for (int c = 1; c < 4; ++c) t = fmaf(cw[c], static_cast<float>(v[r][c][i]), t);
+                        for (int c = 1; c < NC; ++c) t = fmaf(cw[c], static_cast<float>(v[r][c][i]), t);
                         acc[i] = fmaf(rw[r], t, acc[i]);
                       }
                     }
+                  }
+              };
+#pragma nounroll
+              for (int cc = 0; cc < col_max; cc += 4) {
+                int coff[4];
+                float cw[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                  const MergedEntry e = clist[min(cc + k, M::LCAP - 1)];
+                  const bool ok = cc + k < nc;
+                  coff[k] = ok ? e.off + lane_off : kDead;
+                  cw[k] = ok ? e.w : 0.0f;
+                }
+                const bool narrow = col_max - cc <= 2;   // (the same for every lane)
+#pragma nounroll
+                for (int r0 = 0; r0 < nr; r0 += 4) {
+                  int roff[4];
+                  float rw[4];
+                  bool rlive[4];
+#pragma unroll
+                  for (int k = 0; k < 4; ++k) {
+                    const MergedEntry e = rlist[min(r0 + k, nr - 1)];
+                    roff[k] = uni_i(e.off); rw[k] = uni_f(e.w);
+                    rlive[k] = r0 + k < nr;
+                  }
+                  if (narrow) block(roff, rw, rlive, coff, cw, std::integral_constant<int, 2>());
+                  else block(roff, rw, rlive, coff, cw, std::integral_constant<int, 4>());
                 }
               }
             }
           }
         }
+        // (the reference divides by the number of samples; multiplying by its reciprocal
+        // differs in the last bit only where that number is no power of two)
 #pragma unroll
-        for (int i = 0; i < CPL; ++i) acc[i] /= count;
+        for (int i = 0; i < CPL; ++i) acc[i] *= inv_count;
         if (NHWC) {
           // y[roi][ph][pw][C]: the lane's channels of its bin are 16 contiguous bytes
           if (bin_on) {

@@ -367,8 +367,9 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   const size_t b_units = align_up(sizeof(roialign::AxisUnit) * n_units, 256) + 256;  // blocks are read whole
   const int cblk = (p.C + 31) / 32;
   // dyb: one slab per channel block (all ROIs), 256-byte aligned
-  const size_t b_slab = with_dyb ? align_up(sizeof(float) * 32 * plan->layout.pw_padded * p.R * p.PH, 256) : 0;
-  const size_t b_dyt = b_slab * cblk;
+  // (a multiple of 128 bytes; the slabs follow each other as the transposition writes them)
+  const size_t b_slab = with_dyb ? sizeof(float) * 32 * p.PW * p.R * p.PH : 0;
+  const size_t b_dyt = align_up(b_slab * cblk, 256);
   // work lists: every tap of every ROI once per tile column it spans
   // (windows: the bound that came back with their number)
   const long long n_entries = (windows ? window_entries : items * 2 * p.PH * (p.S == 1 ? 1 : 2) * g.tx) +
@@ -407,7 +408,7 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   const DyLaunch dl = dy_launch<T>(p);
   if (fuse_dy != nullptr && with_dyb && dl.per > 0 && dl.blocks > 0 && dl.blocks + list_blocks < (1ll << 31)) {
     roialign::lists_and_dy_kernel<T><<<static_cast<unsigned>(dl.blocks + list_blocks), 256, dl.lds, stream>>>(
-        la, static_cast<unsigned>(list_blocks), fuse_dy, plan->dyb, plan->layout.pw_padded, cblk, dl.per, p.C);
+        la, static_cast<unsigned>(list_blocks), fuse_dy, plan->dyb, p.PW, cblk, dl.per, p.C);
     plan->dy_transposed = true;
   } else {
     roialign::build_lists_kernel<<<static_cast<unsigned>(list_blocks), 256, 0, stream>>>(la);
@@ -521,7 +522,7 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
     const DyLaunch dl = dy_launch<T>(p);
     if (grid < (1ll << 31) && dl.blocks < (1ll << 31) && (dl.per > 0 || dl.cap >= 4)) {
-      const int pwp = plan.layout.pw_padded;
+      const int pwp = p.PW;   // (the blocked copy's pooled rows are not padded)
       if (p.R > 0 && !plan.dy_transposed)
         roialign::transpose_dy_blocked_kernel<T><<<static_cast<unsigned>(dl.blocks), 256, dl.lds, side.get()>>>(
             dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dl.per, p.R, dl.cap);

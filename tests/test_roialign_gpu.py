@@ -319,11 +319,11 @@ def test_tiled_backward_with_large_pooled_sizes(pooled, S):
 
 
 def test_tiled_backward_beyond_two_gib_of_blocked_gradient():
-    """10000 ROIs x 256 channels x 14 x 14: the channel-blocked copy of dy holds 2.3 GB (every channel block
+    """11500 ROIs x 256 channels x 14 x 14: the channel-blocked copy of dy holds 2.3 GB (every channel block
     a slab of its own, addressed with 32-bit offsets).  Checked against the straightforward kernel on the
     same inputs and by the adjoint identity with the forward."""
     g = torch.Generator(device='cuda').manual_seed(77)
-    N, C, H, W, R, pooled, scale, S = 8, 256, 128, 128, 10000, (14, 14), 0.125, 2
+    N, C, H, W, R, pooled, scale, S = 8, 256, 128, 128, 11500, (14, 14), 0.125, 2
     size = torch.exp(torch.rand(R, 2, device='cuda', generator=g) * np.log(16.0) + np.log(32.0))
     centre = torch.rand(R, 2, device='cuda', generator=g) * 1024.0
     rois = torch.cat([torch.randint(0, N, (R, 1), device='cuda', generator=g).float(), centre - size / 2,
