@@ -533,6 +533,8 @@ struct WorkRange { int begin; int count; };
 // The order in which tiles take their space varies from run to run; what is
 // written into it does not.
 // WIN: the items are windows of merged weights (WindowRowTable) rather than sample lists.
+constexpr int kTileListCap = 4096;   // items of one tile that LDS holds (longer lists go through memory)
+
 template <bool WIN>
 __global__ void __launch_bounds__(kTileRows * 64)
 build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict__ tile_rois,
@@ -542,45 +544,56 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
   __shared__ int hits[kTileRows];
   __shared__ int row_total[kTileRows];
   __shared__ int list_base, tile_base;
+  // the tile's items and the ROIs whose dy they read (<< 2, as the entries hold them), in item
+  // order: in LDS, so that the wavefronts below need not wait for memory to see the list
+  __shared__ int item_s[kTileListCap];
+  __shared__ int owner_s[kTileListCap];
   const long long tile = blockIdx.x;
   const int lane = threadIdx.x & 63, row = threadIdx.x >> 6;
   const int image = static_cast<int>(tile / tg.per_image);
   const int t = static_cast<int>(tile % tg.per_image);
   const int ty = t / tg.tx, tx = t % tg.tx;
 
-  // ---- the tile's ROI list ----
+  // ---- the tile's item list ----
   const int share = ((R + kTileRows * 64 - 1) / (kTileRows * 64)) * 64;
   const int r_begin = row * share, r_end = min(R, r_begin + share);
-  auto hit_of = [&](int r) {
+  auto hit_of = [&](int r, int* owner) {
     if (r >= r_end) return false;
     const TileBox b = boxes[r];
+    *owner = b.roi << 2;
     return b.batch == image && ty >= (b.ty & 0xffff) && ty <= (b.ty >> 16) && tx >= (b.tx & 0xffff) &&
            tx <= (b.tx >> 16);
   };
-  int mine = 0;
-  for (int base = r_begin; base < r_end; base += 64) mine += __popcll(__ballot(hit_of(base + lane)));
+  int mine = 0, unused_owner = 0;
+  for (int base = r_begin; base < r_end; base += 64) mine += __popcll(__ballot(hit_of(base + lane, &unused_owner)));
   if (lane == 0) hits[row] = mine;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int sum = 0;
-    for (int r = 0; r < kTileRows; ++r) sum += hits[r];
-    list_base = sum > 0 ? atomicAdd(cursors, sum) : 0;
-  }
-  __syncthreads();
-  int written = list_base, count = 0;
+  int written = 0, count = 0;
   for (int r = 0; r < kTileRows; ++r) {
     if (r < row) written += hits[r];
     count += hits[r];
   }
-  const int begin = list_base, end = list_base + count;
+  const bool in_lds = count <= kTileListCap;   // (the same for the whole workgroup)
+  if (!in_lds) {
+    if (threadIdx.x == 0) list_base = atomicAdd(cursors, count);
+    __syncthreads();
+  }
+  int* const long_list = tile_rois + (in_lds ? 0 : list_base);
   for (int base = r_begin; base < r_end && mine > 0; base += 64) {
-    const bool hit = hit_of(base + lane);
+    int owner = 0;
+    const bool hit = hit_of(base + lane, &owner);
     const unsigned long long mask = __ballot(hit);
-    if (hit) tile_rois[written + __popcll(mask & ((1ull << lane) - 1ull))] = base + lane;
+    if (hit) {
+      const int at = written + __popcll(mask & ((1ull << lane) - 1ull));
+      if (in_lds) { item_s[at] = base + lane; owner_s[at] = owner; }
+      else long_list[at] = base + lane;
+    }
     written += __popcll(mask);
     mine -= __popcll(mask);
   }
   __syncthreads();   // the list is complete and visible to the whole workgroup
+  auto item_at = [&](int i) { return in_lds ? item_s[i] : long_list[i]; };
+  auto owner_at = [&](int i, int item) { return in_lds ? owner_s[i] : boxes[item].roi << 2; };
 
   // ---- the work lists of the sixteen rows ----
   // taps of list item `roi` on this wavefront's tile row: where they start, how many
@@ -598,11 +611,17 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
     *taps = tb->taps + (idx & 0xffu);
     return static_cast<int>(idx >> 8);
   };
-  int total = 0;
-  for (int base = begin; base < end; base += 64) {
-    int c = 0;
-    const RowTap* unused;
-    if (base + lane < end) c = taps_of(tile_rois[base + lane], &unused);
+  // (what the first 64 items gave is kept for the second walk: most tiles have no more)
+  int total = 0, first_c = 0, first_item = 0;
+  const RowTap* first_taps = nullptr;
+  for (int base = 0; base < count; base += 64) {
+    int c = 0, item = 0;
+    const RowTap* taps = nullptr;
+    if (base + lane < count) {
+      item = item_at(base + lane);
+      c = taps_of(item, &taps);
+    }
+    if (base == 0) { first_c = c; first_item = item; first_taps = taps; }
     for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
     total += c;
   }
@@ -621,28 +640,40 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
   int out = tile_base;
   for (int r = 0; r < row; ++r) out += row_total[r];
   if (lane == 0) ranges[tile * kTileRows + row] = WorkRange{out, padded};
-  for (int base = begin; base < end; base += 64) {
-    int c = 0, roi = 0, owner = 0;
-    const RowTap* taps = nullptr;
-    if (base + lane < end) {
-      roi = tile_rois[base + lane];
-      owner = boxes[roi].roi << 2;
-      c = taps_of(roi, &taps);
+  for (int base = 0; base < count; base += 64) {
+    int c = first_c, roi = first_item, owner = 0;
+    const RowTap* taps = first_taps;
+    if (base > 0) {
+      c = 0; roi = 0; taps = nullptr;
+      if (base + lane < count) {
+        roi = item_at(base + lane);
+        c = taps_of(roi, &taps);
+      }
     }
+    if (base + lane < count) owner = owner_at(base + lane, roi);
     int incl = c;
     for (int off = 1; off < 64; off <<= 1) {
       const int up = __shfl_up(incl, off);
       if (lane >= off) incl += up;
     }
     WorkEntry* dst = entries + out + incl - c;
-    for (int q = 0; q < c; ++q)
-      dst[q] = WorkEntry{roi, taps[q].ph, taps[q].wy, (q > 0 ? 1 : 0) | (q == c - 1 ? 2 : 0) | owner};
+    // (four taps at a time: their loads go out together instead of one after the other)
+    for (int q0 = 0; q0 < c; q0 += 4) {
+      RowTap four[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) four[k] = taps[min(q0 + k, c - 1)];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int q = q0 + k;
+        if (q < c) dst[q] = WorkEntry{roi, four[k].ph, four[k].wy, (q > 0 ? 1 : 0) | (q == c - 1 ? 2 : 0) | owner};
+      }
+    }
     out += __shfl(incl, 63);
   }
   // padding: taps of weight zero that continue the last ROI and never end it
   if (lane < reserved - total) {
-    const int item = tile_rois[end - 1];
-    entries[out + lane] = WorkEntry{item, 0, 0.0f, 1 | (boxes[item].roi << 2)};
+    const int item = item_at(count - 1);
+    entries[out + lane] = WorkEntry{item, 0, 0.0f, 1 | owner_at(count - 1, item)};
   }
 }
 

@@ -284,6 +284,29 @@ def test_four_column_write_out_with_odd_channel_counts(C):
                       'bwd accumulate, shift {}'.format(shift))
 
 
+@pytest.mark.parametrize('S', [2, 3])
+def test_more_boxes_in_one_tile_than_the_list_builder_keeps_on_chip(S):
+    """The pre-pass keeps a tile's list of boxes in LDS up to 4096 entries and in memory
+    beyond: 5000 boxes on a map of one tile (with S = 3: about two list items per box)."""
+    abi.set_impl('tiled')
+    rng = np.random.default_rng(90 + S)
+    N, C, H, W, PH, PW, scale, R = 1, 8, 16, 48, 2, 3, 1.0, 5000
+    x1 = rng.uniform(-2, W, R); y1 = rng.uniform(-2, H, R)
+    rois = np.stack([np.zeros(R), x1, y1, x1 + rng.uniform(0.5, 30, R), y1 + rng.uniform(0.5, 12, R)],
+                    1).astype(np.float32)
+    dy = rng.standard_normal((R, C, PH, PW)).astype(np.float32)
+    want = oracle.backward(dy, rois, (N, C, H, W), scale, S, impl='ordered')
+    d_dy, d_rois = abi.to_dev(dy), abi.to_dev(rois)
+    native.set_option('kernel_timing', 1)
+    try:
+        first = abi.backward(d_dy, d_rois, (N, C, H, W), scale, S, assign=True)
+        assert _last_bracketed_kernel() == 'backward_blocked_kernel'
+    finally:
+        native.set_option('kernel_timing', 0)
+    assert_parity(first.cpu().numpy(), want, BWD_TOL, 'bwd assign')
+    assert torch.equal(first, abi.backward(d_dy, d_rois, (N, C, H, W), scale, S, assign=True))
+
+
 def _last_bracketed_kernel():
     import ctypes
     lib = native.library()
