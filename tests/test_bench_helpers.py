@@ -19,6 +19,15 @@ def test_traffic_summary_names_the_kernel_sources_of_this_tree():
         'FETCH_SIZE / WRITE_SIZE runs again (the file says how)')
 
 
+def test_every_roialign_summary_names_the_kernel_sources_of_this_tree():
+    import glob
+    files = sorted(glob.glob(os.path.join(ROOT, 'profiles', 'roialign_*.txt')))
+    assert len(files) >= 5
+    for f in files:
+        assert 'kernel sources: ' + bench.kernel_source_digest() in open(f).read(), (
+            os.path.basename(f) + ' was measured on other kernel sources: run its command again')
+
+
 def test_conv_summary_names_the_kernel_sources_of_this_tree():
     assert 'kernel sources: ' + bench.conv_source_digest() in open(CONV).read(), (
         'profiles/conv2d_cfg5_mfma.txt was measured on other Conv2D kernel sources: collect its runs again '
