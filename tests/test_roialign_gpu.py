@@ -317,7 +317,8 @@ def _last_bracketed_kernel():
     return name.value.decode() if ms >= 0 and name.value else None
 
 
-@pytest.mark.parametrize('pooled,S', [((28, 28), 2), ((32, 20), 2), ((17, 32), 1), ((9, 30), 3)])
+@pytest.mark.parametrize('pooled,S', [((28, 28), 2), ((32, 20), 2), ((17, 32), 1), ((9, 30), 3), ((32, 32), 0),
+                                      ((28, 28), 4)])
 def test_tiled_backward_with_large_pooled_sizes(pooled, S):
     """Up to 64 sample rows and columns per ROI (32 x 32 bins of 2 x 2 points, mask heads pool 28 x 28)
     stay on the tile owners; every element against the oracle."""
