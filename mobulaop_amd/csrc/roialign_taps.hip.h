@@ -315,19 +315,32 @@ __device__ __forceinline__ void build_lists_body(unsigned block, const ListsArgs
     for (int ty = rec.row_lo / tg.th; ty <= rec.row_hi / tg.th; ++ty) {
       const AxisUnit u = clip_unit(ph, a, ty * tg.th, tg.th, inv_count);
       RowTapTable* const table = reinterpret_cast<RowTapTable*>(base + ty * ll.row_stride);
-      // each unit lands on up to two tile rows; order the taps by row, then by lane
+      // Each unit lands on up to two tile rows; the taps are ordered by row, and within a row
+      // the high parts (of the units whose low row is the row above) come before the low parts,
+      // each in lane order: sample order, since sample coordinates never decrease with the lane.
+      // That also makes the lanes of a row contiguous among the live ones, so a tap's place
+      // follows from counts alone: lane r < 16 holds the numbers of row r.
       const int row0 = u.w0 != 0.0f ? u.pos : -1, row1 = u.w1 != 0.0f ? u.pos + 1 : -1;
-      int start = 0;
+      const unsigned long long below = (1ull << lane) - 1ull;
+      const int before0 = __popcll(__ballot(row0 >= 0) & below), before1 = __popcll(__ballot(row1 >= 0) & below);
+      int n0 = 0, n1 = 0;   // low and high parts on row `lane`
+#pragma unroll
       for (int r = 0; r < kTileRows; ++r) {
-        const unsigned long long m0 = __ballot(row0 == r), m1 = __ballot(row1 == r);
-        const unsigned long long below = (1ull << lane) - 1ull;
-        // a unit's high row is the next unit's low row: high parts first keeps sample order
-        const int n1 = __popcll(m1), n0 = __popcll(m0);
-        if (row1 == r) table->taps[start + __popcll(m1 & below)] = RowTap{ph, u.w1};
-        if (row0 == r) table->taps[start + n1 + __popcll(m0 & below)] = RowTap{ph, u.w0};
-        if (lane == 0) table->index[r] = static_cast<unsigned short>(start | ((n0 + n1) << 8));
-        start += n0 + n1;
+        const int c0 = __popcll(__ballot(row0 == r)), c1 = __popcll(__ballot(row1 == r));
+        if (lane == r) { n0 = c0; n1 = c1; }
       }
+      int upto0 = n0, upto1 = n1;   // inclusive sums over the rows up to this lane's
+      for (int off = 1; off < kTileRows; off <<= 1) {
+        const int a0 = __shfl_up(upto0, off), a1 = __shfl_up(upto1, off);
+        if (lane >= off) { upto0 += a0; upto1 += a1; }
+      }
+      // row r starts at (low parts before r) + (high parts before r); its high parts come first
+      const int low_before = __shfl(upto0 - n0, max(row1, 0));    // low parts on rows above row1
+      const int high_upto = __shfl(upto1, max(row0, 0));          // high parts on rows up to and including row0
+      if (row1 >= 0) table->taps[low_before + before1] = RowTap{ph, u.w1};
+      if (row0 >= 0) table->taps[high_upto + before0] = RowTap{ph, u.w0};
+      if (lane < kTileRows)
+        table->index[lane] = static_cast<unsigned short>((upto0 - n0 + upto1 - n1) | ((n0 + n1) << 8));
     }
   }
   {
@@ -564,8 +577,22 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
     return b.batch == image && ty >= (b.ty & 0xffff) && ty <= (b.ty >> 16) && tx >= (b.tx & 0xffff) &&
            tx <= (b.tx >> 16);
   };
-  int mine = 0, unused_owner = 0;
-  for (int base = r_begin; base < r_end; base += 64) mine += __popcll(__ballot(hit_of(base + lane, &unused_owner)));
+  // (what the first kKept chunks of 64 boxes of the wavefront's share gave is kept for the second
+  // walk: with up to 4096 boxes in all that is every chunk, and the boxes are read once)
+  constexpr int kKept = 4;
+  bool kept_hit[kKept];
+  int kept_owner[kKept];
+  int mine = 0;
+#pragma unroll
+  for (int k = 0; k < kKept; ++k) {
+    kept_owner[k] = 0;
+    kept_hit[k] = hit_of(r_begin + 64 * k + lane, &kept_owner[k]);
+    mine += __popcll(__ballot(kept_hit[k]));
+  }
+  for (int base = r_begin + 64 * kKept; base < r_end; base += 64) {
+    int unused_owner = 0;
+    mine += __popcll(__ballot(hit_of(base + lane, &unused_owner)));
+  }
   if (lane == 0) hits[row] = mine;
   __syncthreads();
   int written = 0, count = 0;
@@ -579,9 +606,7 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
     __syncthreads();
   }
   int* const long_list = tile_rois + (in_lds ? 0 : list_base);
-  for (int base = r_begin; base < r_end && mine > 0; base += 64) {
-    int owner = 0;
-    const bool hit = hit_of(base + lane, &owner);
+  auto put = [&](int base, bool hit, int owner) {
     const unsigned long long mask = __ballot(hit);
     if (hit) {
       const int at = written + __popcll(mask & ((1ull << lane) - 1ull));
@@ -590,6 +615,14 @@ build_tile_work_kernel(const TileBox* __restrict__ boxes, int R, int* __restrict
     }
     written += __popcll(mask);
     mine -= __popcll(mask);
+  };
+#pragma unroll
+  for (int k = 0; k < kKept; ++k)
+    if (mine > 0) put(r_begin + 64 * k, kept_hit[k], kept_owner[k]);
+  for (int base = r_begin + 64 * kKept; base < r_end && mine > 0; base += 64) {
+    int owner = 0;
+    const bool hit = hit_of(base + lane, &owner);
+    put(base, hit, owner);
   }
   __syncthreads();   // the list is complete and visible to the whole workgroup
   auto item_at = [&](int i) { return in_lds ? item_s[i] : long_list[i]; };
