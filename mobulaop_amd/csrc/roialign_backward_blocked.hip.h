@@ -13,8 +13,13 @@
 // are 8 pooled columns x 8 channel quads: a lane folds the row taps of a ROI
 // into four gradients (its pooled column, its four channels) and adds them to
 // the two cells of each of its column samples with 16-byte LDS accesses.
-// Pooled columns whose cells may coincide are taken in separate turns (the
-// pre-pass stores the spacing at which they cannot).
+// Pooled columns whose cells may coincide (the pre-pass stores the spacing at
+// which they cannot) are not added in the same instruction: the two columns of
+// a pair of lane groups are taken one after the other by both groups, one group
+// adding the low corners and the other the high ones -- an LDS instruction
+// costs the same with eight active lanes as with 64, so nobody sits out.
+// Sampling grids of more than two points per bin come as windows of merged
+// weights instead (WIN): up to seven consecutive cells per pooled column.
 //
 // dy is read from a channel-blocked copy dyb[C/32][R][PH][PW][32]: one 16-byte
 // load per lane fetches (eight pooled columns of) a pooled row, up to 1 KB; the
