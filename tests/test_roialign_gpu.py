@@ -500,6 +500,33 @@ def test_channels_last_rejects_what_it_does_not_take():
     assert abi.forward_nhwc(torch.zeros(1, 8, 8, 8, device='cuda'), rois, (2, 2), 1.0, 2).shape == (1, 2, 2, 8)
 
 
+def test_a_backward_with_a_dense_grid_can_be_recorded_too():
+    """The merged lists of a dense sampling grid are sized by a number that comes back from
+    the device, which a capturing stream cannot wait for: such a call is recorded with the
+    straightforward kernel (atomic adds: same sums, any order) and the replays give the
+    direct call's result within the tolerance."""
+    rng = np.random.default_rng(123)
+    N, C, H, W, R, pooled, scale, S = 2, 16, 40, 60, 50, (5, 6), 0.5, 3
+    ext = np.array([W / scale, H / scale])
+    c = rng.uniform(0, 1, (R, 2)) * ext
+    wh = rng.uniform(2, 60, (R, 2))
+    rois = abi.to_dev(np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32))
+    dy = abi.to_dev(rng.standard_normal((R, C) + pooled).astype(np.float32))
+    dx = torch.empty((N, C, H, W), device='cuda')
+    want = abi.backward(dy, rois, dx.shape, scale, S, assign=True).clone()   # the tile owners
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        abi.backward(dy, rois, dx.shape, scale, S, dx=dx, assign=True, stream=torch.cuda.current_stream().cuda_stream)
+    for replay in range(3):
+        dx.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_parity(dx.cpu().numpy(), want.cpu().numpy(), BWD_TOL, 'replay %d' % replay)
+    native.unpin_workspace()
+
+
 F64_TOL = 1e-12   # binary64: only the backward's summation order may differ
 
 
