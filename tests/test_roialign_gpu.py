@@ -900,6 +900,37 @@ def test_full_size_properties(cfg):
     assert_parity(dx_l.permute(0, 3, 1, 2).cpu().numpy(), dx.cpu().numpy(), BWD_TOL, cfg + ' bwd channels-last')
 
 
+def test_full_size_with_an_adaptive_grid():
+    """The cfg2 tensors with sampling_ratio 0 (ceil(bin size) points per bin and axis: merged
+    lists in both passes): oracle on a subset of the ROIs (forward) and on eight channel planes
+    (backward), the adjoint identity at full size, and the channels-last entry points."""
+    w = workloads.make_workload('cfg2')
+    pooled, scale, S = w['pooled_size'], w['spatial_scale'], 0
+    x, rois, dy = abi.to_dev(w['data']), abi.to_dev(w['rois']), abi.to_dev(w['dy'])
+    abi.set_impl('auto')
+    native.set_option('kernel_timing', 1)
+    try:
+        y = abi.forward(x, rois, pooled, scale, S)
+        dx = abi.backward(dy, rois, x.shape, scale, S, assign=True)
+        assert _last_bracketed_kernel() == 'backward_blocked_kernel'
+    finally:
+        native.set_option('kernel_timing', 0)
+    pick = np.random.default_rng(3).choice(w['rois'].shape[0], 48, replace=False)
+    want = oracle.forward(w['data'], w['rois'][pick], pooled, scale, S)
+    assert_parity(y[torch.from_numpy(pick).cuda()].cpu().numpy(), want, FWD_TOL, 'fwd subset')
+    lhs = float((y.double() * dy.double()).sum())
+    rhs = float((x.double() * dx.double()).sum())
+    assert abs(lhs - rhs) <= 1e-6 * float((y.double().abs() * dy.double().abs()).sum())
+    ch = [0, 37, 70, 103, 136, 169, 202, 255]
+    want_dx = oracle.backward(np.ascontiguousarray(w['dy'][:, ch]), w['rois'],
+                              (x.shape[0], len(ch)) + tuple(x.shape[2:]), scale, S, impl='ordered')
+    assert_parity(dx[:, ch].cpu().numpy(), want_dx, BWD_TOL, 'bwd planes')
+    assert torch.equal(dx, abi.backward(dy, rois, x.shape, scale, S, assign=True)), 'repeats bit for bit'
+    dx_l = abi.backward_nhwc(dy.permute(0, 2, 3, 1).contiguous(), rois,
+                             (x.shape[0], x.shape[2], x.shape[3], x.shape[1]), scale, S, assign=True)
+    assert_parity(dx_l.permute(0, 3, 1, 2).cpu().numpy(), dx.cpu().numpy(), BWD_TOL, 'bwd channels-last')
+
+
 def test_fp16_full_size_subset():
     w = workloads.make_workload('cfg4')
     pooled, scale, S = w['pooled_size'], w['spatial_scale'], w['sampling_ratio']
