@@ -260,10 +260,10 @@ void conv2d_backward_data_ecf81c91(const int device_id, const int n, const float
                                    const int pad_h, const int pad_w, const int stride_h,
                                    const int stride_w, const int dilation_h, const int dilation_w,
                                    float* dx);
-/* (With the option "conv_compute" set to 1 and unit strides the weight gradient is formed from
- * whole zero-padded planes: a non-finite value of x then also meets zeros of dy that belong to a
- * neighbouring channel's or image's positions, and 0 x inf = NaN ends up in the gradient of that
- * neighbouring channel's weights.  Modes 0 and 2 confine a non-finite x to its own channel.) */
+/* (With the option "conv_compute" set to 1 or 2 and unit strides the weight gradient is formed
+ * from whole zero-padded planes: a non-finite value of x then also meets zeros of dy that belong
+ * to a neighbouring channel's or image's positions, and 0 x inf = NaN ends up in the gradient of
+ * that neighbouring channel's weights.  Mode 0 confines a non-finite x to its own channel.) */
 void conv2d_backward_weight_ecf81c91(const int device_id, const int n, const float* dy, const float* x,
                                      const int accumulate, const int batch, const int channels,
                                      const int height, const int width, const int filters,
@@ -298,7 +298,7 @@ void mobula_hip_clear_error(void);
  * in fp32 (results about 2e-3 off; a non-finite value in x can make the weight
  * gradient of a neighbouring channel NaN, see conv2d_backward_weight), 2 splits
  * every operand into two bf16 and forms three bf16 products per multiply-add
- * (results about 5e-6 off);
+ * (results about 5e-6 off; non-finite values as in mode 1);
  * "roialign_tile_columns": 0 (default) lets the backward pass choose its tile
  * width from the size of the map, 56 or 28 fixes it; "roialign_row_split": 0
  * (default) lets it choose how many wavefronts share a tile row's work list,

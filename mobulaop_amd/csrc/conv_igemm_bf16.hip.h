@@ -262,40 +262,52 @@ struct BackwardDataOpsB16 : GatheredB16 {
 // 8, at most kPaddedSpan; blockIdx.y counts the spans of a plane); neighbouring lanes read
 // neighbouring positions, the bf16 values go through LDS and leave 16 bytes per lane.
 constexpr int kPaddedSpan = 4096;
+// The bf16 a copy holds of v: its head (v rounded to bf16, part 0) or its tail (what the head
+// leaves, rounded to bf16, part 1): head + tail carry sixteen significant bits of v.
+__device__ __forceinline__ unsigned short bf16_part(float v, int part) {
+  const unsigned head = pack_bf16(v, 0.0f) & 0xffffu;
+  if (part == 0) return static_cast<unsigned short>(head);
+  return static_cast<unsigned short>(pack_bf16(v - __uint_as_float(head << 16), 0.0f));
+}
 __global__ void __launch_bounds__(256)
 to_padded_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst,
                       unsigned short* __restrict__ shifted, int H, int W, int off_h, int off_w, int Hg, int Wg,
-                      int Gp, int span) {
-  __shared__ __attribute__((aligned(16))) unsigned short vals[kPaddedSpan + 8];
+                      int Gp, int span, size_t tail) {
+  // (tail != 0: the tails of the values as a second set of planes, `tail` halves after the heads)
+  __shared__ __attribute__((aligned(16))) unsigned short vals_s[2][kPaddedSpan + 8];
   const int plane = blockIdx.x, base = blockIdx.y * span;
   const float* in = src + static_cast<size_t>(plane) * H * W;
   auto value_at = [&](int gh, int gw) {
     const int ih = gh - off_h, iw = gw - off_w;
     const bool inside = (gh < Hg) & (static_cast<unsigned>(ih) < static_cast<unsigned>(H)) &
                         (static_cast<unsigned>(iw) < static_cast<unsigned>(W));
-    return static_cast<unsigned short>(
-        pack_bf16(inside ? __builtin_nontemporal_load(in + (inside ? ih * W + iw : 0)) : 0.0f, 0.0f));
+    return inside ? __builtin_nontemporal_load(in + (inside ? ih * W + iw : 0)) : 0.0f;
   };
   const int step_h = 256 / Wg, step_w = 256 - step_h * Wg;   // 256 positions further on
   int g = base + threadIdx.x, gh = g / Wg, gw = g - gh * Wg;
   for (int j = threadIdx.x; j <= span; j += 256) {   // (position base + span: for the shifted copy)
-    vals[j] = value_at(gh, gw);
+    const float v = value_at(gh, gw);
+    vals_s[0][j] = bf16_part(v, 0);
+    if (tail != 0) vals_s[1][j] = bf16_part(v, 1);
     gh += step_h; gw += step_w;
     if (gw >= Wg) { gw -= Wg; ++gh; }
   }
   __syncthreads();
-  for (int j = 8 * threadIdx.x; j < span; j += 8 * 256) {
-    const int g0 = base + j;
-    if (g0 >= Gp) break;
-    const u32x4 a = *reinterpret_cast<const u32x4*>(vals + j);
-    const size_t at = static_cast<size_t>(plane) * Gp + g0;
-    *reinterpret_cast<u32x4*>(dst + at) = a;
-    if (shifted != nullptr) {
-      const unsigned next = vals[j + 8];
-      u32x4 b;
+  for (int part = 0; part < (tail != 0 ? 2 : 1); ++part) {
+    const unsigned short* const vals = vals_s[part];
+    for (int j = 8 * threadIdx.x; j < span; j += 8 * 256) {
+      const int g0 = base + j;
+      if (g0 >= Gp) break;
+      const u32x4 a = *reinterpret_cast<const u32x4*>(vals + j);
+      const size_t at = static_cast<size_t>(plane) * Gp + g0 + part * tail;
+      *reinterpret_cast<u32x4*>(dst + at) = a;
+      if (shifted != nullptr) {
+        const unsigned next = vals[j + 8];
+        u32x4 b;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) b[k] = (a[k] >> 16) | ((k < 3 ? a[k + 1] : next) << 16);
-      *reinterpret_cast<u32x4*>(shifted + at) = b;
+        for (int k = 0; k < 4; ++k) b[k] = (a[k] >> 16) | ((k < 3 ? a[k + 1] : next) << 16);
+        *reinterpret_cast<u32x4*>(shifted + at) = b;
+      }
     }
   }
 }
@@ -309,65 +321,85 @@ to_padded_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict_
 __global__ void __launch_bounds__(256)
 to_padded_bf16_rows_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst,
                            unsigned short* __restrict__ shifted, int H, int W, int off_h, int off_w, int Hg,
-                           int Wg, int Gp, int rows) {
+                           int Wg, int Gp, int rows, size_t tail) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
-  __shared__ __attribute__((aligned(16))) unsigned short vals[kPaddedSpan + 8];
+  __shared__ __attribute__((aligned(16))) unsigned short vals_s[2][kPaddedSpan + 8];
   const int plane = blockIdx.x, r0 = blockIdx.y * rows, r1 = min(r0 + rows, Hg);
   const bool last = (blockIdx.y + 1) * rows >= Hg;
   const int base = r0 * Wg, end = last ? Gp : r1 * Wg, count = end - base;   // (multiples of 8: the launcher sees to it)
-  for (int j = 4 * threadIdx.x; j < count + 8; j += 4 * 256) *reinterpret_cast<unsigned long long*>(vals + j) = 0ull;
+  const int parts = tail != 0 ? 2 : 1;
+  for (int part = 0; part < parts; ++part)
+    for (int j = 4 * threadIdx.x; j < count + 8; j += 4 * 256) *reinterpret_cast<unsigned long long*>(vals_s[part] + j) = 0ull;
   __syncthreads();
   const float* in = src + static_cast<size_t>(plane) * H * W;
   const int ih0 = max(r0 - off_h, 0), ih1 = min(r1 - off_h, H);   // source rows under the span
   for (int i = ih0 * W + 4 * threadIdx.x; i < ih1 * W; i += 4 * 256) {
     const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(in + i));
     const int ih = i / W, iw = i - ih * W;   // (four elements of one row: W is a multiple of four)
-    unsigned short* const out = vals + (ih + off_h) * Wg + iw + off_w - base;
+    const int at = (ih + off_h) * Wg + iw + off_w - base;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) out[k] = static_cast<unsigned short>(pack_bf16(v[k], 0.0f));
+    for (int k = 0; k < 4; ++k) vals_s[0][at + k] = bf16_part(v[k], 0);
+    if (tail != 0) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) vals_s[1][at + k] = bf16_part(v[k], 1);
+    }
   }
   if (threadIdx.x == 0 && !last) {   // the position after the span, for the shifted copy
     const int ih = r1 - off_h, iw = -off_w;
-    if (ih >= 0 && ih < H && iw >= 0 && iw < W) vals[count] = static_cast<unsigned short>(pack_bf16(in[ih * W + iw], 0.0f));
+    if (ih >= 0 && ih < H && iw >= 0 && iw < W) {
+      vals_s[0][count] = bf16_part(in[ih * W + iw], 0);
+      if (tail != 0) vals_s[1][count] = bf16_part(in[ih * W + iw], 1);
+    }
   }
   __syncthreads();
-  for (int j = 8 * threadIdx.x; j < count; j += 8 * 256) {
-    const u32x4 a = *reinterpret_cast<const u32x4*>(vals + j);
-    const size_t at = static_cast<size_t>(plane) * Gp + base + j;
-    *reinterpret_cast<u32x4*>(dst + at) = a;
-    if (shifted != nullptr) {
-      const unsigned next = vals[j + 8];
-      u32x4 b;
+  for (int part = 0; part < parts; ++part) {
+    const unsigned short* const vals = vals_s[part];
+    for (int j = 8 * threadIdx.x; j < count; j += 8 * 256) {
+      const u32x4 a = *reinterpret_cast<const u32x4*>(vals + j);
+      const size_t at = static_cast<size_t>(plane) * Gp + base + j + part * tail;
+      *reinterpret_cast<u32x4*>(dst + at) = a;
+      if (shifted != nullptr) {
+        const unsigned next = vals[j + 8];
+        u32x4 b;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) b[k] = (a[k] >> 16) | ((k < 3 ? a[k + 1] : next) << 16);
-      *reinterpret_cast<u32x4*>(shifted + at) = b;
+        for (int k = 0; k < 4; ++k) b[k] = (a[k] >> 16) | ((k < 3 ? a[k + 1] : next) << 16);
+        *reinterpret_cast<u32x4*>(shifted + at) = b;
+      }
     }
   }
 }
 
 // Rows: filters d; columns: (tap, channel), tap-major; K: (image, grid position).
 struct WeightGradOpsB16 {
-  const unsigned short* __restrict__ dyg;   // [N][D][Gp]
-  const unsigned short* __restrict__ xg;    // [2][N][C][Gp], the second copy shifted by one position
+  const unsigned short* __restrict__ dyg;   // [sets][N][D][Gp]
+  const unsigned short* __restrict__ xg;    // [2][sets][N][C][Gp], the second copy shifted by one position
   float* __restrict__ dw;
   Geometry g; int M, Ncols, K, Gp, Wg, accumulate; unsigned copy_bytes;
-  struct Cursor { int n, j; };   // image, K step within the image
+  // split != 0: dyg and xg hold two sets of planes each, heads then tails of the operands (two
+  // bf16 for every fp32), and K runs over the images three times: dy heads x x heads, dy heads x
+  // x tails, dy tails x x heads
+  int split;
+  struct Cursor { int n, j, pass; };   // image, K step within the image, pass over the images
   struct Step { int delta, a_delta; };
   struct BCtx { int anchor; };   // (kDead for a column past the last)
   struct Column { float* p; bool ok; };
   __device__ __amdgpu_buffer_rsrc_t a_buffer() const {
-    return buffer_of_bytes(dyg, static_cast<unsigned>(g.N) * g.D * Gp * 2u);
+    return buffer_of_bytes(dyg, static_cast<unsigned>(split ? 2 : 1) * g.N * g.D * Gp * 2u);
   }
   __device__ int a_offset(int m) const { return m * Gp * 2; }
   __device__ Cursor cursor(int s) const {
-    const int per_image = Gp / TileB16::BK, n = s / per_image;
-    return Cursor{n, s - n * per_image};
+    const int per_image = Gp / TileB16::BK, n = s / per_image, pass = n / g.N;
+    return Cursor{n - pass * g.N, s - n * per_image, pass};
   }
   __device__ void advance(Cursor& c) const {
-    if (++c.j == Gp / TileB16::BK) { c.j = 0; ++c.n; }
+    if (++c.j == Gp / TileB16::BK) {
+      c.j = 0;
+      if (++c.n == g.N) { c.n = 0; ++c.pass; }
+    }
   }
   __device__ Step step_at(const Cursor& c, int) const {
-    return Step{(c.n * g.C * Gp + c.j * TileB16::BK) * 2, (c.n * g.D * Gp + c.j * TileB16::BK) * 2};
+    const int nx = c.n + (c.pass == 1 ? g.N : 0), ny = c.n + (c.pass == 2 ? g.N : 0);   // which set of planes
+    return Step{(nx * g.C * Gp + c.j * TileB16::BK) * 2, (ny * g.D * Gp + c.j * TileB16::BK) * 2};
   }
   __device__ __amdgpu_buffer_rsrc_t b_buffer(int) const { return buffer_of_bytes(xg, 2u * copy_bytes); }
   __device__ BCtx b_ctx(int n, int) const {

@@ -427,12 +427,19 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
     return;
   }
   hipStream_t stream = call_state().stream;
-  if (compute_mode() == conv::kBf16 && g.stride_h == 1 && g.stride_w == 1 && wt > 0 && g.N > 0) {
-    // bf16 operands in memory on a common padded grid, one plain product per tap
+  if ((compute_mode() == conv::kBf16 || compute_mode() == conv::kBf16x3) && g.stride_h == 1 && g.stride_w == 1 &&
+      wt > 0 && g.N > 0) {
+    // bf16 operands in memory on a common padded grid, one plain product per tap.  With split
+    // operands (head + tail, two bf16 for every fp32) the copies hold two sets of planes, heads
+    // then tails, and the product walks the images three times: head x head, head x tail, tail x head.
+    const bool split = compute_mode() == conv::kBf16x3;
+    const int sets = split ? 2 : 1;
     const int Hg = g.H + 2 * g.pad_h, Wg = g.W + 2 * g.pad_w;
     const long long G = static_cast<long long>(Hg) * Wg, Gp = (G + 31) / 32 * 32;
-    const long long dy_bytes = 2ll * g.N * g.D * Gp, x_bytes = 2ll * g.N * g.C * Gp;
-    if (dy_bytes < (1ll << 31) && 2 * x_bytes < (1ll << 31) && g.OH <= Hg && g.OW <= Wg) {
+    const long long dy_set = 2ll * g.N * g.D * Gp, x_set = 2ll * g.N * g.C * Gp;   // bytes of one set of planes
+    const long long dy_bytes = sets * dy_set, x_bytes = sets * x_set;
+    if (dy_bytes < (1ll << 31) && 2 * x_bytes < (1ll << 31) && 3ll * g.N * Gp < (1ll << 31) && g.OH <= Hg &&
+        g.OW <= Wg) {
       mobula_hip::KernelTimer timer("conv2d_backward_weight", stream);
       const size_t dy_room = (dy_bytes + 255) / 256 * 256, x_room = (x_bytes + 255) / 256 * 256;
       const size_t piece_bytes = sizeof(float) * kMaxPieceBlocks * conv::Tile::BM * conv::Tile::BN;
@@ -442,12 +449,15 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
       unsigned short* const dyg = reinterpret_cast<unsigned short*>(ws);
       unsigned short* const xg = reinterpret_cast<unsigned short*>(ws + dy_room);
       ob.dyg = dyg; ob.xg = xg; ob.dw = dw; ob.g = g; ob.M = g.D; ob.Ncols = g.C * g.KH * g.KW;
-      ob.K = static_cast<int>(g.N * Gp); ob.Gp = static_cast<int>(Gp); ob.Wg = Wg; ob.accumulate = accumulate;
+      ob.split = split ? 1 : 0;
+      ob.K = static_cast<int>((split ? 3 : 1) * g.N * Gp); ob.Gp = static_cast<int>(Gp); ob.Wg = Wg;
+      ob.accumulate = accumulate;
       // the shifted copy follows the first one directly (x_bytes is a multiple of 64): the reads of
       // the last plane that run past its end then land in the other copy or beyond the buffer
       // (zeros), never in workspace bytes that nothing wrote
       ob.copy_bytes = static_cast<unsigned>(x_bytes);
       unsigned short* const xg1 = reinterpret_cast<unsigned short*>(ws + dy_room + x_bytes);
+      const size_t dy_tail = split ? static_cast<size_t>(dy_set / 2) : 0, x_tail = split ? static_cast<size_t>(x_set / 2) : 0;
       // whole grid rows per workgroup and 16-byte loads where rows of both tensors allow it (a span
       // of rows must be a multiple of 8 positions: Wg even and four rows, or any rows if Wg % 8 == 0)
       int rows = (conv::kPaddedSpan - 32) / Wg;   // (the last span also takes the tail of the plane: up to 31 positions)
@@ -458,17 +468,17 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
         rows = std::min(rows, (Hg + 3) / 4 * 4);
         const unsigned spans = static_cast<unsigned>((Hg + rows - 1) / rows);
         conv::to_padded_bf16_rows_kernel<<<dim3(g.N * g.D, spans), 256, 0, stream>>>(
-            dy, dyg, nullptr, g.OH, g.OW, 0, 0, Hg, Wg, static_cast<int>(Gp), rows);
+            dy, dyg, nullptr, g.OH, g.OW, 0, 0, Hg, Wg, static_cast<int>(Gp), rows, dy_tail);
         conv::to_padded_bf16_rows_kernel<<<dim3(g.N * g.C, spans), 256, 0, stream>>>(
-            x, xg, xg1, g.H, g.W, g.pad_h, g.pad_w, Hg, Wg, static_cast<int>(Gp), rows);
+            x, xg, xg1, g.H, g.W, g.pad_h, g.pad_w, Hg, Wg, static_cast<int>(Gp), rows, x_tail);
       } else {
         // a plane in as few, equally long spans as fit the kernel's LDS
         const int spans = static_cast<int>((Gp + conv::kPaddedSpan - 1) / conv::kPaddedSpan);
         const int span = static_cast<int>((Gp / 8 + spans - 1) / spans * 8);
         conv::to_padded_bf16_kernel<<<dim3(g.N * g.D, spans), 256, 0, stream>>>(dy, dyg, nullptr, g.OH, g.OW, 0, 0, Hg,
-                                                                               Wg, static_cast<int>(Gp), span);
+                                                                               Wg, static_cast<int>(Gp), span, dy_tail);
         conv::to_padded_bf16_kernel<<<dim3(g.N * g.C, spans), 256, 0, stream>>>(
-            x, xg, xg1, g.H, g.W, g.pad_h, g.pad_w, Hg, Wg, static_cast<int>(Gp), span);
+            x, xg, xg1, g.H, g.W, g.pad_h, g.pad_w, Hg, Wg, static_cast<int>(Gp), span, x_tail);
       }
       launch_igemm_b16(ob, reinterpret_cast<float*>(ws + dy_room + 2 * x_room), stream);
       MOBULA_HIP_TRY(hipGetLastError());

@@ -220,6 +220,49 @@ def test_full_cfg5_against_torch(mode):
         native.set_option('conv_compute', 0)
 
 
+@pytest.mark.parametrize('shape', [
+    # N, C, H, W, D, kernel, pad: stride 1 (the weight gradient on bf16 planes)
+    (3, 40, 24, 24, 72, (3, 3), (1, 1)),    # rows of four: the 16-byte conversion
+    (2, 33, 19, 21, 50, (3, 2), (2, 0)),    # odd rows: the element-wise conversion
+    (4, 64, 56, 56, 64, (3, 3), (1, 1)),    # planes longer than one conversion span
+    (1, 3, 12, 12, 5, (3, 3), (1, 1)),      # N * C odd: the sets of planes end off a 256-byte boundary
+    (3, 5, 9, 11, 7, (3, 3), (1, 1)),       # likewise with an odd grid width
+    (1, 4, 70, 71, 6, (3, 3), (1, 1)),      # the element-wise conversion over planes of two spans
+])
+def test_split_operands_keep_every_cross_term(shape):
+    # Two bf16 per fp32 and three products (head x head, head x tail, tail x head) leave errors of
+    # about 2^-16 of the operands; leaving out one cross term would leave about 2^-9, the error
+    # of operands rounded to bf16.  Reference: the same sums in float64.
+    N, C, H, W, D, kernel, pad = shape
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(N, C, H, W, generator=g)
+    w = torch.randn(D, C, *kernel, generator=g) * 0.1
+    xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    y_ref = F.conv2d(xr, wr, None, padding=pad)
+    dy = torch.randn(y_ref.shape, generator=g)
+    y_ref.backward(dy.double())
+    try:
+        native.set_option('conv_compute', 1)
+        _leave_nan_patterns_in_the_workspace()
+        native.set_option('conv_compute', 2)
+        xd, wd, dyd = x.cuda(), w.cuda(), dy.cuda()
+        geo = _ci(N, C, H, W, D, kernel[0], kernel[1], pad[0], pad[1], 1, 1, 1, 1)
+        y = torch.full(y_ref.shape, float('nan'), device='cuda')
+        _call('conv2d_forward_c6a7aa85', ctypes.c_int(y.numel()), _ptr(xd), _ptr(wd), _ptr(wd), ctypes.c_int(0),
+              *geo, _ptr(y))
+        _close(y, y_ref, 'y', 3e-5)
+        dx = torch.full(x.shape, float('nan'), device='cuda')
+        _call('conv2d_backward_data_ecf81c91', ctypes.c_int(dx.numel()), _ptr(dyd), _ptr(wd), ctypes.c_int(0),
+              *geo, _ptr(dx))
+        _close(dx, xr.grad, 'dx', 3e-5)
+        dw = torch.full(w.shape, float('nan'), device='cuda')
+        _call('conv2d_backward_weight_ecf81c91', ctypes.c_int(dw.numel()), _ptr(dyd), _ptr(xd), ctypes.c_int(0),
+              *geo, _ptr(dw))
+        _close(dw, wr.grad, 'dw', 3e-5)
+    finally:
+        native.set_option('conv_compute', 0)
+
+
 def _leave_nan_patterns_in_the_workspace():
     # The bf16 products keep copies of their operands in the calling thread's workspace, which
     # is not cleared between calls: a product of NaN inputs (conv_compute must be 1) leaves NaN
