@@ -12,6 +12,8 @@
 // spatial order, so what one L2 has to hold is a 128-byte-per-pixel slice of
 // the neighbourhood the XCD is currently working in.
 #pragma once
+#include <type_traits>
+
 #include "roialign_geometry.h"
 
 namespace roialign {
@@ -334,85 +336,137 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
     for (int pwb = 0; pwb < PW; pwb += K::PWB) {
       const int pw = pwb + grp;
       const bool bin_on = pw < PW && quad_on;
+      // Column corners of this lane's pooled column (samples 0 and 1: the grid is at most
+      // 2 x 2 here).  A corner that does not exist (outside the map, past the grid, no bin
+      // for this lane) or that repeats an earlier one is not loaded.
+      int coff[4];
+      float cw[4];
+      if (image_ok) {
+        need_cols(pwb, 0, gw);
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          const ColEntry e = cols[grp * CWIN + min(a, gw - 1) - col_x0];
+          const bool ok = e.lo >= 0 && a < gw && bin_on;
+          coff[2 * a] = ok ? e.lo + lane_off : kDead;
+          coff[2 * a + 1] = ok ? e.hi + lane_off : kDead;
+          cw[2 * a] = ok ? e.wl : 0.0f;
+          cw[2 * a + 1] = ok ? e.wh : 0.0f;
+        }
+        const bool both = coff[0] != kDead && coff[2] != kDead;
+        const bool same = both && coff[2] == coff[0];
+        const bool next = both && !same && coff[2] == coff[1];
+        cw[0] += same ? cw[2] : 0.0f;
+        cw[1] += same ? cw[3] : (next ? cw[2] : 0.0f);
+        if (same || next) { coff[2] = coff[3]; cw[2] = cw[3]; coff[3] = kDead; cw[3] = 0.0f; }
+        if (same) { coff[2] = kDead; cw[2] = 0.0f; }
+      }
+      // how many of the four corner slots any lane uses: boxes whose samples are at most a
+      // pixel apart need three (two when both samples of every bin share their pixels)
+      const int ncol = !image_ok ? 2 : __ballot(coff[3] != kDead) != 0 ? 4 : __ballot(coff[2] != kDead) != 0 ? 3 : 2;
+      // A map row's contribution to this lane's pooled column, t(row) = sum over the column
+      // corners of weight x value, is the same for every sample that touches the row: samples
+      // less than a pixel apart share rows, within a bin and from one bin to the next (rows
+      // only go up), so t of the two rows of the last sample is carried along and a row is
+      // fetched once per pooled column however many samples use it.
+      // (With eight channels per lane the carried sums would not fit the registers that four
+      // wavefronts per SIMD leave: 16-bit maps share rows within a pooled row only.)
+      constexpr bool CARRY = CPL <= 4;
+      int carry_off[2] = {kDead, kDead};   // (no row has this offset)
+      float carry[2][CPL];
+#pragma unroll
+      for (int i = 0; i < CPL; ++i) carry[0][i] = carry[1][i] = 0.0f;
+      auto pooled_rows = [&](auto corner_slots) {
+      constexpr int NC = decltype(corner_slots)::value;
 #pragma nounroll
       for (int ph = ph0; ph < ph0 + rp; ++ph) {
         float acc[CPL];
 #pragma unroll
         for (int i = 0; i < CPL; ++i) acc[i] = 0.0f;
         if (image_ok) {
-#pragma nounroll
-          for (int iy0 = 0; iy0 < gh; iy0 += 2) {
-            // Row corners of samples iy0, iy0 + 1: the same for every lane, so they
-            // sit in scalar registers and steer uniform branches.
-            const int ny = min(2, gh - iy0);
-            need_rows(ph * gh + iy0, ny);
-            int roff[4];
-            float rw[4];
-            bool rlive[4];
+          // Row corners of samples 0 and 1: the same for every lane, so they sit in scalar
+          // registers and steer uniform branches.
+          need_rows(ph * gh, gh);
+          int roff[4];
+          float rw[4];
+          int from[4];   // -1: no such corner; 0: loaded; 5, 6: the carried rows; 7: the sample's other row
+          {
+            int known[2] = {carry_off[0], carry_off[1]};   // the carried rows by the time of each sample
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
-              const RowEntry e = rows[ph * gh + iy0 + min(a, ny - 1) - row_s0];
-              roff[2 * a] = uni_i(e.lo); roff[2 * a + 1] = uni_i(e.hi);
+              const RowEntry e = rows[ph * gh + min(a, gh - 1) - row_s0];
+              const int lo = uni_i(e.lo), hi = uni_i(e.hi);
+              roff[2 * a] = lo; roff[2 * a + 1] = hi;
               rw[2 * a] = uni_f(e.wl); rw[2 * a + 1] = uni_f(e.wh);
-              rlive[2 * a] = rlive[2 * a + 1] = roff[2 * a] >= 0 && a < ny;
-            }
-            // samples less than a pixel apart share rows: fetch a shared row once
-            if (rlive[0] && rlive[2]) {
-              if (roff[2] == roff[0]) {
-                rw[0] += rw[2]; rw[1] += rw[3];
-                rlive[2] = rlive[3] = false;
-              } else if (roff[2] == roff[1]) {
-                rw[1] += rw[2];
-                rlive[2] = false;
+              if (lo >= 0 && a < gh) {
+                from[2 * a] = lo == known[0] ? 5 : lo == known[1] ? 6 : 0;
+                from[2 * a + 1] = hi == lo ? 7 : hi == known[0] ? 5 : hi == known[1] ? 6 : 0;
+                known[0] = lo; known[1] = hi;
+              } else {
+                from[2 * a] = from[2 * a + 1] = -1;
               }
             }
-#pragma nounroll
-            for (int ix0 = 0; ix0 < gw; ix0 += 2) {
-              // Column corners of samples ix0, ix0 + 1 of this lane's pooled column.
-              // A corner that does not exist (outside the map, past the grid, no
-              // bin for this lane) or that repeats an earlier one is not loaded.
-              const int nx = min(2, gw - ix0);
-              need_cols(pwb, ix0, nx);
-              int coff[4];
-              float cw[4];
+          }
+          // up to sixteen corners: four rows (scalar) x four columns (per lane)
+          typename LaneData<T>::type v[4][NC];
 #pragma unroll
-              for (int a = 0; a < 2; ++a) {
-                const ColEntry e = cols[grp * CWIN + ix0 + min(a, nx - 1) - col_x0];
-                const bool ok = e.lo >= 0 && a < nx && bin_on;
-                coff[2 * a] = ok ? e.lo + lane_off : kDead;
-                coff[2 * a + 1] = ok ? e.hi + lane_off : kDead;
-                cw[2 * a] = ok ? e.wl : 0.0f;
-                cw[2 * a + 1] = ok ? e.wh : 0.0f;
-              }
-              {
-                const bool both = coff[0] != kDead && coff[2] != kDead;
-                const bool same = both && coff[2] == coff[0];
-                const bool next = both && !same && coff[2] == coff[1];
-                cw[0] += same ? cw[2] : 0.0f;
-                cw[1] += same ? cw[3] : (next ? cw[2] : 0.0f);
-                if (same || next) { coff[2] = kDead; cw[2] = 0.0f; }
-                if (same) { coff[3] = kDead; cw[3] = 0.0f; }
-              }
-              // sixteen corners: four rows (scalar) x four columns (per lane)
-              typename LaneData<T>::type v[4][4];
+          for (int r = 0; r < 4; ++r)
+            if (from[r] == 0) {
 #pragma unroll
-              for (int r = 0; r < 4; ++r)
-                if (rlive[r]) {
+              for (int c = 0; c < NC; ++c) v[r][c] = buffer_load_lane<T>(plane, coff[c], roff[r]);
+            }
+          if constexpr (CARRY) {
 #pragma unroll
-                  for (int c = 0; c < 4; ++c) v[r][c] = buffer_load_lane<T>(plane, coff[c], roff[r]);
-                }
+            for (int a = 0; a < 2; ++a) {
+              if (from[2 * a] < 0) continue;
+              float t[2][CPL];
 #pragma unroll
-              for (int r = 0; r < 4; ++r)
-                if (rlive[r]) {
+              for (int k = 0; k < 2; ++k) {
+                const int r = 2 * a + k;
+                if (from[r] == 0) {
 #pragma unroll
                   for (int i = 0; i < CPL; ++i) {
-                    float t = cw[0] * static_cast<float>(v[r][0][i]);
+                    float u = cw[0] * static_cast<float>(v[r][0][i]);
 #pragma unroll
-                    for (int c = 1; c < 4; ++c) t = fmaf(cw[c], static_cast<float>(v[r][c][i]), t);
-                    acc[i] = fmaf(rw[r], t, acc[i]);
+                    for (int c = 1; c < NC; ++c) u = fmaf(cw[c], static_cast<float>(v[r][c][i]), u);
+                    t[k][i] = u;
                   }
+                } else if (from[r] == 5) {
+#pragma unroll
+                  for (int i = 0; i < CPL; ++i) t[k][i] = carry[0][i];
+                } else if (from[r] == 6) {
+#pragma unroll
+                  for (int i = 0; i < CPL; ++i) t[k][i] = carry[1][i];
+                } else {
+#pragma unroll
+                  for (int i = 0; i < CPL; ++i) t[k][i] = t[0][i];
                 }
+#pragma unroll
+                for (int i = 0; i < CPL; ++i) acc[i] = fmaf(rw[r], t[k][i], acc[i]);
+              }
+              carry_off[0] = roff[2 * a]; carry_off[1] = roff[2 * a + 1];
+#pragma unroll
+              for (int i = 0; i < CPL; ++i) { carry[0][i] = t[0][i]; carry[1][i] = t[1][i]; }
             }
+          } else {
+            // a repeated row's weight goes to the corner that fetched the row
+            if (from[1] == 7) rw[0] += rw[1];
+            if (from[3] == 7) rw[2] += rw[3];
+#pragma unroll
+            for (int r = 2; r < 4; ++r) {
+              if (from[r] == 5) rw[0] += rw[r];
+              if (from[r] == 6) rw[1] += rw[r];
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (from[r] == 0) {
+#pragma unroll
+                for (int i = 0; i < CPL; ++i) {
+                  float u = cw[0] * static_cast<float>(v[r][0][i]);
+#pragma unroll
+                  for (int c = 1; c < NC; ++c) u = fmaf(cw[c], static_cast<float>(v[r][c][i]), u);
+                  acc[i] = fmaf(rw[r], u, acc[i]);
+                }
+              }
           }
         }
         if (pow2) {
@@ -438,6 +492,10 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
             stage[(CPL * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i]);
         }
       }
+      };
+      if (ncol == 4) pooled_rows(std::integral_constant<int, 4>());
+      else if (ncol == 3) pooled_rows(std::integral_constant<int, 3>());
+      else pooled_rows(std::integral_constant<int, 2>());
     }
     if (NHWC) continue;
     // the wavefront's outputs of this pass leave LDS in the order of y

@@ -320,7 +320,24 @@ __device__ __forceinline__ void build_lists_body(unsigned block, const ListsArgs
       // each in lane order: sample order, since sample coordinates never decrease with the lane.
       // That also makes the lanes of a row contiguous among the live ones, so a tap's place
       // follows from counts alone: lane r < 16 holds the numbers of row r.
-      const int row0 = u.w0 != 0.0f ? u.pos : -1, row1 = u.w1 != 0.0f ? u.pos + 1 : -1;
+      int row0 = u.w0 != 0.0f ? u.pos : -1, row1 = u.w1 != 0.0f ? u.pos + 1 : -1;
+      float w0 = u.w0, w1 = u.w1;
+      if (S == 2) {
+        // Samples less than a pixel apart share rows: the second sample of a pooled row hands
+        // the parts that land on a row of the first one to it (one tap, the weights added up:
+        // a tap is a load of a row of dy for the tile owner).
+        const int next_row0 = __shfl_down(row0, 1), next_row1 = __shfl_down(row1, 1);
+        const float next_w0 = __shfl_down(w0, 1), next_w1 = __shfl_down(w1, 1);
+        const int first_row0 = __shfl_up(row0, 1), first_row1 = __shfl_up(row1, 1);
+        if ((lane & 1) == 0) {
+          if (next_row0 >= 0 && next_row0 == row0) w0 += next_w0;
+          if (next_row0 >= 0 && next_row0 == row1) w1 += next_w0;
+          if (next_row1 >= 0 && next_row1 == row1) w1 += next_w1;
+        } else {
+          if (row0 >= 0 && (row0 == first_row0 || row0 == first_row1)) row0 = -1;
+          if (row1 >= 0 && row1 == first_row1) row1 = -1;
+        }
+      }
       const unsigned long long below = (1ull << lane) - 1ull;
       const int before0 = __popcll(__ballot(row0 >= 0) & below), before1 = __popcll(__ballot(row1 >= 0) & below);
       int n0 = 0, n1 = 0;   // low and high parts on row `lane`
@@ -337,8 +354,8 @@ __device__ __forceinline__ void build_lists_body(unsigned block, const ListsArgs
       // row r starts at (low parts before r) + (high parts before r); its high parts come first
       const int low_before = __shfl(upto0 - n0, max(row1, 0));    // low parts on rows above row1
       const int high_upto = __shfl(upto1, max(row0, 0));          // high parts on rows up to and including row0
-      if (row1 >= 0) table->taps[low_before + before1] = RowTap{ph, u.w1};
-      if (row0 >= 0) table->taps[high_upto + before0] = RowTap{ph, u.w0};
+      if (row1 >= 0) table->taps[low_before + before1] = RowTap{ph, w1};
+      if (row0 >= 0) table->taps[high_upto + before0] = RowTap{ph, w0};
       if (lane < kTileRows)
         table->index[lane] = static_cast<unsigned short>((upto0 - n0 + upto1 - n1) | ((n0 + n1) << 8));
     }
