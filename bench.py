@@ -204,7 +204,7 @@ def short_roialign_run(name, steps=20, warmup=3, nhwc=False):
     return out
 
 
-def short_conv_run(mode='fp32', steps=5, warmup=2):
+def short_conv_run(mode='fp32', steps=20, warmup=5):
     """cfg5 with fp32 products, with operands rounded to bf16, or with every operand split
     into two bf16 (three products): ms per step (forward + data gradient + weight gradient),
     fraction of the matrix peak of that type, parity against torch's conv2d on the CPU (outputs

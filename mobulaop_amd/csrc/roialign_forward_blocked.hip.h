@@ -7,7 +7,9 @@
 // 16-byte load per lane fetches one bilinear corner of eight bins (1 KB),
 // sixteen such loads are in flight per lane, and every lane sums its own bin:
 // no cross-lane traffic.  Row corners are the same for the
-// whole wavefront and live in scalar registers.
+// whole wavefront and live in scalar registers; a map row that several samples
+// of a pooled column touch (samples less than a pixel apart, within a bin or in
+// neighbouring bins) is fetched once and its weighted column sum reused.
 // Channel block b is only ever read by XCD b % 8 and ROIs are visited in
 // spatial order, so what one L2 has to hold is a 128-byte-per-pixel slice of
 // the neighbourhood the XCD is currently working in.
@@ -20,8 +22,8 @@ namespace roialign {
 
 struct FwdBlocked {
   static constexpr int NW = 4;         // independent wavefronts per workgroup
-  static constexpr int MAXT = 128;     // column samples held in LDS (16 for each of 8 pooled columns)
-  static constexpr int ROWT = 96;      // row samples held in LDS
+  static constexpr int MAXT = 16;      // column samples held in LDS (two for each of 8 pooled columns)
+  static constexpr int ROWT = 64;      // row samples held in LDS at a time
   static constexpr int PWB = 8;        // pooled columns per step (one per group of 8 lanes)
   static constexpr int CELL = 32;      // side of the sorting cells in pixels
   static constexpr int MAXCELLS = 8192;

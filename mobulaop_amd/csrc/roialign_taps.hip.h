@@ -16,7 +16,9 @@
 // reads them back:
 //   row taps  of (roi, ty): for each of the tile's rows the (pooled row, weight)
 //                           pairs that land on it, weights already divided by
-//                           the sample count of the bin: a 16-entry index
+//                           the sample count of the bin (the two samples of a
+//                           bin that share a map row give it one tap, their
+//                           weights added up): a 16-entry index
 //                           (start | count << 8) followed by the taps, sorted
 //                           by tile row, then by sample order
 //   col list  of (roi, tx): one 16-byte ColPair per pooled column (padded to a
