@@ -436,6 +436,49 @@ def test_ragged_shapes(impl, shape):
         assert_parity(dx.cpu().numpy(), want, BWD_TOL, 'bwd assign=%s' % assign)
 
 
+@pytest.mark.parametrize('layout', ['nchw', 'nhwc'])
+@pytest.mark.parametrize('pooled,S', [((7, 7), 2), ((14, 14), 2), ((5, 9), 1), ((16, 3), 2)])
+def test_boxes_whose_samples_share_rows_and_columns(pooled, S, layout):
+    # Boxes of 0 .. 1.5 pooled sizes in pixels: samples less than a pixel apart, so a map row (or
+    # column) serves several samples of a bin and of neighbouring bins -- the forward gather fetches
+    # it once and carries its column sum along, the list builder folds a bin's two taps on it into
+    # one.  Boxes sit anywhere, also across the map's borders, where the two rows (columns) of
+    # a sample collapse into one.
+    abi.set_impl('auto')
+    N, C, H, W, R, scale = 2, 40, 23, 37, 120, 0.5
+    rng = np.random.default_rng(4242 + 7 * pooled[0] + S)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    ext_w, ext_h = W / scale, H / scale
+    c = np.stack([rng.uniform(-3, ext_w + 3, R), rng.uniform(-3, ext_h + 3, R)], 1)
+    wh = np.stack([rng.uniform(0, 1.5 * pooled[1] / scale, R), rng.uniform(0, 1.5 * pooled[0] / scale, R)], 1)
+    wh[::7] = 0.0                                        # boxes without an extent
+    c[1::9, 1] = ext_h - rng.uniform(0, 1.0, len(c[1::9]))   # on the last row
+    c[2::11, 0] = rng.uniform(-1.0, 0.5, len(c[2::11]))      # on the first column
+    rois = np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+    dy = rng.standard_normal((R, C) + pooled).astype(np.float32)
+    want_y = oracle.forward(x, rois, pooled, scale, S)
+    want_dx = oracle.backward(dy, rois, x.shape, scale, S, impl='ordered')
+    if layout == 'nchw':
+        y = abi.forward(abi.to_dev(x), abi.to_dev(rois), pooled, scale, S).cpu().numpy()
+        dx = abi.backward(abi.to_dev(dy), abi.to_dev(rois), x.shape, scale, S, assign=True).cpu().numpy()
+    else:
+        y = abi.forward_nhwc(abi.to_dev(x.transpose(0, 2, 3, 1)), abi.to_dev(rois), pooled, scale, S)
+        y = y.cpu().numpy().transpose(0, 3, 1, 2)
+        dx = abi.backward_nhwc(abi.to_dev(dy.transpose(0, 2, 3, 1)), abi.to_dev(rois), (N, H, W, C), scale, S,
+                               assign=True).cpu().numpy().transpose(0, 3, 1, 2)
+    assert_parity(y, want_y, FWD_TOL, 'fwd')
+    assert_parity(dx, want_dx, BWD_TOL, 'bwd')
+    # 16-bit maps take the path that shares rows within a bin only
+    x16 = x.astype(np.float16)
+    if layout == 'nchw':
+        y16 = abi.forward(abi.to_dev(x16), abi.to_dev(rois), pooled, scale, S).cpu().numpy()
+    else:
+        y16 = abi.forward_nhwc(abi.to_dev(np.ascontiguousarray(x16.transpose(0, 2, 3, 1))), abi.to_dev(rois), pooled,
+                               scale, S).cpu().numpy().transpose(0, 3, 1, 2)
+    want16 = oracle.forward(x16.astype(np.float32), rois, pooled, scale, S)
+    assert_parity(y16.astype(np.float32), want16.astype(np.float16).astype(np.float32), FP16_TOL, 'fwd fp16')
+
+
 @pytest.mark.parametrize('shape', [
     # N, C, H, W, R, pooled, scale, S
     (3, 68, 33, 47, 37, (7, 7), 0.25, 2),     # ragged last channel block
