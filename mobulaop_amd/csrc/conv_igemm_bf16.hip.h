@@ -34,6 +34,13 @@
 // in slots chunk ^ ((r >> 2) & 3), which puts the 16-byte fragment reads of
 // sixteen neighbouring rows on all 64 banks, each once.
 //
+// Split operands (fp32-like results at the matrix cores' bf16 rate): every fp32
+// value as two bf16, its head (the value rounded to bf16) and its tail (what the
+// head leaves, rounded to bf16), 16 significant bits together.  The pre-passes
+// write both in one pass over the fp32 tensor, the tails as a second set of
+// planes, and a product walks its K steps three times: head x head, head x tail,
+// tail x head (tail x tail is below fp32's own rounding).
+//
 // Replaces, like conv_igemm.hip.h, the per-image im2col + matrix product of
 // opzoo/Convolution/Convolution.py:17-57.
 #pragma once
@@ -47,13 +54,28 @@ struct TileB16 {
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
+// The bf16 a copy holds of v: its head (v rounded to bf16, part 0) or its tail (what the head
+// leaves, rounded to bf16, part 1): head + tail carry sixteen significant bits of v.
+__device__ __forceinline__ unsigned short bf16_part(float v, int part) {
+  const unsigned head = pack_bf16(v, 0.0f) & 0xffffu;
+  if (part == 0) return static_cast<unsigned short>(head);
+  return static_cast<unsigned short>(pack_bf16(v - __uint_as_float(head << 16), 0.0f));
+}
+// heads (part 0) or tails (part 1) of two values, packed like pack_bf16
+__device__ __forceinline__ unsigned pack_bf16_parts(float lo, float hi, int part) {
+  return static_cast<unsigned>(bf16_part(lo, part)) | (static_cast<unsigned>(bf16_part(hi, part)) << 16);
+}
+
 // dst[n][c / 32][p][c % 32] = bf16(src[n][c][p]) for c < C, zero for C <= c < Cpad.  One
 // workgroup: 64 pixels x 64 channels (two channel blocks) through LDS.  VEC: P is a multiple
 // of four and src 16-byte aligned, a lane reads four pixels at a time.  The source is read
 // once: its loads leave the caches to the copy that is about to be read.
+// tail != 0: a second copy, `tail` halves after the first, holds the tails of the values (what
+// their bf16 heads leave).
 template <bool VEC>
 __global__ void __launch_bounds__(256)
-to_blocked_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst, int C, int Cpad, int P) {
+to_blocked_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst, int C, int Cpad, int P,
+                       size_t tail) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   __shared__ float tile[64][65];
   const int n = blockIdx.z, c0 = blockIdx.y * 64, p0 = blockIdx.x * 64;
@@ -87,16 +109,24 @@ to_blocked_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict
       u32x4 v;
 #pragma unroll
       for (int j = 0; j < 4; ++j) v[j] = pack_bf16(tile[cl + 2 * j][pl], tile[cl + 2 * j + 1][pl]);
-      *reinterpret_cast<u32x4*>(dst + ((static_cast<size_t>(n) * (Cpad / 32) + c / 32) * P + p) * 32 + 8 * cq) = v;
+      unsigned short* const to = dst + ((static_cast<size_t>(n) * (Cpad / 32) + c / 32) * P + p) * 32 + 8 * cq;
+      *reinterpret_cast<u32x4*>(to) = v;
+      if (tail != 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = pack_bf16_parts(tile[cl + 2 * j][pl], tile[cl + 2 * j + 1][pl], 1);
+        *reinterpret_cast<u32x4*>(to + tail) = v;
+      }
     }
   }
 }
 
 // out[(c / 32) * taps + tap][m][c % 32] = bf16(w[m * stride_m + c * stride_c + tap]) for m < M and
-// c < C, else 0 (m < Mpad, c < Cpad).
+// c < C, else 0 (m < Mpad, c < Cpad).  tail != 0: three copies `tail` halves apart, heads, heads
+// again and tails (what the bf16 heads leave): the weights of the three passes of a product with
+// split operands, one after the other like the K steps that read them.
 __global__ void __launch_bounds__(256)
 arrange_weights_bf16_kernel(const float* __restrict__ w, unsigned short* __restrict__ out, int M, int Mpad,
-                            int C, int Cpad, int taps, long long stride_m, long long stride_c) {
+                            int C, int Cpad, int taps, long long stride_m, long long stride_c, size_t tail) {
   const long long total = static_cast<long long>(Mpad) * taps * Cpad / 2;   // pairs of channels
   const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= total) return;
@@ -106,6 +136,10 @@ arrange_weights_bf16_kernel(const float* __restrict__ w, unsigned short* __restr
   const float lo = (m < M && c < C) ? w[m * stride_m + c * stride_c + tap] : 0.0f;
   const float hi = (m < M && c + 1 < C) ? w[m * stride_m + (c + 1) * stride_c + tap] : 0.0f;
   reinterpret_cast<unsigned*>(out)[i] = pack_bf16(lo, hi);
+  if (tail != 0) {
+    reinterpret_cast<unsigned*>(out + tail)[i] = pack_bf16(lo, hi);
+    reinterpret_cast<unsigned*>(out + 2 * tail)[i] = pack_bf16_parts(lo, hi, 1);
+  }
 }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of_bytes(const void* base, unsigned bytes) {
@@ -116,28 +150,44 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of_bytes(const void* ba
 constexpr int kFarOutside = -(1 << 30);
 
 // A K step as (filter row, filter column, channel block); wavefront-uniform, kept in scalar registers.
-struct StepCursor { int kh, kw, cb; };
+struct StepCursor { int kh, kw, cb, pass; };
 
 // What the operand functors of igemm_tile_b16 have in common: the weights and the walk over K.
 struct GatheredB16 {
   const unsigned short* __restrict__ wp;    // [K / 32][mpad][32]
-  const unsigned short* __restrict__ src;   // [images][cpad / 32][pixels][32]
-  Geometry g; int M, Ncols, K, cpad, mpad;
+  const unsigned short* __restrict__ src;   // [sets][images][cpad / 32][pixels][32]
+  // K: what the tile loop runs over.  Plain bf16 operands: K = taps * cpad, one set of source
+  // planes.  Split operands (source_tail != 0; two bf16 for every fp32, head and tail): K is three
+  // times that, the steps three times over -- weight heads x source heads, weight heads x source
+  // tails, weight tails x source heads -- with the weights of the three passes one after the other
+  // in wp and the source's tails `source_tail` bytes after its heads.
+  Geometry g; int M, Ncols, K, cpad, mpad, source_tail;
+  __device__ int steps_of_a_pass() const { return g.KH * g.KW * (cpad / 32); }
   __device__ __amdgpu_buffer_rsrc_t a_buffer() const {
     return buffer_of_bytes(wp, static_cast<unsigned>(mpad) * static_cast<unsigned>(K) * 2u);
   }
   __device__ int a_offset(int m) const { return m * 64; }
   typedef StepCursor Cursor;
   __device__ StepCursor cursor(int s) const {
-    const int taps = g.KH * g.KW, cb = s / taps, tap = s - cb * taps, kh = tap / g.KW;
-    return StepCursor{kh, tap - kh * g.KW, cb};
+    const int pass = s / steps_of_a_pass(), s1 = s - pass * steps_of_a_pass();
+    const int taps = g.KH * g.KW, cb = s1 / taps, tap = s1 - cb * taps, kh = tap / g.KW;
+    return StepCursor{kh, tap - kh * g.KW, cb, pass};
   }
   __device__ void advance(StepCursor& c) const {
-    if (++c.kw == g.KW) { c.kw = 0; if (++c.kh == g.KH) { c.kh = 0; ++c.cb; } }
+    if (++c.kw == g.KW) {
+      c.kw = 0;
+      if (++c.kh == g.KH) {
+        c.kh = 0;
+        if (++c.cb == cpad / 32) { c.cb = 0; ++c.pass; }
+      }
+    }
   }
+  // byte offset of the set of source planes that the cursor's pass reads
+  __device__ int source_set_bytes(const StepCursor& c) const { return c.pass == 1 ? source_tail : 0; }
   // the images from the one column n0 lies in, as a raw buffer
   __device__ __amdgpu_buffer_rsrc_t images_from(int first, size_t image_bytes) const {
-    const size_t skip = static_cast<size_t>(first) * image_bytes, left = static_cast<size_t>(g.N) * image_bytes - skip;
+    const size_t skip = static_cast<size_t>(first) * image_bytes;
+    const size_t left = static_cast<size_t>(source_tail != 0 ? 2 : 1) * g.N * image_bytes - skip;
     return buffer_of_bytes(reinterpret_cast<const char*>(src) + skip,
                            static_cast<unsigned>(left < kRecordLimit ? left : kRecordLimit));
   }
@@ -161,7 +211,7 @@ struct ForwardOpsB16 : GatheredB16 {
   __device__ int plane_bytes() const { return g.H * g.W * 64; }
   __device__ Step step_at(const StepCursor& c, int s) const {
     const int dh = c.kh * g.dil_h, dw = c.kw * g.dil_w;
-    return Step{dh, dw, c.cb * plane_bytes() + (dh * g.W + dw) * 64, s * mpad * 64};
+    return Step{dh, dw, c.cb * plane_bytes() + (dh * g.W + dw) * 64 + source_set_bytes(c), s * mpad * 64};
   }
   __device__ __amdgpu_buffer_rsrc_t b_buffer(int n0) const {
     return images_from(__builtin_amdgcn_readfirstlane(n0 / (g.OH * g.OW)), static_cast<size_t>(plane_bytes()) * (cpad / 32));
@@ -202,7 +252,8 @@ struct BackwardDataOpsB16 : GatheredB16 {
   __device__ Step step_at(const StepCursor& c, int s) const {
     const int dh = c.kh * g.dil_h, dw = c.kw * g.dil_w;
     // stride 1: the tap's offset from the anchor pixel (ih + pad, iw + pad) of dy
-    return Step{dh, dw, c.cb * plane_bytes() - (unit_stride() ? (dh * g.OW + dw) * 64 : 0), s * mpad * 64};
+    return Step{dh, dw, c.cb * plane_bytes() - (unit_stride() ? (dh * g.OW + dw) * 64 : 0) + source_set_bytes(c),
+                s * mpad * 64};
   }
   __device__ __amdgpu_buffer_rsrc_t b_buffer(int n0) const {
     return images_from(__builtin_amdgcn_readfirstlane(n0 / (g.H * g.W)), static_cast<size_t>(plane_bytes()) * (cpad / 32));
@@ -262,13 +313,6 @@ struct BackwardDataOpsB16 : GatheredB16 {
 // 8, at most kPaddedSpan; blockIdx.y counts the spans of a plane); neighbouring lanes read
 // neighbouring positions, the bf16 values go through LDS and leave 16 bytes per lane.
 constexpr int kPaddedSpan = 4096;
-// The bf16 a copy holds of v: its head (v rounded to bf16, part 0) or its tail (what the head
-// leaves, rounded to bf16, part 1): head + tail carry sixteen significant bits of v.
-__device__ __forceinline__ unsigned short bf16_part(float v, int part) {
-  const unsigned head = pack_bf16(v, 0.0f) & 0xffffu;
-  if (part == 0) return static_cast<unsigned short>(head);
-  return static_cast<unsigned short>(pack_bf16(v - __uint_as_float(head << 16), 0.0f));
-}
 __global__ void __launch_bounds__(256)
 to_padded_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst,
                       unsigned short* __restrict__ shifted, int H, int W, int off_h, int off_w, int Hg, int Wg,

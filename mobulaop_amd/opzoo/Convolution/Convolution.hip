@@ -229,23 +229,34 @@ bool plan_gather(GatherPlan* plan, const char* what, const conv::Geometry& g, co
 // Workspace of a gathered product with bf16 operands in memory (conv_igemm_bf16.hip.h): the
 // weights as [K step][Mpad][32] bf16, the gathered tensor `src` ([images][channels][src_pixels]
 // fp32) as [images][channel block][src_pixels][32] bf16, the piece buffer.  Fills in the
-// fields of `ops` that describe them.
+// fields of `ops` that describe them.  split: two sets of each, heads then tails of the fp32
+// values, and three passes over K.  *taken = false (and no error): the shape does not fit this
+// path's 32-bit offsets with split operands; the caller has other kernels for that mode.
 bool plan_gather_b16(conv::GatheredB16* ops, float** pieces, const char* what, const conv::Geometry& g,
                      const float* w, int M, int channels, const float* src, int images, int src_pixels,
-                     int columns_per_image, long long stride_m, long long stride_c, hipStream_t stream) {
+                     int columns_per_image, long long stride_m, long long stride_c, bool split, bool* taken,
+                     hipStream_t stream) {
+  *taken = true;
+  const int sets = split ? 2 : 1;
   const int taps = g.KH * g.KW, cpad = (channels + 31) / 32 * 32;
   const long long image_bytes = static_cast<long long>(src_pixels) * cpad * 2;
   // a tile's columns span this many images at most; their byte offsets must stay below 2^31
   const long long span = (conv::TileB16::BN - 1) / std::max(columns_per_image, 1) + 2;
+  if (split && (span + images) * image_bytes >= (1ll << 31)) { *taken = false; return false; }
   if (span * image_bytes >= (1ll << 31)) {
     set_error("%s: images of %lld bytes are too large for the 32-bit offsets of the gather", what, image_bytes);
     return false;
   }
   const int mpad = (M + 255) / 256 * 256;   // (covers row tiles of 128 and of 256)
   const long long k = static_cast<long long>(taps) * cpad, wcount = k * mpad;
-  if (k >= (1ll << 31) || 2 * wcount >= (1ll << 31)) { set_error("%s: weights too large", what); return false; }
-  const size_t weight_bytes = (2 * wcount + 255) / 256 * 256;
-  const size_t source_bytes = (static_cast<size_t>(images) * image_bytes + 255) / 256 * 256;
+  const int weight_sets = split ? 3 : 1;   // (heads, heads again, tails: one per pass)
+  if (3 * k >= (1ll << 31) || 2 * weight_sets * wcount >= (1ll << 31)) {
+    if (split) { *taken = false; return false; }
+    set_error("%s: weights too large", what);
+    return false;
+  }
+  const size_t weight_bytes = (2 * weight_sets * wcount + 255) / 256 * 256;
+  const size_t source_bytes = (static_cast<size_t>(sets) * images * image_bytes + 255) / 256 * 256;
   const size_t piece_bytes = sizeof(float) * kMaxPieceBlocks * conv::Tile::BM * conv::Tile::BN;
   char* ws = static_cast<char*>(mobula_hip::workspace(weight_bytes + source_bytes + piece_bytes));
   if (failed()) return false;
@@ -253,14 +264,19 @@ bool plan_gather_b16(conv::GatheredB16* ops, float** pieces, const char* what, c
   unsigned short* const source = reinterpret_cast<unsigned short*>(ws + weight_bytes);
   *pieces = reinterpret_cast<float*>(ws + weight_bytes + source_bytes);
   ops->wp = weights; ops->src = source; ops->g = g; ops->M = M;
-  ops->K = static_cast<int>(k); ops->cpad = cpad; ops->mpad = mpad;
+  ops->K = static_cast<int>((split ? 3 : 1) * k); ops->cpad = cpad; ops->mpad = mpad;
+  ops->source_tail = split ? static_cast<int>(images * image_bytes) : 0;
+  const size_t weight_tail = split ? static_cast<size_t>(wcount) : 0;                      // (in halves)
+  const size_t source_tail = split ? static_cast<size_t>(images) * image_bytes / 2 : 0;
   conv::arrange_weights_bf16_kernel<<<blocks_for_all(wcount / 2), 256, 0, stream>>>(
-      w, weights, M, mpad, channels, cpad, taps, stride_m, stride_c);
+      w, weights, M, mpad, channels, cpad, taps, stride_m, stride_c, weight_tail);
   const dim3 tgrid((src_pixels + 63) / 64, (cpad + 63) / 64, images);
   if (src_pixels % 4 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0)
-    conv::to_blocked_bf16_kernel<true><<<tgrid, 256, 0, stream>>>(src, source, channels, cpad, src_pixels);
+    conv::to_blocked_bf16_kernel<true><<<tgrid, 256, 0, stream>>>(src, source, channels, cpad, src_pixels,
+                                                                  source_tail);
   else
-    conv::to_blocked_bf16_kernel<false><<<tgrid, 256, 0, stream>>>(src, source, channels, cpad, src_pixels);
+    conv::to_blocked_bf16_kernel<false><<<tgrid, 256, 0, stream>>>(src, source, channels, cpad, src_pixels,
+                                                                   source_tail);
   return true;
 }
 
@@ -324,19 +340,24 @@ MOBULA_KERNEL conv2d_forward_kernel(const int n, const T* x, const T* weight, co
   conv::ForwardOps ops;
   ops.x = x; ops.bias = has_bias ? bias : nullptr; ops.y = y; ops.g = g;
   ops.M = g.D; ops.Ncols = g.N * g.OH * g.OW;
-  if (compute_mode() == conv::kBf16 && g.N < 65536) {
-    // operands as bf16 in memory: channel-blocked copy of x, weights by K step
-    mobula_hip::KernelTimer timer("conv2d_forward", stream);
-    conv::ForwardOpsB16 ob;
-    ob.bias = ops.bias; ob.y = y; ob.Ncols = ops.Ncols;
-    float* pieces = nullptr;
-    const long long taps = g.KH * g.KW;
-    if (!plan_gather_b16(&ob, &pieces, "conv2d_forward", g, weight, g.D, g.C, x, g.N, g.H * g.W, g.OH * g.OW,
-                         g.C * taps, taps, stream))
-      return;
-    launch_igemm_b16(ob, pieces, stream);
-    MOBULA_HIP_TRY(hipGetLastError());
-    return;
+  if ((compute_mode() == conv::kBf16 || compute_mode() == conv::kBf16x3) && g.N < 65536) {
+    // operands as bf16 in memory: channel-blocked copy of x, weights by K step (heads and tails
+    // of both with split operands)
+    bool taken = true;
+    {
+      mobula_hip::KernelTimer timer("conv2d_forward", stream);
+      conv::ForwardOpsB16 ob;
+      ob.bias = ops.bias; ob.y = y; ob.Ncols = ops.Ncols;
+      float* pieces = nullptr;
+      const long long taps = g.KH * g.KW;
+      if (plan_gather_b16(&ob, &pieces, "conv2d_forward", g, weight, g.D, g.C, x, g.N, g.H * g.W, g.OH * g.OW,
+                          g.C * taps, taps, compute_mode() == conv::kBf16x3, &taken, stream)) {
+        launch_igemm_b16(ob, pieces, stream);
+        MOBULA_HIP_TRY(hipGetLastError());
+        return;
+      }
+    }
+    if (taken) return;   // (with an error; not taken: the kernels below split fp32 operands themselves)
   }
   {
     mobula_hip::KernelTimer timer("conv2d_forward", stream);
@@ -375,19 +396,23 @@ MOBULA_KERNEL conv2d_backward_data_kernel(const int n, const T* dy, const T* wei
   conv::BackwardDataOps ops;
   ops.dy = dy; ops.dx = dx; ops.g = g; ops.accumulate = accumulate;
   ops.M = g.C; ops.Ncols = g.N * g.H * g.W;
-  if (compute_mode() == conv::kBf16 && g.N < 65536) {
-    mobula_hip::KernelTimer timer("conv2d_backward_data", stream);
-    conv::BackwardDataOpsB16 ob;
-    ob.dx = dx; ob.accumulate = accumulate; ob.Ncols = ops.Ncols;
-    float* pieces = nullptr;
-    const long long taps = g.KH * g.KW;
-    // row m of the left operand is input channel m: element [m][tap][d] = weight[d][m][tap]
-    if (!plan_gather_b16(&ob, &pieces, "conv2d_backward_data", g, weight, g.C, g.D, dy, g.N, g.OH * g.OW,
-                         g.H * g.W, taps, g.C * taps, stream))
-      return;
-    launch_igemm_b16(ob, pieces, stream);
-    MOBULA_HIP_TRY(hipGetLastError());
-    return;
+  if ((compute_mode() == conv::kBf16 || compute_mode() == conv::kBf16x3) && g.N < 65536) {
+    bool taken = true;
+    {
+      mobula_hip::KernelTimer timer("conv2d_backward_data", stream);
+      conv::BackwardDataOpsB16 ob;
+      ob.dx = dx; ob.accumulate = accumulate; ob.Ncols = ops.Ncols;
+      float* pieces = nullptr;
+      const long long taps = g.KH * g.KW;
+      // row m of the left operand is input channel m: element [m][tap][d] = weight[d][m][tap]
+      if (plan_gather_b16(&ob, &pieces, "conv2d_backward_data", g, weight, g.C, g.D, dy, g.N, g.OH * g.OW,
+                          g.H * g.W, taps, g.C * taps, compute_mode() == conv::kBf16x3, &taken, stream)) {
+        launch_igemm_b16(ob, pieces, stream);
+        MOBULA_HIP_TRY(hipGetLastError());
+        return;
+      }
+    }
+    if (taken) return;
   }
   {
     mobula_hip::KernelTimer timer("conv2d_backward_data", stream);

@@ -221,24 +221,27 @@ def test_full_cfg5_against_torch(mode):
 
 
 @pytest.mark.parametrize('shape', [
-    # N, C, H, W, D, kernel, pad: stride 1 (the weight gradient on bf16 planes)
-    (3, 40, 24, 24, 72, (3, 3), (1, 1)),    # rows of four: the 16-byte conversion
-    (2, 33, 19, 21, 50, (3, 2), (2, 0)),    # odd rows: the element-wise conversion
-    (4, 64, 56, 56, 64, (3, 3), (1, 1)),    # planes longer than one conversion span
-    (1, 3, 12, 12, 5, (3, 3), (1, 1)),      # N * C odd: the sets of planes end off a 256-byte boundary
-    (3, 5, 9, 11, 7, (3, 3), (1, 1)),       # likewise with an odd grid width
-    (1, 4, 70, 71, 6, (3, 3), (1, 1)),      # the element-wise conversion over planes of two spans
+    # N, C, H, W, D, kernel, pad, stride, dilation
+    (3, 40, 24, 24, 72, (3, 3), (1, 1), (1, 1), (1, 1)),    # rows of four: the 16-byte conversion
+    (2, 33, 19, 21, 50, (3, 2), (2, 0), (1, 1), (1, 1)),    # odd rows: the element-wise conversion
+    (4, 64, 56, 56, 64, (3, 3), (1, 1), (1, 1), (1, 1)),    # planes longer than one conversion span
+    (1, 3, 12, 12, 5, (3, 3), (1, 1), (1, 1), (1, 1)),      # N * C odd: the sets of planes end off a 256-byte boundary
+    (3, 5, 9, 11, 7, (3, 3), (1, 1), (1, 1), (1, 1)),       # likewise with an odd grid width
+    (1, 4, 70, 71, 6, (3, 3), (1, 1), (1, 1), (1, 1)),      # the element-wise conversion over planes of two spans
+    (3, 8, 17, 13, 20, (3, 2), (2, 1), (2, 1), (1, 2)),     # strides and dilation: the gathered weight gradient
+    (4, 32, 30, 30, 140, (5, 5), (2, 2), (2, 2), (1, 1)),   # several channel blocks and row tiles, strides
+    (2, 70, 23, 17, 200, (3, 3), (1, 1), (1, 1), (1, 1)),   # channels not a multiple of 32
 ])
 def test_split_operands_keep_every_cross_term(shape):
     # Two bf16 per fp32 and three products (head x head, head x tail, tail x head) leave errors of
     # about 2^-16 of the operands; leaving out one cross term would leave about 2^-9, the error
     # of operands rounded to bf16.  Reference: the same sums in float64.
-    N, C, H, W, D, kernel, pad = shape
+    N, C, H, W, D, kernel, pad, stride, dil = shape
     g = torch.Generator().manual_seed(77)
     x = torch.randn(N, C, H, W, generator=g)
     w = torch.randn(D, C, *kernel, generator=g) * 0.1
     xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
-    y_ref = F.conv2d(xr, wr, None, padding=pad)
+    y_ref = F.conv2d(xr, wr, None, stride=stride, padding=pad, dilation=dil)
     dy = torch.randn(y_ref.shape, generator=g)
     y_ref.backward(dy.double())
     try:
@@ -246,7 +249,7 @@ def test_split_operands_keep_every_cross_term(shape):
         _leave_nan_patterns_in_the_workspace()
         native.set_option('conv_compute', 2)
         xd, wd, dyd = x.cuda(), w.cuda(), dy.cuda()
-        geo = _ci(N, C, H, W, D, kernel[0], kernel[1], pad[0], pad[1], 1, 1, 1, 1)
+        geo = _ci(N, C, H, W, D, kernel[0], kernel[1], pad[0], pad[1], stride[0], stride[1], dil[0], dil[1])
         y = torch.full(y_ref.shape, float('nan'), device='cuda')
         _call('conv2d_forward_c6a7aa85', ctypes.c_int(y.numel()), _ptr(xd), _ptr(wd), _ptr(wd), ctypes.c_int(0),
               *geo, _ptr(y))
