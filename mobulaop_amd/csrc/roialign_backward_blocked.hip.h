@@ -488,8 +488,18 @@ backward_blocked_kernel(const void* __restrict__ dy_any, TO* __restrict__ dx_any
               // this lane's corner of the two samples: its cell, its weight, whether it counts
               float* const a0 = cell0 + ((pc & 0xffff) + which) * K::CS;
               float* const a1 = cell0 + ((pc >> 16) + which) * K::CS;
-              const float w0 = which ? m0 : 1.0f - m0, w1 = which ? m1 : 1.0f - m1;
-              const bool live0 = ((pf >> which) & 1) != 0, live1 = ((pf >> (2 + which)) & 1) != 0;
+              float w0 = which ? m0 : 1.0f - m0;
+              const float w1 = which ? m1 : 1.0f - m1;
+              const bool live0 = ((pf >> which) & 1) != 0;
+              bool live1 = ((pf >> (2 + which)) & 1) != 0;
+              // samples in one pixel pair (bins well under a pixel): one update of the cell for both
+              // (only where the first sample's update is there anyway: the columns that share an
+              // instruction are spaced so that their first samples touch different cells, and so
+              // that their second samples do -- not first against second)
+              if (live0 && live1 && a0 == a1) {
+                w0 += w1;
+                live1 = false;
+              }
               auto add_corner = [&](float* a, float w) {
                 float4 v = *reinterpret_cast<const float4*>(a);
                 v.x = fmaf(gg[0], w, v.x); v.y = fmaf(gg[1], w, v.y);
