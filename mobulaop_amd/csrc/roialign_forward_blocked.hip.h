@@ -30,12 +30,14 @@ struct FwdBlocked {
 };
 
 // Per element type: channels per lane (16 bytes), channels per block of the
-// blocked layout (8 lanes: 128 bytes per pixel), staged outputs per wavefront.
+// blocked layout (8 lanes: 128 bytes per pixel), staged outputs per wavefront
+// (8704 bytes: with the sample tables 39.9 KB per workgroup of four, four workgroups
+// to a CU, which the registers allow anyway; 14 x 14 pooled maps go in four passes).
 template <typename T>
 struct BlockOf {
   static constexpr int CPL = 16 / sizeof(T);
   static constexpr int CB = 8 * CPL;
-  static constexpr int STAGE = 6400 / sizeof(T);
+  static constexpr int STAGE = 8704 / sizeof(T);
 };
 
 // Pooled rows staged per pass, 0 if the shape is not taken by this path.
