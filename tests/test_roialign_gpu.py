@@ -436,6 +436,28 @@ def test_ragged_shapes(impl, shape):
         assert_parity(dx.cpu().numpy(), want, BWD_TOL, 'bwd assign=%s' % assign)
 
 
+@pytest.mark.parametrize('pooled', [(3, 60), (2, 68), (1, 69), (40, 9)])
+@pytest.mark.parametrize('S', [2, 0])
+def test_forward_with_very_wide_or_tall_pooled_maps(pooled, S):
+    # up to 68 pooled columns go through the staged gather (one pooled row per pass at that
+    # width), 69 through the straightforward kernel; 40 pooled rows of 2 samples are more row
+    # samples than the gather holds at a time
+    abi.set_impl('auto')
+    N, C, H, W, R, scale = 2, 36, 50, 90, 14, 0.5
+    rng = np.random.default_rng(99 + pooled[1] + S)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    ext_w, ext_h = W / scale, H / scale
+    c = np.stack([rng.uniform(0, ext_w, R), rng.uniform(0, ext_h, R)], 1)
+    wh = np.stack([rng.uniform(0, ext_w, R), rng.uniform(0, ext_h, R)], 1)
+    wh[::5] *= 0.05
+    rois = np.concatenate([rng.integers(0, N, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+    y = abi.forward(abi.to_dev(x), abi.to_dev(rois), pooled, scale, S).cpu().numpy()
+    assert_parity(y, oracle.forward(x, rois, pooled, scale, S), FWD_TOL, 'fwd')
+    dy = rng.standard_normal((R, C) + pooled).astype(np.float32)
+    dx = abi.backward(abi.to_dev(dy), abi.to_dev(rois), x.shape, scale, S, assign=True).cpu().numpy()
+    assert_parity(dx, oracle.backward(dy, rois, x.shape, scale, S, impl='ordered'), BWD_TOL, 'bwd')
+
+
 @pytest.mark.parametrize('layout', ['nchw', 'nhwc'])
 @pytest.mark.parametrize('pooled,S', [((7, 7), 2), ((14, 14), 2), ((5, 9), 1), ((16, 3), 2)])
 def test_boxes_whose_samples_share_rows_and_columns(pooled, S, layout):
