@@ -380,122 +380,122 @@ forward_blocked_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
 #pragma unroll
       for (int i = 0; i < CPL; ++i) carry[0][i] = carry[1][i] = 0.0f;
       auto pooled_rows = [&](auto corner_slots) {
-      constexpr int NC = decltype(corner_slots)::value;
+        constexpr int NC = decltype(corner_slots)::value;
 #pragma nounroll
-      for (int ph = ph0; ph < ph0 + rp; ++ph) {
-        float acc[CPL];
+        for (int ph = ph0; ph < ph0 + rp; ++ph) {
+          float acc[CPL];
 #pragma unroll
-        for (int i = 0; i < CPL; ++i) acc[i] = 0.0f;
-        if (image_ok) {
-          // Row corners of samples 0 and 1: the same for every lane, so they sit in scalar
-          // registers and steer uniform branches.
-          need_rows(ph * gh, gh);
-          int roff[4];
-          float rw[4];
-          int from[4];   // -1: no such corner; 0: loaded; 5, 6: the carried rows; 7: the sample's other row
-          {
-            int known[2] = {carry_off[0], carry_off[1]};   // the carried rows by the time of each sample
+          for (int i = 0; i < CPL; ++i) acc[i] = 0.0f;
+          if (image_ok) {
+            // Row corners of samples 0 and 1: the same for every lane, so they sit in scalar
+            // registers and steer uniform branches.
+            need_rows(ph * gh, gh);
+            int roff[4];
+            float rw[4];
+            int from[4];   // -1: no such corner; 0: loaded; 5, 6: the carried rows; 7: the sample's other row
+            {
+              int known[2] = {carry_off[0], carry_off[1]};   // the carried rows by the time of each sample
 #pragma unroll
-            for (int a = 0; a < 2; ++a) {
-              const RowEntry e = rows[ph * gh + min(a, gh - 1) - row_s0];
-              const int lo = uni_i(e.lo), hi = uni_i(e.hi);
-              roff[2 * a] = lo; roff[2 * a + 1] = hi;
-              rw[2 * a] = uni_f(e.wl); rw[2 * a + 1] = uni_f(e.wh);
-              if (lo >= 0 && a < gh) {
-                from[2 * a] = lo == known[0] ? 5 : lo == known[1] ? 6 : 0;
-                from[2 * a + 1] = hi == lo ? 7 : hi == known[0] ? 5 : hi == known[1] ? 6 : 0;
-                known[0] = lo; known[1] = hi;
-              } else {
-                from[2 * a] = from[2 * a + 1] = -1;
+              for (int a = 0; a < 2; ++a) {
+                const RowEntry e = rows[ph * gh + min(a, gh - 1) - row_s0];
+                const int lo = uni_i(e.lo), hi = uni_i(e.hi);
+                roff[2 * a] = lo; roff[2 * a + 1] = hi;
+                rw[2 * a] = uni_f(e.wl); rw[2 * a + 1] = uni_f(e.wh);
+                if (lo >= 0 && a < gh) {
+                  from[2 * a] = lo == known[0] ? 5 : lo == known[1] ? 6 : 0;
+                  from[2 * a + 1] = hi == lo ? 7 : hi == known[0] ? 5 : hi == known[1] ? 6 : 0;
+                  known[0] = lo; known[1] = hi;
+                } else {
+                  from[2 * a] = from[2 * a + 1] = -1;
+                }
               }
             }
-          }
-          // up to sixteen corners: four rows (scalar) x four columns (per lane)
-          typename LaneData<T>::type v[4][NC];
+            // up to sixteen corners: four rows (scalar) x four columns (per lane)
+            typename LaneData<T>::type v[4][NC];
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (from[r] == 0) {
+            for (int r = 0; r < 4; ++r)
+              if (from[r] == 0) {
 #pragma unroll
-              for (int c = 0; c < NC; ++c) v[r][c] = buffer_load_lane<T>(plane, coff[c], roff[r]);
-            }
-          if constexpr (CARRY) {
+                for (int c = 0; c < NC; ++c) v[r][c] = buffer_load_lane<T>(plane, coff[c], roff[r]);
+              }
+            if constexpr (CARRY) {
 #pragma unroll
-            for (int a = 0; a < 2; ++a) {
-              if (from[2 * a] < 0) continue;
-              float t[2][CPL];
+              for (int a = 0; a < 2; ++a) {
+                if (from[2 * a] < 0) continue;
+                float t[2][CPL];
 #pragma unroll
-              for (int k = 0; k < 2; ++k) {
-                const int r = 2 * a + k;
+                for (int k = 0; k < 2; ++k) {
+                  const int r = 2 * a + k;
+                  if (from[r] == 0) {
+#pragma unroll
+                    for (int i = 0; i < CPL; ++i) {
+                      float u = cw[0] * static_cast<float>(v[r][0][i]);
+#pragma unroll
+                      for (int c = 1; c < NC; ++c) u = fmaf(cw[c], static_cast<float>(v[r][c][i]), u);
+                      t[k][i] = u;
+                    }
+                  } else if (from[r] == 5) {
+#pragma unroll
+                    for (int i = 0; i < CPL; ++i) t[k][i] = carry[0][i];
+                  } else if (from[r] == 6) {
+#pragma unroll
+                    for (int i = 0; i < CPL; ++i) t[k][i] = carry[1][i];
+                  } else {
+#pragma unroll
+                    for (int i = 0; i < CPL; ++i) t[k][i] = t[0][i];
+                  }
+#pragma unroll
+                  for (int i = 0; i < CPL; ++i) acc[i] = fmaf(rw[r], t[k][i], acc[i]);
+                }
+                carry_off[0] = roff[2 * a]; carry_off[1] = roff[2 * a + 1];
+#pragma unroll
+                for (int i = 0; i < CPL; ++i) { carry[0][i] = t[0][i]; carry[1][i] = t[1][i]; }
+              }
+            } else {
+              // a repeated row's weight goes to the corner that fetched the row
+              if (from[1] == 7) rw[0] += rw[1];
+              if (from[3] == 7) rw[2] += rw[3];
+#pragma unroll
+              for (int r = 2; r < 4; ++r) {
+                if (from[r] == 5) rw[0] += rw[r];
+                if (from[r] == 6) rw[1] += rw[r];
+              }
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
                 if (from[r] == 0) {
 #pragma unroll
                   for (int i = 0; i < CPL; ++i) {
                     float u = cw[0] * static_cast<float>(v[r][0][i]);
 #pragma unroll
                     for (int c = 1; c < NC; ++c) u = fmaf(cw[c], static_cast<float>(v[r][c][i]), u);
-                    t[k][i] = u;
+                    acc[i] = fmaf(rw[r], u, acc[i]);
                   }
-                } else if (from[r] == 5) {
-#pragma unroll
-                  for (int i = 0; i < CPL; ++i) t[k][i] = carry[0][i];
-                } else if (from[r] == 6) {
-#pragma unroll
-                  for (int i = 0; i < CPL; ++i) t[k][i] = carry[1][i];
-                } else {
-#pragma unroll
-                  for (int i = 0; i < CPL; ++i) t[k][i] = t[0][i];
                 }
-#pragma unroll
-                for (int i = 0; i < CPL; ++i) acc[i] = fmaf(rw[r], t[k][i], acc[i]);
-              }
-              carry_off[0] = roff[2 * a]; carry_off[1] = roff[2 * a + 1];
-#pragma unroll
-              for (int i = 0; i < CPL; ++i) { carry[0][i] = t[0][i]; carry[1][i] = t[1][i]; }
             }
+          }
+          if (pow2) {
+#pragma unroll
+            for (int i = 0; i < CPL; ++i) acc[i] *= inv_count;
           } else {
-            // a repeated row's weight goes to the corner that fetched the row
-            if (from[1] == 7) rw[0] += rw[1];
-            if (from[3] == 7) rw[2] += rw[3];
+            asm volatile("" ::: "memory");   // keeps the division out of the common path
 #pragma unroll
-            for (int r = 2; r < 4; ++r) {
-              if (from[r] == 5) rw[0] += rw[r];
-              if (from[r] == 6) rw[1] += rw[r];
+            for (int i = 0; i < CPL; ++i) acc[i] /= count;
+          }
+          if (NHWC) {
+            // y[roi][ph][pw][C]: the lane's channels of its bin are 16 contiguous bytes
+            if (bin_on) {
+              T out[CPL];
+#pragma unroll
+              for (int i = 0; i < CPL; ++i) out[i] = from_float<T>(acc[i]);
+              T* const dst = y + ((static_cast<size_t>(roi) * PH + ph) * PW + pw) * C + c0 + CPL * quad;
+              *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(out);
             }
+          } else if (bin_on) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (from[r] == 0) {
-#pragma unroll
-                for (int i = 0; i < CPL; ++i) {
-                  float u = cw[0] * static_cast<float>(v[r][0][i]);
-#pragma unroll
-                  for (int c = 1; c < NC; ++c) u = fmaf(cw[c], static_cast<float>(v[r][c][i]), u);
-                  acc[i] = fmaf(rw[r], u, acc[i]);
-                }
-              }
+            for (int i = 0; i < CPL; ++i)
+              stage[(CPL * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i]);
           }
         }
-        if (pow2) {
-#pragma unroll
-          for (int i = 0; i < CPL; ++i) acc[i] *= inv_count;
-        } else {
-          asm volatile("" ::: "memory");   // keeps the division out of the common path
-#pragma unroll
-          for (int i = 0; i < CPL; ++i) acc[i] /= count;
-        }
-        if (NHWC) {
-          // y[roi][ph][pw][C]: the lane's channels of its bin are 16 contiguous bytes
-          if (bin_on) {
-            T out[CPL];
-#pragma unroll
-            for (int i = 0; i < CPL; ++i) out[i] = from_float<T>(acc[i]);
-            T* const dst = y + ((static_cast<size_t>(roi) * PH + ph) * PW + pw) * C + c0 + CPL * quad;
-            *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(out);
-          }
-        } else if (bin_on) {
-#pragma unroll
-          for (int i = 0; i < CPL; ++i)
-            stage[(CPL * quad + i) * seg + (ph - ph0) * PW + pw] = from_float<T>(acc[i]);
-        }
-      }
       };
       if (ncol == 4) pooled_rows(std::integral_constant<int, 4>());
       else if (ncol == 3) pooled_rows(std::integral_constant<int, 3>());
