@@ -266,6 +266,67 @@ def test_split_operands_keep_every_cross_term(shape):
         native.set_option('conv_compute', 0)
 
 
+def test_random_shapes_in_every_mode():
+    # sixty seeded shapes (channel counts around the 32-channel blocks, strides, dilation, padding
+    # beyond the kernel, widths with and without 16-byte rows), each in one of the three ways of
+    # forming the products, against torch's float64 convolution and its autograd
+    tol = {0: 2e-5, 2: 3e-5}
+    done = 0
+    for case in range(80):
+        rng = np.random.default_rng(5000 + case)
+        N, C, D = int(rng.integers(1, 5)), int(rng.choice([1, 3, 8, 31, 32, 33, 64, 70])), int(rng.choice([1, 5, 32, 100, 129, 260]))
+        H, W = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        if rng.integers(0, 2):
+            W = (W + 3) // 4 * 4
+        kh, kw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        ph, pw = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+        sh, sw = (1, 1) if rng.integers(0, 3) else (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        dh, dw_ = (1, 1) if rng.integers(0, 3) else (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        mode = int(rng.integers(0, 3))
+        if H + 2 * ph < dh * (kh - 1) + 1 or W + 2 * pw < dw_ * (kw - 1) + 1:
+            continue
+        g = torch.Generator().manual_seed(5000 + case)
+        x = torch.randn(N, C, H, W, generator=g)
+        w = torch.randn(D, C, kh, kw, generator=g) * 0.2
+        xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+        y_ref = F.conv2d(xr, wr, None, stride=(sh, sw), padding=(ph, pw), dilation=(dh, dw_))
+        dy = torch.randn(y_ref.shape, generator=g)
+        y_ref.backward(dy.double())
+        what = 'case {}: mode {} N{} C{} {}x{} D{} k{}x{} p{},{} s{},{} d{},{}'.format(
+            case, mode, N, C, H, W, D, kh, kw, ph, pw, sh, sw, dh, dw_)
+        print(what, flush=True)
+        native.set_option('conv_compute', mode)
+        try:
+            xd, wd, dyd = x.cuda(), w.cuda(), dy.cuda()
+            geo = _ci(N, C, H, W, D, kh, kw, ph, pw, sh, sw, dh, dw_)
+            y = torch.full(y_ref.shape, float('nan'), device='cuda')
+            _call('conv2d_forward_c6a7aa85', ctypes.c_int(y.numel()), _ptr(xd), _ptr(wd), _ptr(wd), ctypes.c_int(0),
+                  *geo, _ptr(y))
+            dx = torch.full(x.shape, float('nan'), device='cuda')
+            _call('conv2d_backward_data_ecf81c91', ctypes.c_int(dx.numel()), _ptr(dyd), _ptr(wd), ctypes.c_int(0),
+                  *geo, _ptr(dx))
+            dw = torch.full(w.shape, float('nan'), device='cuda')
+            _call('conv2d_backward_weight_ecf81c91', ctypes.c_int(dw.numel()), _ptr(dyd), _ptr(xd), ctypes.c_int(0),
+                  *geo, _ptr(dw))
+        finally:
+            native.set_option('conv_compute', 0)
+        if mode == 1:
+            # operands rounded to bf16 are off by up to 2^-9 each: the bound is a share of the sum of
+            # the terms' magnitudes, which a sum that cancels can be far below
+            xa, wa = x.double().abs().requires_grad_(True), w.double().abs().requires_grad_(True)
+            ya = F.conv2d(xa, wa, None, stride=(sh, sw), padding=(ph, pw), dilation=(dh, dw_))
+            ya.backward(dy.double().abs())
+            for got, want, mag, name in ((y, y_ref, ya, ' y'), (dx, xr.grad, xa.grad, ' dx'), (dw, wr.grad, wa.grad, ' dw')):
+                err = float((got.cpu().double() - want.detach()).abs().max())
+                assert err <= 2.0 ** -7 * float(mag.detach().max()), what + name
+        else:
+            _close(y, y_ref, what + ' y', tol[mode])
+            _close(dx, xr.grad, what + ' dx', tol[mode])
+            _close(dw, wr.grad, what + ' dw', tol[mode])
+        done += 1
+    assert done >= 60
+
+
 def _leave_nan_patterns_in_the_workspace():
     # The bf16 products keep copies of their operands in the calling thread's workspace, which
     # is not cleared between calls: a product of NaN inputs (conv_compute must be 1) leaves NaN
