@@ -436,6 +436,65 @@ def test_ragged_shapes(impl, shape):
         assert_parity(dx.cpu().numpy(), want, BWD_TOL, 'bwd assign=%s' % assign)
 
 
+def test_random_shapes_both_layouts():
+    # sixty seeded problems -- odd map sizes, boxes across the borders, tiny and empty boxes, image
+    # numbers outside the batch, every kind of sampling grid, fp16 maps, both tile widths, split rows
+    # and both write-outs of the backward -- against the oracle, in both layouts where channels-last
+    # takes the shape
+    abi.set_impl('auto')
+    for case in range(60):
+        rng = np.random.default_rng(31000 + case)
+        N, C = int(rng.integers(1, 4)), int(rng.choice([4, 8, 12, 32, 36, 64, 68, 100]))
+        H, W, R = int(rng.integers(1, 70)), int(rng.integers(1, 130)), int(rng.integers(0, 60))
+        if rng.integers(0, 2):
+            W = (W + 3) // 4 * 4
+        PH, PW = int(rng.integers(1, 15)), int(rng.integers(1, 20))
+        S = int(rng.choice([0, 0, 1, 2, 2, 3, 4, 5, 7]))
+        scale = float(rng.choice([1.0, 0.5, 0.25, 0.125, 0.3]))
+        fp16 = bool(rng.integers(0, 4) == 0)
+        x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        ew, eh = W / scale, H / scale
+        kind = rng.integers(0, 4, R)
+        c = np.stack([rng.uniform(-0.3 * ew, 1.3 * ew, R), rng.uniform(-0.3 * eh, 1.3 * eh, R)], 1)
+        wh = np.stack([rng.uniform(0, ew, R), rng.uniform(0, eh, R)], 1)
+        wh[kind == 1] *= 0.05
+        wh[kind == 2] = 0.0
+        rois = np.concatenate([rng.integers(-1, N + 1, (R, 1)), c - wh / 2, c + wh / 2], 1).astype(np.float32)
+        dy = rng.standard_normal((R, C, PH, PW)).astype(np.float32)
+        native.set_option('roialign_tile_columns', int(rng.choice([0, 28, 56])))
+        native.set_option('roialign_row_split', int(rng.choice([0, 1, 4])))
+        native.set_option('roialign_row_quads', int(rng.integers(0, 2)))
+        what = 'case {}: N{} C{} {}x{} R{} pooled {}x{} S{} scale {} fp16 {}'.format(case, N, C, H, W, R, PH, PW, S,
+                                                                                   scale, fp16)
+        print(what, flush=True)
+        # (the oracle indexes the map with the box's image number: boxes that name no image are
+        # left out for it; the library gives them zeros)
+        ok = (rois[:, 0] >= 0) & (rois[:, 0] < N)
+        x_in = x.astype(np.float16) if fp16 else x
+        want = oracle.forward(x_in.astype(np.float32), rois[ok], (PH, PW), scale, S)
+        if fp16:
+            want = want.astype(np.float16).astype(np.float32)
+        tol = FP16_TOL if fp16 else FWD_TOL
+        y = abi.forward(abi.to_dev(x_in), abi.to_dev(rois), (PH, PW), scale, S).cpu().numpy().astype(np.float32)
+        if ok.any():
+            assert_parity(y[ok], want, tol, what + ' fwd')
+        assert np.abs(y[~ok]).sum() == 0, what
+        if C % (8 if fp16 else 4) == 0:
+            y_l = abi.forward_nhwc(abi.to_dev(x_in.transpose(0, 2, 3, 1)), abi.to_dev(rois), (PH, PW), scale, S)
+            y_l = y_l.cpu().numpy().astype(np.float32).transpose(0, 3, 1, 2)
+            if ok.any():
+                assert_parity(y_l[ok], want, tol, what + ' fwd channels-last')
+        if fp16:
+            continue
+        want_dx = oracle.backward(dy[ok], rois[ok], x.shape, scale, S, impl='ordered') if ok.any() else np.zeros_like(x)
+        dx = abi.backward(abi.to_dev(dy), abi.to_dev(rois), x.shape, scale, S, assign=bool(case % 2)).cpu().numpy()
+        assert_parity(dx, want_dx, BWD_TOL, what + ' bwd')
+        if native.roialign_channels_last_supported(True, 4, C, H, W, (PH, PW), S, R):
+            dx_l = abi.backward_nhwc(abi.to_dev(dy.transpose(0, 2, 3, 1)), abi.to_dev(rois), (N, H, W, C), scale, S,
+                                     assign=bool(case % 2))
+            assert_parity(dx_l.cpu().numpy().transpose(0, 3, 1, 2), want_dx, BWD_TOL, what + ' bwd channels-last')
+
+
 @pytest.mark.parametrize('pooled', [(3, 60), (2, 68), (1, 69), (40, 9)])
 @pytest.mark.parametrize('S', [2, 0])
 def test_forward_with_very_wide_or_tall_pooled_maps(pooled, S):
