@@ -292,14 +292,17 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // pixels.  Returns false if the problem is too large for the list buffers (or
 // on error); the caller then uses the straightforward kernels.
 // How transpose_dy_blocked_kernel is launched for a problem: channel blocks per
-// workgroup (what 64 KB of LDS hold, at most 4; 0: not at all), workgroups, LDS bytes.
+// workgroup (what 32 KB of LDS hold, at most 4, at least one; 0: not even one in 64 KB), workgroups, LDS bytes.
 struct DyLaunch { int per; long long blocks; size_t lds; int cap; };
 template <typename T>
 DyLaunch dy_launch(const Problem& p) {
   using BB = roialign::BwdBlocked;
   const int cblk = (p.C + BB::CB - 1) / BB::CB;
   const size_t chan_bytes = sizeof(T) * p.PH * p.PW, blk_bytes = BB::CB * chan_bytes;
-  const int per = static_cast<int>(std::min<size_t>(4, (64 * 1024) / blk_bytes));
+  // (as many blocks as 32 KB hold, at least one if 64 KB hold it: with 25 KB blocks -- 14 x 14
+  // pooled maps -- one block per workgroup copies at 5.8 TB/s where two manage 5.1: more
+  // workgroups fit a CU)
+  const int per = blk_bytes > 64 * 1024 ? 0 : static_cast<int>(std::min<size_t>(4, std::max<size_t>(1, (32 * 1024) / blk_bytes)));
   if (per > 0)
     return DyLaunch{per, static_cast<long long>(p.R) * ((cblk + per - 1) / per), per * blk_bytes, 0};
   // large pooled sizes: one channel block per workgroup, in passes of `cap` channels
