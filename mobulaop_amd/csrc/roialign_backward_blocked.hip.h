@@ -64,9 +64,9 @@ inline int backward_row_split(long long images, int H, int W, int cblk) {
   return wide * kTileRows * cblk < 8192 ? BwdBlocked::NSPLIT : 1;
 }
 
-// dy[r][c][ph][pw] -> dyb[cb][r][ph][PWp][32] (R: number of ROIs; PWp >= PW: the pooled columns
-// of a row of the copy, PW as launched), zero where pw >= PW or the channel does not exist.  One workgroup per (ROI, group of `per` channel blocks):
-// the input words of the group are contiguous and so are its output words.
+// dy[r][c][ph][pw] -> dyb[cb][r][ph][pw][32] (R: number of ROIs), zero where the channel does
+// not exist.  One workgroup per (ROI, group of `per` channel blocks): the input words of the
+// group are contiguous and so are the output words of each of its blocks.
 // LDS holds the input as it is; the transposition happens in the reads.
 // T is the element type of dy (float or __half); dyb is fp32 either way.
 // `block`: index among the workgroups (of 256 threads) that transpose.
@@ -76,7 +76,7 @@ inline int backward_row_split(long long images, int H, int W, int cblk) {
 template <typename T>
 __device__ __forceinline__ void transpose_dy_blocked_body(unsigned block, const T* __restrict__ dy,
                                                           float* __restrict__ dyb, int C, int PH, int PW,
-                                                          int PWp, int cblk, int per, int R, int cap) {
+                                                          int cblk, int per, int R, int cap) {
   constexpr int CB = BwdBlocked::CB;
   constexpr int VEC = 16 / sizeof(T);   // elements per 16-byte word
   extern __shared__ __attribute__((aligned(16))) unsigned char tbuf_bytes[];   // [channels][PH * PW] of T
@@ -104,40 +104,35 @@ __device__ __forceinline__ void transpose_dy_blocked_body(unsigned block, const 
       for (int i = threadIdx.x; i < n_in; i += 256) tbuf[i] = src[i];
     }
     __syncthreads();
-    const int per_blk = PH * PWp * (CB / 4);   // 16-byte pieces of one channel block
+    const int per_blk = bins * (CB / 4);   // 16-byte pieces of one channel block
     if (per > 0) {
-      for (int q = threadIdx.x; q < nblk * per_blk; q += 256) {
-        const int blk = q / per_blk, p = q - blk * per_blk;
+      for (int blk = 0; blk < nblk; ++blk) {
         // every channel block has a slab of its own (all ROIs): its owners address it with 32-bit offsets
-        float* const dst = dyb + (static_cast<size_t>(cb0 + blk) * R + r) * PH * PWp * CB;
-        const int cq = p & 7, cell = p >> 3, pw = cell % PWp, ph = cell / PWp;
-        float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if (pw < PW) {
-          const int c = blk * CB + 4 * cq;
-          const T* in = tbuf + c * bins + ph * PW + pw;
+        float* const dst = dyb + (static_cast<size_t>(cb0 + blk) * R + r) * bins * CB;
+        for (int p = threadIdx.x; p < per_blk; p += 256) {
+          const int cq = p & 7, cell = p >> 3, c = blk * CB + 4 * cq;   // channel quad, bin, first channel
+          const T* in = tbuf + c * bins + cell;
+          float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
           if (c + 0 < nch) v.x = to_float(in[0]);
           if (c + 1 < nch) v.y = to_float(in[bins]);
           if (c + 2 < nch) v.z = to_float(in[2 * bins]);
           if (c + 3 < nch) v.w = to_float(in[3 * bins]);
+          __builtin_nontemporal_store(f32x4s{v.x, v.y, v.z, v.w}, reinterpret_cast<f32x4s*>(dst + static_cast<size_t>(p) * 4));
         }
-        __builtin_nontemporal_store(f32x4s{v.x, v.y, v.z, v.w}, reinterpret_cast<f32x4s*>(dst + static_cast<size_t>(p) * 4));
       }
     } else {
       // the channel quads pc / 4 .. of the one block: 16-byte pieces, the quads of a cell side by side;
       // the last pass also writes the zero quads of channels that do not exist
-      float* const dst = dyb + (static_cast<size_t>(cb0) * R + r) * PH * PWp * CB;
+      float* const dst = dyb + (static_cast<size_t>(cb0) * R + r) * bins * CB;
       const int q0 = pc / 4, nq = pc + pass_ch >= nch ? CB / 4 - q0 : pn / 4;
-      for (int q = threadIdx.x; q < nq * PH * PWp; q += 256) {
-        const int cell = q / nq, qi = q - cell * nq, pw = cell % PWp, ph = cell / PWp;
+      for (int q = threadIdx.x; q < nq * bins; q += 256) {
+        const int cell = q / nq, qi = q - cell * nq, c = 4 * qi;   // bin, channel quad and first channel within the pass
+        const T* in = tbuf + c * bins + cell;
         float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if (pw < PW) {
-          const int c = 4 * qi;   // within the pass
-          const T* in = tbuf + c * bins + ph * PW + pw;
-          if (c + 0 < pn) v.x = to_float(in[0]);
-          if (c + 1 < pn) v.y = to_float(in[bins]);
-          if (c + 2 < pn) v.z = to_float(in[2 * bins]);
-          if (c + 3 < pn) v.w = to_float(in[3 * bins]);
-        }
+        if (c + 0 < pn) v.x = to_float(in[0]);
+        if (c + 1 < pn) v.y = to_float(in[bins]);
+        if (c + 2 < pn) v.z = to_float(in[2 * bins]);
+        if (c + 3 < pn) v.w = to_float(in[3 * bins]);
         __builtin_nontemporal_store(f32x4s{v.x, v.y, v.z, v.w},
                                     reinterpret_cast<f32x4s*>(dst + (static_cast<size_t>(cell) * 8 + q0 + qi) * 4));
       }
@@ -148,8 +143,8 @@ __device__ __forceinline__ void transpose_dy_blocked_body(unsigned block, const 
 template <typename T>
 __global__ void __launch_bounds__(256)
 transpose_dy_blocked_kernel(const T* __restrict__ dy, float* __restrict__ dyb, int C, int PH,
-                            int PW, int PWp, int cblk, int per, int R, int cap) {
-  transpose_dy_blocked_body<T>(blockIdx.x, dy, dyb, C, PH, PW, PWp, cblk, per, R, cap);
+                            int PW, int cblk, int per, int R, int cap) {
+  transpose_dy_blocked_body<T>(blockIdx.x, dy, dyb, C, PH, PW, cblk, per, R, cap);
 }
 
 // Both in one launch, for inputs too small to be worth a second stream: the
@@ -160,13 +155,13 @@ transpose_dy_blocked_kernel(const T* __restrict__ dy, float* __restrict__ dyb, i
 template <typename T>
 __global__ void __launch_bounds__(256)
 lists_and_dy_kernel(ListsArgs lists, unsigned list_blocks, const T* __restrict__ dy, float* __restrict__ dyb,
-                    int PWp, int cblk, int per, int C) {
+                    int cblk, int per, int C) {
   if (blockIdx.x < list_blocks) {
     if (lists.window_offsets != nullptr) build_window_lists_body(blockIdx.x, lists);
     else build_lists_body(blockIdx.x, lists);
   }
   else
-    transpose_dy_blocked_body<T>(blockIdx.x - list_blocks, dy, dyb, C, lists.PH, lists.PW, PWp, cblk, per, lists.R, 0);
+    transpose_dy_blocked_body<T>(blockIdx.x - list_blocks, dy, dyb, C, lists.PH, lists.PW, cblk, per, lists.R, 0);
 }
 
 // Number of workgroups for `tiles` tiles and cblk channel blocks (job decode at

@@ -411,7 +411,7 @@ bool plan_tiles(const Problem& p, const float* rois, int th, int tw, bool with_d
   const DyLaunch dl = dy_launch<T>(p);
   if (fuse_dy != nullptr && with_dyb && dl.per > 0 && dl.blocks > 0 && dl.blocks + list_blocks < (1ll << 31)) {
     roialign::lists_and_dy_kernel<T><<<static_cast<unsigned>(dl.blocks + list_blocks), 256, dl.lds, stream>>>(
-        la, static_cast<unsigned>(list_blocks), fuse_dy, plan->dyb, p.PW, cblk, dl.per, p.C);
+        la, static_cast<unsigned>(list_blocks), fuse_dy, plan->dyb, cblk, dl.per, p.C);
     plan->dy_transposed = true;
   } else {
     roialign::build_lists_kernel<<<static_cast<unsigned>(list_blocks), 256, 0, stream>>>(la);
@@ -525,10 +525,9 @@ void backward_device(const Problem& p, const T* dy, const float* rois, T* dx, bo
     const long long grid = roialign::backward_blocked_grid(plan.grid.total, cblk);
     const DyLaunch dl = dy_launch<T>(p);
     if (grid < (1ll << 31) && dl.blocks < (1ll << 31) && (dl.per > 0 || dl.cap >= 4)) {
-      const int pwp = p.PW;   // (the blocked copy's pooled rows are not padded)
       if (p.R > 0 && !plan.dy_transposed)
         roialign::transpose_dy_blocked_kernel<T><<<static_cast<unsigned>(dl.blocks), 256, dl.lds, side.get()>>>(
-            dy, plan.dyb, p.C, p.PH, p.PW, pwp, cblk, dl.per, p.R, dl.cap);
+            dy, plan.dyb, p.C, p.PH, p.PW, cblk, dl.per, p.R, dl.cap);
       side.join();
       {
         mobula_hip::KernelTimer timer("backward_blocked_kernel", stream);
