@@ -38,15 +38,19 @@ struct BlockOf {
   static constexpr int CPL = 16 / sizeof(T);
   static constexpr int CB = 8 * CPL;
   static constexpr int STAGE = 8704 / sizeof(T);
+  // the same for the gather of larger sampling grids (one wavefront per workgroup: with 6400 bytes
+  // the registers, not LDS, bound the wavefronts of a CU)
+  static constexpr int STAGE_MERGED = 6400 / sizeof(T);
 };
 
 // Pooled rows staged per pass, 0 if the shape is not taken by this path.
 template <typename T>
-inline int blocked_rows_per_pass(int C, long long H, long long W, int PH, int PW) {
+inline int blocked_rows_per_pass(int C, long long H, long long W, int PH, int PW, bool merged) {
   using B = BlockOf<T>;
-  if (C % B::CPL != 0 || PW < 1 || B::CB * PW > B::STAGE) return 0;
+  const int stage = merged ? B::STAGE_MERGED : B::STAGE;
+  if (C % B::CPL != 0 || PW < 1 || B::CB * PW > stage) return 0;
   if (H * W * 128 >= (1ll << 31)) return 0;
-  return min(PH, B::STAGE / (B::CB * PW));
+  return min(PH, stage / (B::CB * PW));
 }
 
 struct OrderArgs { const float* rois; int* order; int R; float scale; int H, W; long long num_images; };

@@ -81,7 +81,7 @@ forward_merged_kernel(const T* __restrict__ xt, const float* __restrict__ rois,
                       int rows_per_pass, int R) {
   using K = FwdBlocked;
   using M = FwdMerged;
-  constexpr int CPL = BlockOf<T>::CPL, CB = BlockOf<T>::CB, STAGE = BlockOf<T>::STAGE;
+  constexpr int CPL = BlockOf<T>::CPL, CB = BlockOf<T>::CB, STAGE = BlockOf<T>::STAGE_MERGED;
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   __shared__ MergedEntry rowm_s[M::NW][M::RPH][M::LCAP];
   __shared__ MergedEntry colm_s[M::NW][K::PWB][M::LCAP];

@@ -163,7 +163,7 @@ bool use_tiled();
 // straightforward fallback: the caller converts to NCHW instead).
 template <typename T>
 bool nhwc_forward_supported(const Problem& p) {
-  return roialign::blocked_rows_per_pass<T>(p.C, p.H, p.W, p.PH, p.PW) > 0 &&
+  return roialign::blocked_rows_per_pass<T>(p.C, p.H, p.W, p.PH, p.PW, p.S != 1 && p.S != 2) > 0 &&
          static_cast<long long>(p.H) * p.W * p.C * static_cast<long long>(sizeof(T)) < (1ll << 31);
 }
 
@@ -174,8 +174,8 @@ void forward_device(const Problem& p, const T* x, const float* rois, T* y, hipSt
   constexpr int CB = roialign::BlockOf<T>::CB;
   const long long pixels = static_cast<long long>(p.H) * p.W;
   const int cblk = (p.C + CB - 1) / CB;
-  const int rpp = roialign::blocked_rows_per_pass<T>(p.C, p.H, p.W, p.PH, p.PW);
   const bool small_grid = p.S == 1 || p.S == 2;   // else: sampling grids above 2 x 2, merged lists
+  const int rpp = roialign::blocked_rows_per_pass<T>(p.C, p.H, p.W, p.PH, p.PW, !small_grid);
   const int nw = small_grid ? FB::NW : roialign::FwdMerged::NW;   // wavefronts per workgroup of the gather
   const long long grid = roialign::blocked_grid(p.R, cblk, nw);
   const bool fits = rpp > 0 && p.N > 0 && p.N < 65536 && cblk < 65536 && grid < (1ll << 31);
