@@ -76,7 +76,7 @@ struct ListLayout {
   int row_stride;        // 16-byte units per (item, ty) row-tap table
   int col_stride;        // 16-byte units per (item, tx) column list
   long long roi_stride;  // units per item: ty*row_stride + tx*col_stride
-  int pw_padded;         // PW rounded up to 8: pooled columns of a column list (and of a row of dyb)
+  int pw_padded;         // PW rounded up to 8: pooled columns of a column list
   int windows;           // 1: merged weights (WindowRowTable, ColWindow), 0: sample lists (RowTapTable, ColPair)
 };
 
