@@ -212,11 +212,34 @@ build_taps_kernel(Tap* __restrict__ taps, int count, int KH, int KW, int plane, 
   taps[k] = Tap{ch * plane, static_cast<short>(kh * dil_h), static_cast<short>(kw * dil_w)};
 }
 
+// xp[plane][pad_h + ih][pad_w + iw] = x[plane][ih][iw], zeros around: planes of (H + 2 pad_h) x
+// (W + 2 pad_w), in which every tap of every output pixel is an element (no range tests).
+__global__ void __launch_bounds__(256)
+pad_planes_kernel(const float* __restrict__ x, float* __restrict__ xp, int H, int W, int pad_h, int pad_w,
+                  int Hp, int Wp) {
+  const float* in = x + static_cast<size_t>(blockIdx.x) * H * W;
+  float* out = xp + static_cast<size_t>(blockIdx.x) * Hp * Wp;
+  const int step_h = 256 / Wp, step_w = 256 - step_h * Wp;   // 256 elements further on
+  int i = blockIdx.y * 2048 + threadIdx.x, ph = i / Wp, pw = i - ph * Wp;
+  const int end = min((blockIdx.y + 1) * 2048, Hp * Wp);
+  for (; i < end; i += 256) {
+    const int ih = ph - pad_h, iw = pw - pad_w;
+    const bool inside = static_cast<unsigned>(ih) < static_cast<unsigned>(H) &&
+                        static_cast<unsigned>(iw) < static_cast<unsigned>(W);
+    out[i] = inside ? __builtin_nontemporal_load(in + ih * W + iw) : 0.0f;
+    ph += step_h; pw += step_w;
+    if (pw >= Wp) { pw -= Wp; ++ph; }
+  }
+}
+
 // partial[z][d, (c, kh, kw)] = sum over the k of slice z of dy[img, d, oh, ow] *
 // x[img, c, ih, iw], k = (img, oh, ow) flattened; a slice is a range of k.
 struct BackwardWeightOps {
   const float* __restrict__ dy; const float* __restrict__ x; float* __restrict__ partial;
-  const Tap* __restrict__ taps;   // taps over x
+  const Tap* __restrict__ taps;   // taps over x (over the planes of xp if that is set)
+  // zero-padded copy of x (pad_planes_kernel) of Hp x Wp per plane, or null: the taps of eight
+  // neighbouring output pixels are then two 16-byte loads, no range tests
+  const float* __restrict__ xp; int Hp, Wp;
   Geometry g; int M, Ncols, K;   // K = length of this slice
   int k_begin;                   // first k of this slice
   // image, pixel (flat and as row / column) of the step's first k; k left in the slice
@@ -262,6 +285,29 @@ struct BackwardWeightOps {
     int img = e.img, r = e.r + bk, oh0 = e.oh, ow0 = e.ow + bk;   // scalar: the step and bk are uniform
     while (ow0 >= g.OW) { ow0 -= g.OW; ++oh0; }
     while (r >= ohw) { r -= ohw; oh0 -= g.OH; ++img; }
+    if (xp != nullptr) {
+      const int image_p = g.C * Hp * Wp;
+      if (g.stride_w == 1 && ow0 + 8 <= g.OW && bk + 8 <= e.left) {
+        // eight pixels of one output row: eight neighbouring elements of the padded plane
+        typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+        const __amdgpu_buffer_rsrc_t src = buffer_of(xp + static_cast<size_t>(img) * image_p, image_p * 4u);
+        const int at = c.ok ? (c.off + (oh0 * g.stride_h + c.dh) * Wp + ow0 + c.dw) * 4 : kDead;
+        const u32x4 lo = __builtin_amdgcn_raw_buffer_load_b128(src, at, 0, 0);
+        const u32x4 hi = __builtin_amdgcn_raw_buffer_load_b128(src, at, 16, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { out[j] = __uint_as_float(lo[j]); out[4 + j] = __uint_as_float(hi[j]); }
+        return;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int oh = r / g.OW, ow = r - oh * g.OW;
+        const bool in = c.ok && bk + j < e.left;
+        out[j] = in ? xp[static_cast<size_t>(img) * image_p + c.off + (oh * g.stride_h + c.dh) * Wp +
+                         ow * g.stride_w + c.dw] : 0.0f;
+        if (++r == ohw) { r = 0; ++img; }
+      }
+      return;
+    }
     if (g.stride_w == 1 && ow0 + 8 <= g.OW && bk + 8 <= e.left) {
       // eight pixels of one output row: one row check, loads from one address
       const __amdgpu_buffer_rsrc_t src = buffer_of(x + static_cast<size_t>(img) * image, image * 4u);

@@ -524,13 +524,27 @@ MOBULA_KERNEL conv2d_backward_weight_kernel(const int n, const T* dy, const T* x
   long long slices = std::min<long long>(k_steps, std::max<long long>(1, kWeightSlots / per_slice_tiles));
   const long long k_per_slice = (k_steps + slices - 1) / slices * conv::Tile::BK;
   slices = std::max<long long>(1, (k_total + k_per_slice - 1) / k_per_slice);
+  // a zero-padded copy of x saves the gathered operand its range tests where eight output pixels
+  // of a row are eight neighbouring inputs (unit stride along a row); 32-bit offsets within an image
+  const int Hp = g.H + 2 * g.pad_h, Wp = g.W + 2 * g.pad_w;
+  const long long plane_p = static_cast<long long>(Hp) * Wp;
+  const bool padded = g.stride_w == 1 && g.N > 0 && plane_p * g.C * 4 < (1ll << 31) && plane_p < (1ll << 22);
+  const size_t partial_bytes = (sizeof(float) * static_cast<size_t>(slices) * wt + 255) / 256 * 256;
+  const size_t padded_bytes = padded ? sizeof(float) * static_cast<size_t>(g.N) * g.C * plane_p : 0;
   char* extra = nullptr;
-  ops.taps = make_taps(ops.Ncols, g.KH, g.KW, g.H * g.W, g.dil_h, g.dil_w,
-                       sizeof(float) * static_cast<size_t>(slices) * wt, &extra, stream);
+  ops.taps = make_taps(ops.Ncols, g.KH, g.KW, padded ? static_cast<int>(plane_p) : g.H * g.W, g.dil_h, g.dil_w,
+                       partial_bytes + padded_bytes, &extra, stream);
   if (failed()) return;
   ops.partial = reinterpret_cast<float*>(extra);
+  ops.xp = nullptr; ops.Hp = Hp; ops.Wp = Wp;
   {
     mobula_hip::KernelTimer timer("conv2d_backward_weight", stream);
+    if (padded) {
+      float* const xp = reinterpret_cast<float*>(extra + partial_bytes);
+      conv::pad_planes_kernel<<<dim3(g.N * g.C, static_cast<unsigned>((plane_p + 2047) / 2048)), 256, 0, stream>>>(
+          x, xp, g.H, g.W, g.pad_h, g.pad_w, Hp, Wp);
+      ops.xp = xp;
+    }
     const int tps = static_cast<int>(per_slice_tiles), count = tps * static_cast<int>(slices);
     const dim3 grid(conv::tile_blocks(count));
     switch (compute_mode()) {
